@@ -1,0 +1,133 @@
+"""Device side of the cache: the page tensors of every layer, the block tables, the state slots.
+
+Layout of one layer's pages (chosen for the attention kernels' matrix-core operands):
+
+* keys   ``K[page, kv_head, slot_in_page, head_dim]``: a key is one contiguous row;
+* values ``V[page, kv_head, head_dim, slot_in_page]``: stored transposed, so the positions
+  of a page are contiguous for one channel, which is how the ``P @ V`` product reads them.
+
+One page of one group therefore costs ``2 * kv_heads * head_dim * page_size`` elements in
+each layer of the group.  (The reference keeps token-granular rows ``[tokens, 2 * kv_heads,
+head_dim]``, rapid_llm/executor/kv_cache_manager.py:230-249.)
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from ..parts.base import CacheNeed
+from .manager import CacheManager, GroupSpec
+
+
+@dataclass
+class LayerCache:
+    """What one mixer sees of the cache."""
+
+    layer: int
+    group_id: int | None  # None: the mixer has no paged cache
+    page_size: int
+    k: torch.Tensor | None  # [pages, kv_heads, page_size, head_dim]
+    v: torch.Tensor | None  # [pages, kv_heads, head_dim, page_size]
+    owns_pages: bool  # False: reads another layer's pages and must not write them
+    state: torch.Tensor | None  # [max_seqs, *state_shape], zeroed when a slot is taken
+
+
+def plan_groups(needs: list[CacheNeed]) -> tuple[list[GroupSpec], list[int | None]]:
+    """Group layers by what they keep (all keys / a window of w).  Returns the groups and,
+    per layer, its group id (``None`` for layers without paged cache).  A layer that shares
+    another layer's cache joins that layer's group."""
+    keys: dict[int, int] = {}  # window -> group id
+    layers_of: dict[int, list[int]] = {}
+    group_of: list[int | None] = [None] * len(needs)
+    for i, need in enumerate(needs):
+        if need.kind != "kv" or need.share_with is not None:
+            continue
+        gid = keys.setdefault(need.window, len(keys))
+        layers_of.setdefault(gid, []).append(i)
+        group_of[i] = gid
+    for i, need in enumerate(needs):
+        if need.kind == "kv" and need.share_with is not None:
+            src = need.share_with
+            if not 0 <= src < len(needs) or needs[src].kind != "kv" or needs[src].share_with is not None:
+                raise ValueError(f"layer {i} shares the cache of layer {src}, which owns none")
+            if needs[src].window != need.window:
+                raise ValueError(
+                    f"layer {i} (window {need.window}) shares the cache of layer {src} "
+                    f"(window {needs[src].window}): a shared cache must keep the same positions"
+                )
+            group_of[i] = group_of[src]
+            layers_of[group_of[i]].append(i)
+    windows = {gid: w for w, gid in keys.items()}
+    groups = [GroupSpec(gid, windows[gid], tuple(layers_of[gid])) for gid in sorted(windows)]
+    return groups, group_of
+
+
+def page_bytes(needs: list[CacheNeed], group_of: list[int | None], page_size: int, elem: int) -> dict[int, int]:
+    """Bytes one page id costs in each group (summed over the group's owning layers)."""
+    out: dict[int, int] = {}
+    for need, gid in zip(needs, group_of):
+        if gid is None or need.share_with is not None:
+            continue
+        out[gid] = out.get(gid, 0) + 2 * need.num_kv_heads * need.head_dim * page_size * elem
+    return out
+
+
+class DeviceCache:
+    def __init__(
+        self,
+        manager: CacheManager,
+        needs: list[CacheNeed],
+        group_of: list[int | None],
+        dtype: torch.dtype,
+        device: torch.device,
+    ) -> None:
+        self.manager = manager
+        self.device = device
+        self.dtype = dtype
+        P = manager.page_size
+        self.layers: list[LayerCache] = []
+        for i, need in enumerate(needs):
+            k = v = None
+            gid = group_of[i]
+            owns = False
+            if need.kind == "kv" and need.share_with is None:
+                pages = manager.pools[gid].num_pages
+                # zero-filled once: page 0 is never written, and nothing is ever read from a
+                # page beyond what the masks allow
+                k = torch.zeros((pages, need.num_kv_heads, P, need.head_dim), dtype=dtype, device=device)
+                v = torch.zeros((pages, need.num_kv_heads, need.head_dim, P), dtype=dtype, device=device)
+                owns = True
+            state = None
+            if need.state_shape is not None:
+                sdt = getattr(torch, need.state_dtype) if need.state_dtype else dtype
+                state = torch.zeros((manager.max_seqs, *need.state_shape), dtype=sdt, device=device)
+            self.layers.append(LayerCache(i, gid, P, k, v, owns, state))
+        for i, need in enumerate(needs):
+            if need.kind == "kv" and need.share_with is not None:
+                src = self.layers[need.share_with]
+                self.layers[i].k, self.layers[i].v = src.k, src.v
+        self.tables: dict[int, torch.Tensor] = {
+            gid: torch.zeros(tab.shape, dtype=torch.int32, device=device)
+            for gid, tab in manager.tables.items()
+        }
+
+    def refresh(self) -> None:
+        """Bring the device block tables and state slots up to date with the manager: rows
+        of slots whose pages changed are copied, state of newly taken slots is cleared."""
+        m = self.manager
+        if m.dirty_slots:
+            slots = sorted(m.dirty_slots)
+            index = torch.tensor(slots, dtype=torch.int64, device=self.device)
+            for gid, host in m.tables.items():
+                rows = torch.from_numpy(np.ascontiguousarray(host[slots])).to(self.device)
+                self.tables[gid].index_copy_(0, index, rows)
+            m.dirty_slots.clear()
+        if m.fresh_slots:
+            slots = sorted(m.fresh_slots)
+            for layer in self.layers:
+                if layer.state is not None:
+                    layer.state[slots] = 0
+            m.fresh_slots.clear()

@@ -1,0 +1,31 @@
+from .engine_config import EngineConfig
+from .model_config import (
+    ConfigError,
+    Qwen3Config,
+    normalise_dtype_name,
+    read_architecture,
+    read_config_json,
+)
+from .registry import (
+    ArchitectureEntry,
+    config_from_dict,
+    register_architecture,
+    resolve_architecture,
+    supported_architectures,
+    unregister_architecture,
+)
+
+__all__ = [
+    "ArchitectureEntry",
+    "ConfigError",
+    "EngineConfig",
+    "Qwen3Config",
+    "config_from_dict",
+    "normalise_dtype_name",
+    "read_architecture",
+    "read_config_json",
+    "register_architecture",
+    "resolve_architecture",
+    "supported_architectures",
+    "unregister_architecture",
+]

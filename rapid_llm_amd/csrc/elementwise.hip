@@ -1,0 +1,315 @@
+// Row-wise kernels of the decoder: embedding gather, residual-add + RMSNorm, SwiGLU,
+// rotation tables, the fused per-head norm + rotation + cache write, and a type cast.
+// All arithmetic is float32; the element type only decides loads and stores.
+#include "common.h"
+
+// --------------------------------------------------------------------------- //
+// embedding: residual[t, :] = table[ids[t], :]   (float32 residual stream)
+// rapid_llm/modules/vocab_parallel.py:102-103
+// --------------------------------------------------------------------------- //
+template <typename W>
+__global__ void embed_kernel(const int* __restrict__ ids, const W* __restrict__ table,
+                             float* __restrict__ out, int hidden, int vocab) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    // ids are validated on the host; an id outside the table reads row 0 rather than faulting
+    if (id < 0 || id >= vocab) id = 0;
+    const W* row = table + (size_t)id * hidden;
+    float* dst = out + (size_t)t * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]);
+}
+
+extern "C" int rl_embed(const int* ids, const void* table, int table_type, float* out,
+                        int tokens, int hidden, int vocab, hipStream_t stream) {
+    if (tokens <= 0) return RL_OK;
+    dim3 grid(tokens), block(256);
+    if (table_type == RL_F32)
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids,
+                           (const float*)table, out, hidden, vocab);
+    else if (table_type == RL_BF16)
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids,
+                           (const bf16_t*)table, out, hidden, vocab);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// residual += delta (float32, in place); out = residual * rsqrt(mean(residual^2)+eps) * w
+// One block per produced row; `rows` (optional) selects which residual rows are produced,
+// packed in order.  rapid_llm/kernels/ops/layernorm/skip_rmsnorm.py:51-85: the sum is
+// formed in float32 and the norm reads the unrounded sum.
+// --------------------------------------------------------------------------- //
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                   const float* __restrict__ weight, T* __restrict__ out,
+                                   const int* __restrict__ rows, int hidden, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int row = rows ? rows[r] : r;
+    float* res = residual + (size_t)row * hidden;
+    const T* dl = delta ? delta + (size_t)row * hidden : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = res[i];
+        if (dl) {
+            v += to_float(dl[i]);
+            res[i] = v;
+        }
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float rrms = rsqrtf(ss / (float)hidden + eps);
+    T* o = out + (size_t)r * hidden;
+    // each thread re-reads exactly the elements it wrote above
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+        o[i] = from_float<T>(res[i] * rrms * weight[i]);
+}
+
+extern "C" int rl_add_rmsnorm(float* residual, const void* delta, const float* weight, void* out,
+                              const int* rows, int out_rows, int hidden, float eps, int act_type,
+                              hipStream_t stream) {
+    if (out_rows <= 0) return RL_OK;
+    int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+    dim3 grid(out_rows), block(threads);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, stream, residual,
+                           (const float*)delta, weight, (float*)out, rows, hidden, eps);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, residual,
+                           (const bf16_t*)delta, weight, (bf16_t*)out, rows, hidden, eps);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// SwiGLU on the packed [gate | up] row: out[:, j] = silu(x[:, j]) * x[:, I + j]
+// rapid_llm/kernels/ops/activation/swiglu.py:91-121
+// --------------------------------------------------------------------------- //
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
+                              size_t total) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) {
+        const size_t t = idx / inter;
+        const int j = (int)(idx - t * inter);
+        const T* row = gate_up + t * 2 * (size_t)inter;
+        const float g = to_float(row[j]);
+        const float u = to_float(row[inter + j]);
+        const float s = g / (1.f + expf(-g));
+        out[idx] = from_float<T>(s * u);
+    }
+}
+
+extern "C" int rl_swiglu(const void* gate_up, void* out, int tokens, int inter, int act_type,
+                         hipStream_t stream) {
+    if (tokens <= 0) return RL_OK;
+    const size_t total = (size_t)tokens * inter;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    dim3 grid((unsigned)blocks), block(256);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (const float*)gate_up,
+                           (float*)out, inter, total);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gate_up,
+                           (bf16_t*)out, inter, total);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// cast between float32 and bfloat16 (either direction, or a copy)
+// --------------------------------------------------------------------------- //
+template <typename S, typename D>
+__global__ void cast_kernel(const S* __restrict__ src, D* __restrict__ dst, size_t total) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) dst[idx] = from_float<D>(to_float(src[idx]));
+}
+
+extern "C" int rl_cast(const void* src, int src_type, void* dst, int dst_type, size_t total,
+                       hipStream_t stream) {
+    if (total == 0) return RL_OK;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    dim3 grid((unsigned)blocks), block(256);
+    if (src_type == RL_F32 && dst_type == RL_BF16)
+        hipLaunchKernelGGL((cast_kernel<float, bf16_t>), grid, block, 0, stream,
+                           (const float*)src, (bf16_t*)dst, total);
+    else if (src_type == RL_BF16 && dst_type == RL_F32)
+        hipLaunchKernelGGL((cast_kernel<bf16_t, float>), grid, block, 0, stream,
+                           (const bf16_t*)src, (float*)dst, total);
+    else if (src_type == RL_F32 && dst_type == RL_F32)
+        hipLaunchKernelGGL((cast_kernel<float, float>), grid, block, 0, stream,
+                           (const float*)src, (float*)dst, total);
+    else if (src_type == RL_BF16 && dst_type == RL_BF16)
+        hipLaunchKernelGGL((cast_kernel<bf16_t, bf16_t>), grid, block, 0, stream,
+                           (const bf16_t*)src, (bf16_t*)dst, total);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// rotation tables: cos/sin[p, i] of the float32 product p * inv_freq[i]
+// rapid_llm/modules/rotary_embedding.py:194-202 (float32 outer product, then cos/sin)
+// --------------------------------------------------------------------------- //
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, float* __restrict__ cos_out,
+                                  float* __restrict__ sin_out, int half, size_t total) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) {
+        const size_t p = idx / half;
+        const int i = (int)(idx - p * half);
+        const float ang = (float)p * inv_freq[i];
+        // the angle is the float32 product; its cosine and sine are taken in double so
+        // that range reduction of large angles costs nothing in accuracy
+        cos_out[idx] = (float)cos((double)ang);
+        sin_out[idx] = (float)sin((double)ang);
+    }
+}
+
+extern "C" int rl_rope_table(const float* inv_freq, float* cos_out, float* sin_out,
+                             int positions, int half, hipStream_t stream) {
+    const size_t total = (size_t)positions * half;
+    if (total == 0) return RL_OK;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, inv_freq,
+                       cos_out, sin_out, half, total);
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// Fused per-head RMSNorm (optional) + half-split rotation (optional) of q and k, and the
+// write of k and v into the paged cache.  One wave per (token, head).
+//
+// qkv row layout: [q heads | k heads | v heads], heads adjacent (rapid_llm/modules/linear.py:
+// 236-251).  Norm over head_dim before the rotation (rapid_llm/models/base.py:134-140).
+// Rotation: o1 = x1*c - x2*s, o2 = x2*c + x1*s on the halves
+// (rapid_llm/kernels/ops/rope/rope_emb.py:47-82).
+//
+// Cache layout of one layer, page p, kv head h:
+//   keys   K[p][h][slot_in_page][d]      (row-major, d contiguous)
+//   values V[p][h][d][slot_in_page]      (transposed: the page's positions contiguous)
+// A token at position pos of a request lies in page table[slot_of_request][pos / P] at
+// slot_in_page = pos % P.
+// --------------------------------------------------------------------------- //
+template <typename T>
+__global__ void qknorm_rope_kvwrite_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, const int* __restrict__ positions,
+    const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
+    int page_size, int nq, int nkv, int d, int rotary_half, float eps, int write_cache) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int nwaves = blockDim.x / RL_WAVE;
+    const int half = d / 2;
+    const int pos = positions[t];
+    const int total_heads = nq + 2 * nkv;
+    const T* row = qkv + (size_t)t * total_heads * d;
+
+    size_t page = 0;
+    int off = 0;
+    if (write_cache) {
+        page = (size_t)block_table[(size_t)token_slot[t] * table_stride + pos / page_size];
+        off = pos % page_size;
+    }
+
+    for (int head = wave; head < total_heads; head += nwaves) {
+        const T* x = row + (size_t)head * d;
+        if (head >= nq + nkv) {
+            // value head: copy into the transposed page
+            if (!write_cache) continue;
+            const int h = head - nq - nkv;
+            T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
+            for (int i = lane; i < d; i += RL_WAVE) dst[(size_t)i * page_size] = x[i];
+            continue;
+        }
+        const bool is_q = head < nq;
+        if (!is_q && !write_cache) continue;
+        const float* w = is_q ? q_norm_w : k_norm_w;
+        // lane handles element pairs (i, i + half) for i = lane, lane + 64 (half <= 128)
+        float x1[2], x2[2];
+        float ss = 0.f;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int i = lane + r * RL_WAVE;
+            x1[r] = 0.f;
+            x2[r] = 0.f;
+            if (i < half) {
+                x1[r] = to_float(x[i]);
+                x2[r] = to_float(x[i + half]);
+                ss += x1[r] * x1[r] + x2[r] * x2[r];
+            }
+        }
+        float rrms = 1.f;
+        if (w) {
+            ss = wave_sum(ss);
+            rrms = rsqrtf(ss / (float)d + eps);
+        }
+        T* dst;
+        if (is_q)
+            dst = q_out + ((size_t)t * nq + head) * d;
+        else
+            dst = k_cache + ((page * nkv + (head - nq)) * page_size + off) * d;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int i = lane + r * RL_WAVE;
+            if (i < half) {
+                float a = x1[r], b = x2[r];
+                if (w) {
+                    a = a * rrms * w[i];
+                    b = b * rrms * w[i + half];
+                }
+                if (cos_tab && i < rotary_half) {
+                    const float c = cos_tab[(size_t)pos * rotary_half + i];
+                    const float s = sin_tab[(size_t)pos * rotary_half + i];
+                    const float ra = a * c - b * s;
+                    const float rb = b * c + a * s;
+                    a = ra;
+                    b = rb;
+                }
+                dst[i] = from_float<T>(a);
+                dst[i + half] = from_float<T>(b);
+            }
+        }
+    }
+}
+
+extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cache, void* v_cache,
+                                      const float* q_norm_w, const float* k_norm_w,
+                                      const float* cos_tab, const float* sin_tab,
+                                      const int* positions, const int* token_slot,
+                                      const int* block_table, int table_stride, int page_size,
+                                      int tokens, int nq, int nkv, int d, int rotary_half,
+                                      float eps, int write_cache, int act_type,
+                                      hipStream_t stream) {
+    if (tokens <= 0) return RL_OK;
+    if (d % 2 || d > 256) return RL_ERR_ARG;
+    // only a rotation over the whole head is implemented (pairs i, i + d/2)
+    if (cos_tab && rotary_half != d / 2) return RL_ERR_ARG;
+    dim3 grid(tokens), block(256);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<float>, grid, block, 0, stream,
+                           (const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
+                           q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
+                           block_table, table_stride, page_size, nq, nkv, d, rotary_half, eps,
+                           write_cache);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<bf16_t>, grid, block, 0, stream,
+                           (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
+                           (bf16_t*)v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions,
+                           token_slot, block_table, table_stride, page_size, nq, nkv, d,
+                           rotary_half, eps, write_cache);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}

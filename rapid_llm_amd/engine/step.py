@@ -1,0 +1,295 @@
+"""The one step function: a batch of (request, its next tokens) in, logits at the wanted places out.
+
+A step is one forward pass over a flat, unpadded batch: portions of prompts of some
+requests beside single decoded tokens of others, cut anywhere.  It runs only the tokens it
+is given, reads everything earlier from the cache, writes this step's keys and values into
+their pages, and returns float32 logits for the requested rows only.
+
+The reference runs up to three forwards per scheduler step (a padded prefill grid, a
+chunked/extend pass, a decode pass; rapid_llm/engine/scheduler.py:964-988) described by
+``ModelInput`` spans (rapid_llm/executor/worker.py:69-126).  Here the span description is
+kept (a request's tokens cover its cache positions ``[start, start + n)``) and the three
+passes are one.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Any, Mapping, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheError, CacheManager
+from ..cache.storage import DeviceCache, page_bytes, plan_groups
+from ..config.engine_config import EngineConfig
+from ..config.model_config import read_config_json
+from ..config.registry import config_from_dict
+from ..kernels import ops
+from ..models.causal_lm import CausalLM
+from ..parts.runtime import Runtime
+from ..weights.loader import load_model_dir
+from ..weights.random_init import random_params
+
+_TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+class OutOfPages(CacheError):
+    """A step needs more pages (or slots) than are free; nothing was taken."""
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens and the places among them whose
+    logits are wanted (indices into ``tokens``; may be empty)."""
+
+    request_id: str
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class StepContext:
+    """Everything the parts may read about the batch of one step.  Device tensors are int32."""
+
+    runtime: Runtime
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor  # [T]
+    positions: torch.Tensor  # [T] absolute position of each token in its request
+    token_slot: torch.Tensor  # [T] slot (block-table row, state row) of each token's request
+    seq_slots: torch.Tensor  # [n]
+    seq_starts: torch.Tensor  # [n] tokens of the request already in the cache
+    seq_lens: torch.Tensor  # [n] tokens of the request in this step
+    cu_seqlens: torch.Tensor  # [n + 1] offsets of the requests' tokens in the flat batch
+    logit_rows: torch.Tensor  # [R] flat token indices whose logits are wanted
+    num_logit_rows: int
+    block_tables: dict[int, torch.Tensor]  # group id -> [slots, pages per sequence]
+    # host copies, for launch decisions (never read by kernels)
+    h_seq_slots: list[int] = field(default_factory=list)
+    h_seq_starts: list[int] = field(default_factory=list)
+    h_seq_lens: list[int] = field(default_factory=list)
+    max_position: int = 0
+    max_seq_tokens: int = 0  # longest portion in the batch
+    extra: dict[str, Any] = field(default_factory=dict)  # per-step device metadata of kernels
+
+
+class ModelRunner:
+    """Owns the model, its weights and the cache, and runs steps."""
+
+    def __init__(
+        self,
+        model: str | Path | Mapping[str, Any],
+        engine: EngineConfig | None = None,
+        *,
+        load_format: str = "auto",
+        overrides: Mapping[str, Any] | None = None,
+        device: str | torch.device = "cuda",
+        weight_norm_std: float = 0.0,
+    ) -> None:
+        ops.require_gpu()
+        self.engine = engine or EngineConfig()
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise ops.KernelError(f"the engine runs on a HIP device only, not on {self.device}")
+        self.dtype = _TORCH_DTYPE[self.engine.dtype]
+
+        if isinstance(model, Mapping):
+            body, model_dir = dict(model), None
+            if load_format == "auto":
+                load_format = "random"
+        else:
+            model_dir = Path(model)
+            body = read_config_json(model_dir)
+        self.arch, self.config = config_from_dict(body, overrides)
+        self.spec = self.arch.build_spec(self.config)
+        if self.spec.max_position and self.engine.max_seq_len > self.spec.max_position:
+            # rapid_llm/models/config.py:374-378
+            raise ValueError(
+                f"max_seq_len {self.engine.max_seq_len} exceeds the model's "
+                f"max_position_embeddings {self.spec.max_position}"
+            )
+        self.runtime = Runtime(self.device, self.dtype, self.engine.max_seq_len, self.engine.page_size)
+        self.model = CausalLM(self.spec)
+
+        specs = self.model.param_specs()
+        if load_format == "random":
+            params = random_params(
+                specs, self.engine.seed, engine_dtype=self.dtype, device=self.device,
+                norm_std=weight_norm_std,
+            )
+        elif load_format == "auto":
+            params = load_model_dir(
+                model_dir, specs, engine_dtype=self.dtype, device=self.device,
+                ignore_rules=self.spec.ignore_tensors,
+            )
+        else:
+            raise ValueError(f"load_format must be 'auto' or 'random', got {load_format!r}")
+        self.params = params
+        self.model.bind(params, self.runtime)
+
+        # ---- cache -------------------------------------------------------------
+        needs = self.model.cache_needs()
+        groups, group_of = plan_groups(needs)
+        elem = 4 if self.dtype == torch.float32 else 2
+        self.page_bytes = page_bytes(needs, group_of, self.engine.page_size, elem)
+        num_pages = self._decide_num_pages(groups)
+        self.cache = CacheManager(
+            groups, num_pages, self.engine.page_size, self.engine.max_num_seqs, self.engine.max_seq_len
+        )
+        self.device_cache = DeviceCache(self.cache, needs, group_of, self.dtype, self.device)
+        self.computed: dict[str, int] = {}
+        self.vocab_size = self.spec.vocab_size
+
+    # ------------------------------------------------------------------ sizing
+    def _decide_num_pages(self, groups) -> int:
+        e = self.engine
+        if e.num_pages is not None:
+            return e.num_pages
+        if e.max_gpu_num_blocks is not None:  # the reference's knob counts tokens (README.md:121)
+            return -(-e.max_gpu_num_blocks // e.page_size) + 1
+        # what is left of the device after the weights, times the utilisation, shared by
+        # the groups (rapid_llm/executor/kv_cache_manager.py:91-130)
+        free, total = torch.cuda.mem_get_info(self.device)
+        budget = free - int(total * (1.0 - e.gpu_memory_utilization)) - (2 << 30)
+        per_page = sum(self.page_bytes.values()) or 1
+        pages = max(2, budget // per_page)
+        # never more than every slot at full length can use
+        cap = e.max_num_seqs * (-(-e.max_seq_len // e.page_size)) + 1
+        return int(min(pages, cap))
+
+    # ------------------------------------------------------------------ requests
+    def tokens_cached(self, request_id: str) -> int:
+        return self.computed.get(request_id, 0)
+
+    def can_run(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether ``step(entries)`` would find the slots and pages it needs."""
+        new = [e for e in entries if not self.cache.has(e.request_id)]
+        if len(new) > self.cache.num_free_slots:
+            return False
+        need: dict[int, int] = {}
+        ps = self.cache.page_size
+        for e in entries:
+            start = self.computed.get(e.request_id, 0)
+            if self.cache.has(e.request_id):
+                per = self.cache.pages_needed(e.request_id, start + len(e.tokens), start)
+            else:
+                per = {}
+                for g in self.cache.groups:
+                    per[g.group_id] = -(-(start + len(e.tokens)) // ps)
+            for gid, n in per.items():
+                need[gid] = need.get(gid, 0) + n
+        return all(n <= self.cache.num_free_pages(gid) for gid, n in need.items())
+
+    def finish(self, request_id: str) -> None:
+        """The request is over: its pages and its slot are given back."""
+        if self.cache.has(request_id):
+            self.cache.release(request_id)
+        self.computed.pop(request_id, None)
+
+    # ------------------------------------------------------------------ the step
+    def _prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        cache = self.cache
+        seen = set()
+        for e in entries:
+            if e.request_id in seen:
+                raise ValueError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            n = len(e.tokens)
+            if n < 1:
+                raise ValueError(f"request {e.request_id!r} brings no tokens")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"request {e.request_id!r} wants place {w} of {n} tokens")
+            start = self.computed.get(e.request_id, 0)
+            if start + n > self.engine.max_seq_len:
+                raise ValueError(
+                    f"request {e.request_id!r} would reach {start + n} tokens; max_seq_len is "
+                    f"{self.engine.max_seq_len}"
+                )
+        # slots and pages: all requests of the step or none
+        if not self.can_run(entries):
+            raise OutOfPages(
+                "the step does not fit: "
+                f"{cache.num_free_slots} free slots, {cache.num_free_pages()} free pages"
+            )
+        for e in entries:
+            if not cache.has(e.request_id):
+                cache.admit(e.request_id)
+            start = self.computed.get(e.request_id, 0)
+            if not cache.reserve(e.request_id, start + len(e.tokens), start):
+                raise CacheError("pages counted as free could not be taken")
+
+        vocab = self.vocab_size
+        n_seq = len(entries)
+        lens = [len(e.tokens) for e in entries]
+        total = sum(lens)
+        starts = [self.computed.get(e.request_id, 0) for e in entries]
+        slots = [cache.slot_of(e.request_id) for e in entries]
+        n_rows = sum(len(e.want) for e in entries)
+        # one packed int32 upload: ids | positions | token_slot | slots | starts | lens | cu | rows
+        sizes = [total, total, total, n_seq, n_seq, n_seq, n_seq + 1, n_rows]
+        offs = np.concatenate(([0], np.cumsum(sizes)))
+        host = np.empty(int(offs[-1]), dtype=np.int32)
+        cu = 0
+        row = 0
+        for i, e in enumerate(entries):
+            n = lens[i]
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if toks.min() < 0 or toks.max() >= vocab:
+                raise ValueError(
+                    f"request {e.request_id!r} has a token id outside [0, {vocab}): "
+                    f"min {toks.min()}, max {toks.max()}"
+                )
+            host[offs[0] + cu : offs[0] + cu + n] = toks
+            host[offs[1] + cu : offs[1] + cu + n] = np.arange(starts[i], starts[i] + n)
+            host[offs[2] + cu : offs[2] + cu + n] = slots[i]
+            for w in e.want:
+                host[offs[7] + row] = cu + w
+                row += 1
+            host[offs[6] + i] = cu
+            cu += n
+        host[offs[6] + n_seq] = cu
+        host[offs[3] : offs[4]] = slots
+        host[offs[4] : offs[5]] = starts
+        host[offs[5] : offs[6]] = lens
+        dev = torch.from_numpy(host).to(self.device, non_blocking=False)
+        part = [dev[offs[i] : offs[i + 1]] for i in range(len(sizes))]
+
+        self.device_cache.refresh()
+        return StepContext(
+            runtime=self.runtime,
+            num_tokens=total,
+            num_seqs=n_seq,
+            token_ids=part[0],
+            positions=part[1],
+            token_slot=part[2],
+            seq_slots=part[3],
+            seq_starts=part[4],
+            seq_lens=part[5],
+            cu_seqlens=part[6],
+            logit_rows=part[7],
+            num_logit_rows=n_rows,
+            block_tables=self.device_cache.tables,
+            h_seq_slots=slots,
+            h_seq_starts=starts,
+            h_seq_lens=lens,
+            max_position=max(s + n for s, n in zip(starts, lens)) - 1,
+            max_seq_tokens=max(lens),
+        )
+
+    @torch.no_grad()
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run one batch; returns float32 logits ``[wanted, vocab]`` in the order of the
+        entries and of each entry's ``want``.  Raises :class:`OutOfPages`, with nothing
+        changed, when slots or pages do not suffice."""
+        if not entries:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        ctx = self._prepare(entries)
+        logits = self.model.forward(ctx, self.device_cache.layers)
+        for e in entries:
+            done = self.computed.get(e.request_id, 0) + len(e.tokens)
+            self.computed[e.request_id] = done
+            self.cache.trim(e.request_id, done)  # pages a window has passed come back now
+        return logits

@@ -1,0 +1,312 @@
+"""Call wrappers around the HIP kernels: host-side checks, then one launch on the current stream.
+
+Nothing here computes: every function validates its operands (device, type, contiguity,
+shape) and hands raw pointers to the compiled library.  There is no fallback; without a
+GPU or without the compiled library these raise.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_TAG = {torch.float32: F32, torch.bfloat16: BF16}
+
+_core: ctypes.CDLL | None = None
+_attn: dict[int, ctypes.CDLL] = {}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def require_gpu() -> None:
+    if not torch.cuda.is_available():
+        raise KernelError(
+            "rapid_llm_amd runs its model on a HIP device only (no CPU implementation exists) "
+            "and no GPU is visible to this process"
+        )
+
+
+def core() -> ctypes.CDLL:
+    global _core
+    if _core is None:
+        _core = build.load(build.core_library())
+    return _core
+
+
+def attention_lib(head_dim: int) -> ctypes.CDLL:
+    lib = _attn.get(head_dim)
+    if lib is None:
+        lib = build.load(build.attention_library(head_dim))
+        _attn[head_dim] = lib
+    return lib
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _tag(dtype: torch.dtype) -> int:
+    try:
+        return _TAG[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 tensors, got {dtype}") from None
+
+
+def _need(t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape=None) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{name} must live on the GPU, is on {t.device}")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous (shape {tuple(t.shape)}, strides {t.stride()})")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, is {t.dtype}")
+    if shape is not None:
+        if len(shape) != t.dim() or any(s is not None and s != a for s, a in zip(shape, t.shape)):
+            raise KernelError(f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+
+
+def _ok(code: int, what: str) -> None:
+    if code != 0:
+        reason = {1: "an argument the kernel refuses", 2: "the launch failed"}.get(code, "unknown")
+        raise KernelError(f"{what}: error {code} ({reason})")
+
+
+# --------------------------------------------------------------------------- #
+
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+    tokens = ids.numel()
+    vocab, hidden = table.shape
+    _need(ids, "ids", torch.int32)
+    _need(table, "embedding table")
+    _need(out, "out", torch.float32, (tokens, hidden))
+    _ok(
+        core().rl_embed(_p(ids), _p(table), _tag(table.dtype), _p(out), tokens, hidden, vocab, _stream()),
+        "rl_embed",
+    )
+
+
+def add_rmsnorm(
+    residual: torch.Tensor,
+    delta: Optional[torch.Tensor],
+    weight: torch.Tensor,
+    out: torch.Tensor,
+    eps: float,
+    rows: Optional[torch.Tensor] = None,
+) -> None:
+    tokens, hidden = residual.shape
+    _need(residual, "residual", torch.float32)
+    _need(weight, "norm weight", torch.float32, (hidden,))
+    out_rows = tokens if rows is None else rows.numel()
+    _need(out, "out", None, (out_rows, hidden))
+    if delta is not None:
+        _need(delta, "delta", out.dtype, (tokens, hidden))
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+    _ok(
+        core().rl_add_rmsnorm(
+            _p(residual), _p(delta), _p(weight), _p(out), _p(rows), out_rows, hidden,
+            ctypes.c_float(eps), _tag(out.dtype), _stream(),
+        ),
+        "rl_add_rmsnorm",
+    )
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    tokens, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError(f"the packed [gate | up] row must have even width, has {two_i}")
+    _need(gate_up, "gate_up")
+    _need(out, "out", gate_up.dtype, (tokens, two_i // 2))
+    _ok(
+        core().rl_swiglu(_p(gate_up), _p(out), tokens, two_i // 2, _tag(out.dtype), _stream()),
+        "rl_swiglu",
+    )
+
+
+def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
+    _need(src, "src")
+    _need(dst, "dst")
+    if src.numel() != dst.numel():
+        raise KernelError(f"cast of {src.numel()} elements into {dst.numel()}")
+    _ok(
+        core().rl_cast(
+            _p(src), _tag(src.dtype), _p(dst), _tag(dst.dtype), ctypes.c_size_t(src.numel()), _stream()
+        ),
+        "rl_cast",
+    )
+
+
+def rope_table(inv_freq: torch.Tensor, positions: int) -> tuple[torch.Tensor, torch.Tensor]:
+    _need(inv_freq, "inv_freq", torch.float32)
+    half = inv_freq.numel()
+    cos = torch.empty((positions, half), dtype=torch.float32, device=inv_freq.device)
+    sin = torch.empty_like(cos)
+    _ok(core().rl_rope_table(_p(inv_freq), _p(cos), _p(sin), positions, half, _stream()), "rl_rope_table")
+    return cos, sin
+
+
+def qknorm_rope_kvwrite(
+    qkv: torch.Tensor,
+    q_out: torch.Tensor,
+    k_cache: Optional[torch.Tensor],
+    v_cache: Optional[torch.Tensor],
+    q_norm_w: Optional[torch.Tensor],
+    k_norm_w: Optional[torch.Tensor],
+    cos: Optional[torch.Tensor],
+    sin: Optional[torch.Tensor],
+    positions: torch.Tensor,
+    token_slot: torch.Tensor,
+    block_table: torch.Tensor,
+    page_size: int,
+    nq: int,
+    nkv: int,
+    d: int,
+    eps: float,
+    max_position: int,
+) -> None:
+    """Norm + rotate q and k, write k and v to the cache pages (skipped when the caches
+    are ``None``: a layer that reads another layer's cache).  ``max_position`` is the
+    largest position in the batch, checked against the rotation table and block table."""
+    tokens = qkv.shape[0]
+    _need(qkv, "qkv", None, (tokens, (nq + 2 * nkv) * d))
+    _need(q_out, "q_out", qkv.dtype, (tokens, nq * d))
+    _need(positions, "positions", torch.int32, (tokens,))
+    _need(token_slot, "token_slot", torch.int32, (tokens,))
+    _need(block_table, "block_table", torch.int32)
+    write = k_cache is not None
+    if write:
+        pages = k_cache.shape[0]
+        _need(k_cache, "k_cache", qkv.dtype, (pages, nkv, page_size, d))
+        _need(v_cache, "v_cache", qkv.dtype, (pages, nkv, d, page_size))
+        if max_position // page_size >= block_table.shape[1]:
+            raise KernelError(
+                f"position {max_position} needs page {max_position // page_size} of a block "
+                f"table with {block_table.shape[1]} columns"
+            )
+    for w, name in ((q_norm_w, "q_norm weight"), (k_norm_w, "k_norm weight")):
+        if w is not None:
+            _need(w, name, torch.float32, (d,))
+    half = 0
+    if cos is not None:
+        half = cos.shape[1]
+        _need(cos, "cos table", torch.float32, (None, half))
+        _need(sin, "sin table", torch.float32, tuple(cos.shape))
+        if max_position >= cos.shape[0]:
+            raise KernelError(
+                f"position {max_position} is beyond the rotation table of {cos.shape[0]} positions"
+            )
+    _ok(
+        core().rl_qknorm_rope_kvwrite(
+            _p(qkv), _p(q_out), _p(k_cache), _p(v_cache), _p(q_norm_w), _p(k_norm_w), _p(cos),
+            _p(sin), _p(positions), _p(token_slot), _p(block_table), block_table.stride(0),
+            page_size, tokens, nq, nkv, d, half, ctypes.c_float(eps), int(write), _tag(qkv.dtype),
+            _stream(),
+        ),
+        "rl_qknorm_rope_kvwrite",
+    )
+
+
+def attention_generic(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    out: torch.Tensor,
+    positions: torch.Tensor,
+    token_slot: torch.Tensor,
+    block_table: torch.Tensor,
+    page_size: int,
+    nq: int,
+    nkv: int,
+    d: int,
+    window: int,
+    scale: float,
+    max_position: int,
+) -> None:
+    tokens = q.shape[0]
+    pages = k_cache.shape[0]
+    _need(q, "q", None, (tokens, nq * d))
+    _need(out, "out", q.dtype, (tokens, nq * d))
+    _need(k_cache, "k_cache", q.dtype, (pages, nkv, page_size, d))
+    _need(v_cache, "v_cache", q.dtype, (pages, nkv, d, page_size))
+    _need(positions, "positions", torch.int32, (tokens,))
+    _need(token_slot, "token_slot", torch.int32, (tokens,))
+    _need(block_table, "block_table", torch.int32)
+    if max_position // page_size >= block_table.shape[1]:
+        raise KernelError(
+            f"position {max_position} needs page {max_position // page_size} of a block table "
+            f"with {block_table.shape[1]} columns"
+        )
+    _ok(
+        core().rl_attention_generic(
+            _p(q), _p(k_cache), _p(v_cache), _p(out), _p(positions), _p(token_slot),
+            _p(block_table), block_table.stride(0), page_size, tokens, nq, nkv, d, window,
+            ctypes.c_float(scale), _tag(q.dtype), _stream(),
+        ),
+        "rl_attention_generic",
+    )
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[M,N] = a[M,K] @ w[N,K]^T`` in true float32.  Rows may be strided (views of wider
+    matrices); the inner dimension must be contiguous."""
+    for t, name in ((a, "a"), (w, "w"), (out, "out")):
+        if not t.is_cuda or t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1:
+            raise KernelError(f"gemm_f32 operand {name} must be a float32 GPU matrix with unit inner stride")
+    m, k = a.shape
+    n, k2 = w.shape
+    if k != k2 or out.shape != (m, n):
+        raise KernelError(f"gemm_f32 shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    _ok(
+        core().rl_gemm_f32(_p(a), _p(w), _p(out), m, n, k, a.stride(0), w.stride(0), out.stride(0), _stream()),
+        "rl_gemm_f32",
+    )
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    rows, vocab = logits.shape
+    _need(logits, "logits", torch.float32)
+    _need(out, "out", torch.int32, (rows,))
+    _ok(core().rl_argmax(_p(logits), _p(out), rows, vocab, _stream()), "rl_argmax")
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """``x[M,K] @ w[N,K]^T`` with bfloat16 operands and float32 accumulation.  Returns
+    bfloat16, or float32 when ``out_dtype`` is float32 and the kernel used can write it."""
+    _need(x, "x", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    if x.shape[1] != w.shape[1]:
+        raise KernelError(f"gemm_bf16 shapes do not agree: x {tuple(x.shape)}, w {tuple(w.shape)}")
+    # the library product, as the reference's dense products are (F.linear)
+    return torch.matmul(x, w.t())
+
+
+def paged_attention(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    out: torch.Tensor,
+    ctx,
+    block_table: torch.Tensor,
+    page_size: int,
+    nq: int,
+    nkv: int,
+    d: int,
+    window: int,
+    scale: float,
+) -> None:
+    """Attention of every token of the step over its request's cached keys."""
+    attention_generic(
+        q, k_cache, v_cache, out, ctx.positions, ctx.token_slot, block_table, page_size,
+        nq, nkv, d, window, scale, ctx.max_position,
+    )

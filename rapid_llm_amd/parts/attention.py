@@ -1,0 +1,122 @@
+"""Grouped-query attention over the paged cache.
+
+Per step: fused QKV projection (rapid_llm/models/base.py:121-132), per-head RMSNorm of q
+and k over head_dim before the rotation (:134-137), rotation (:139-140), write of this
+step's keys and values into their pages (rapid_llm/modules/attention.py:126-138), attention
+of every query over its request's cached keys up to its own position (:157-240), output
+projection (base.py:164-165).  The norm, the rotation and the cache write are one kernel.
+
+Keys and values are always read back from the pages, also for the tokens of the current
+step, so that one code path serves whole prompts, portions and single decoded tokens
+(the reference switches kernels by phase, attention.py:179-240).  ``window`` > 0 limits a
+query at position p to keys ``[p - window + 1, p]`` (rapid_llm/engine/kv_cache_spec.py:203-222).
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..kernels import ops
+from .base import MIXERS, CacheNeed, Mixer, ParamSpec, Source
+from .linear import Linear
+
+
+class GQAAttention(Mixer):
+    def __init__(
+        self,
+        hidden_size: int,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        checkpoint_prefix: str,
+        qk_norm_eps: float | None = None,
+        window: int = 0,
+        position=None,
+        softmax_scale: float | None = None,
+        name: str = "mixer",
+        q_name: str = "q_proj.weight",
+        k_name: str = "k_proj.weight",
+        v_name: str = "v_proj.weight",
+        o_name: str = "o_proj.weight",
+        q_norm_name: str = "q_norm.weight",
+        k_norm_name: str = "k_norm.weight",
+    ) -> None:
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not divisible by {num_kv_heads} kv heads")
+        if head_dim % 16 or not 16 <= head_dim <= 256:
+            raise ValueError(f"attention kernels take head sizes in steps of 16 up to 256, got {head_dim}")
+        self.hidden_size = hidden_size
+        self.nq, self.nkv, self.d = num_heads, num_kv_heads, head_dim
+        self.prefix = checkpoint_prefix
+        self.qk_norm_eps = qk_norm_eps
+        self.window = int(window)
+        self.position = position
+        self.scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(head_dim)
+        self.name = name
+        self.names = dict(q=q_name, k=k_name, v=v_name, o=o_name, qn=q_norm_name, kn=k_norm_name)
+        self.qkv = Linear(hidden_size, (num_heads + 2 * num_kv_heads) * head_dim)
+        self.o = Linear(num_heads * head_dim, hidden_size)
+        self.q_norm_w = self.k_norm_w = None
+
+    # ---- tensors ---------------------------------------------------------------
+    def param_specs(self) -> list[ParamSpec]:
+        p, n = self.prefix, self.names
+        q_rows, kv_rows = self.nq * self.d, self.nkv * self.d
+        specs = [
+            ParamSpec(
+                self.name + ".qkv",
+                (q_rows + 2 * kv_rows, self.hidden_size),
+                "matrix",
+                (Source(p + n["q"], q_rows), Source(p + n["k"], kv_rows), Source(p + n["v"], kv_rows)),
+            ),
+            ParamSpec(self.name + ".o", (self.hidden_size, q_rows), "matrix", (Source(p + n["o"], self.hidden_size),)),
+        ]
+        if self.qk_norm_eps is not None:
+            specs += [
+                ParamSpec(self.name + ".q_norm", (self.d,), "vector", (Source(p + n["qn"], self.d),), init="norm"),
+                ParamSpec(self.name + ".k_norm", (self.d,), "vector", (Source(p + n["kn"], self.d),), init="norm"),
+            ]
+        return specs
+
+    def bind(self, params, runtime) -> None:
+        self.qkv.bind(params[self.name + ".qkv"])
+        self.o.bind(params[self.name + ".o"])
+        if self.qk_norm_eps is not None:
+            self.q_norm_w = params[self.name + ".q_norm"]
+            self.k_norm_w = params[self.name + ".k_norm"]
+        self.runtime = runtime
+
+    # ---- cache -----------------------------------------------------------------
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed("kv", window=self.window, num_kv_heads=self.nkv, head_dim=self.d)
+
+    # ---- step ------------------------------------------------------------------
+    def forward(self, x, ctx, cache):
+        tokens = x.shape[0]
+        qkv = self.qkv(x)
+        q = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
+        table = ctx.block_tables[cache.group_id]
+        pos_enc = self.position
+        ops.qknorm_rope_kvwrite(
+            qkv, q,
+            cache.k if cache.owns_pages else None,
+            cache.v if cache.owns_pages else None,
+            self.q_norm_w, self.k_norm_w,
+            pos_enc.cos if pos_enc is not None else None,
+            pos_enc.sin if pos_enc is not None else None,
+            ctx.positions, ctx.token_slot, table, cache.page_size,
+            self.nq, self.nkv, self.d,
+            self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
+            ctx.max_position,
+        )
+        out = torch.empty_like(q)
+        ops.paged_attention(
+            q, cache.k, cache.v, out, ctx, table, cache.page_size,
+            self.nq, self.nkv, self.d, self.window, self.scale,
+        )
+        return self.o(out)
+
+
+MIXERS.register("gqa_attention", GQAAttention)

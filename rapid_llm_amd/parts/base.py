@@ -1,0 +1,185 @@
+"""Interfaces of the parts a model is put together from, and their registries.
+
+A part takes its sizes and constants as constructor parameters and never learns which
+model it sits in.  Five kinds exist:
+
+* ``Mixer``: mixes information across the positions of a sequence (attention here).
+  It may need cache: pages of keys and values (all of them or a window), and/or a
+  fixed-size state per request.
+* ``FeedForward``: per-token transformation (dense SwiGLU here; routed experts later).
+* ``Norm``: normalisation, fused with the residual add in front of it.
+* ``PositionEncoding``: what a mixer consults to encode positions (rotation tables here).
+* ``Block``: the arrangement of mixer, feed-forward and norms around the residual stream.
+
+Every part declares its tensors as :class:`ParamSpec` (``param_specs``), receives them
+loaded (``bind``), and runs on a flat batch of tokens described by a
+:class:`~rapid_llm_amd.engine.step.StepContext` (``forward``).  The reference reaches the
+same seams by constructor injection (rapid_llm/models/base.py:188-216: ``mlp=`` and
+``attention=`` arguments of ``DecoderLayer``).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import TYPE_CHECKING, Any, Callable
+
+if TYPE_CHECKING:  # pragma: no cover
+    import torch
+
+    from ..engine.step import StepContext
+
+
+# --------------------------------------------------------------------------- #
+# tensors a part needs
+# --------------------------------------------------------------------------- #
+
+
+@dataclass(frozen=True)
+class Source:
+    """One checkpoint tensor feeding ``rows`` rows (dim 0) of a parameter."""
+
+    name: str
+    rows: int
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One tensor of the model as the engine holds it.
+
+    ``sources`` are concatenated along dim 0 in order: a fused matrix such as the packed
+    query/key/value projection lists its three checkpoint tensors
+    (rapid_llm/modules/linear.py:253-271 writes the same row blocks).
+
+    ``role`` decides the storage type:
+      * ``"matrix"``: the engine's compute type; in a bfloat16 engine a tensor the
+        checkpoint stores in 32-bit stays 32-bit.
+      * ``"vector"``: small per-channel weights (norms); always held in float32, which
+        represents a bfloat16 checkpoint value exactly.
+      * ``"table"``: integer lookup tables, held as int32.
+    ``fallback`` names another parameter whose tensor is shared when the checkpoint has
+    none of this one's sources (a tied output projection).
+    ``init`` is the distribution the random-weights mode draws the sources from.
+    """
+
+    name: str
+    shape: tuple[int, ...]
+    role: str
+    sources: tuple[Source, ...]
+    init: str = "normal"  # "normal" | "norm" | "zeros" | "table"
+    fallback: str | None = None
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """What a mixer asks of the cache manager.
+
+    ``kind == "kv"``: paged keys and values; ``window`` 0 keeps every position, otherwise
+    only the last ``window`` positions of a request are kept and older pages are given back.
+    ``kind == "state"``: nothing paged.  ``state_shape`` (may accompany either kind) is a
+    fixed-size per-request tensor the mixer owns, zeroed when a request takes the slot.
+    ``share_with`` names the place in the run order whose cache this one reads instead of
+    writing its own.
+    """
+
+    kind: str  # "kv" | "state" | "none"
+    window: int = 0
+    num_kv_heads: int = 0
+    head_dim: int = 0
+    state_shape: tuple[int, ...] | None = None
+    state_dtype: str | None = None  # torch dtype name; None: the engine's compute type
+    share_with: int | None = None
+
+
+class Part:
+    """Common protocol: declare tensors, receive them, run."""
+
+    def param_specs(self) -> list[ParamSpec]:
+        return []
+
+    def bind(self, params: dict[str, "torch.Tensor"], runtime: Any) -> None:
+        """Receive the loaded tensors (keyed by ``ParamSpec.name``) and the runtime
+        (device, compute type, kernel library, largest sequence length)."""
+
+
+class PositionEncoding(Part):
+    """Supplies what a mixer needs to encode a token's absolute position."""
+
+    kind = "none"
+
+
+class Mixer(Part):
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed("none")
+
+    def forward(self, x: "torch.Tensor", ctx: "StepContext", cache: Any) -> "torch.Tensor":
+        """``x [T, hidden]`` (normalised) -> the mixer's contribution ``[T, hidden]``.
+        ``cache`` is the :class:`~rapid_llm_amd.cache.storage.LayerCache` of this place in
+        the run order: a layer that runs twice has a cache for each run."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: "torch.Tensor", ctx: "StepContext") -> "torch.Tensor":
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(
+        self,
+        residual: "torch.Tensor",
+        delta: "torch.Tensor | None",
+        ctx: "StepContext",
+        rows: "torch.Tensor | None" = None,
+    ) -> "torch.Tensor":
+        """``residual += delta`` (in place, float32) and return ``norm(residual)`` in the
+        compute type.  With ``rows`` (int32 indices) only those rows are produced, packed."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    def forward(self, residual: "torch.Tensor", delta, ctx: "StepContext", cache: Any):
+        """Advance the residual stream through one layer; returns the pending ``delta``
+        (the last sub-layer's output, to be added by whoever normalises next)."""
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------- #
+# registries: kind name -> constructor
+# --------------------------------------------------------------------------- #
+
+
+@dataclass
+class PartRegistry:
+    what: str
+    _table: dict[str, Callable[..., Any]] = field(default_factory=dict)
+
+    def register(self, kind: str, ctor: Callable[..., Any] | None = None, *, replace=False):
+        def _do(c):
+            if kind in self._table and not replace:
+                raise ValueError(f"{self.what} kind {kind!r} is already registered")
+            self._table[kind] = c
+            return c
+
+        return _do if ctor is None else _do(ctor)
+
+    def unregister(self, kind: str) -> None:
+        self._table.pop(kind, None)
+
+    def create(self, kind: str, /, **params: Any) -> Any:
+        try:
+            ctor = self._table[kind]
+        except KeyError:
+            raise ValueError(
+                f"unknown {self.what} kind {kind!r}; known: {', '.join(sorted(self._table))}"
+            ) from None
+        return ctor(**params)
+
+    def kinds(self) -> list[str]:
+        return sorted(self._table)
+
+
+MIXERS = PartRegistry("mixer")
+FEED_FORWARDS = PartRegistry("feed-forward")
+NORMS = PartRegistry("norm")
+POSITION_ENCODINGS = PartRegistry("position encoding")
+BLOCKS = PartRegistry("block")

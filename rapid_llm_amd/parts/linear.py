@@ -1,0 +1,50 @@
+"""``y = x W^T`` with ``W [out, in]`` as the checkpoint stores it (no bias in this family).
+
+Which product runs is decided by the weight's storage type:
+
+* float32 weight: the hand-written float32 FMA kernel (true 32-bit; the only product of
+  the float32 engine).  A bfloat16 activation is widened first, so a matrix that the
+  checkpoint stores in 32-bit is used at full precision in a bfloat16 engine too.
+* bfloat16 weight: few rows (decode) go to the hand-written bandwidth-bound matrix-core
+  kernel; many rows go to the library product, as in the reference, whose dense products
+  are ``F.linear`` (rapid_llm/kernels/ops/gemm/linear.py:17-40).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+
+
+class Linear:
+    def __init__(self, in_features: int, out_features: int) -> None:
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight: torch.Tensor | None = None
+
+    def bind(self, weight: torch.Tensor) -> None:
+        if tuple(weight.shape) != (self.out_features, self.in_features):
+            raise ValueError(
+                f"linear weight must be {(self.out_features, self.in_features)}, is {tuple(weight.shape)}"
+            )
+        self.weight = weight
+
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        w = self.weight
+        rows = x.shape[0]
+        out_dtype = out_dtype or x.dtype
+        if w.dtype == torch.float32:
+            if x.dtype != torch.float32:
+                wide = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+                ops.cast(x, wide)
+                x = wide
+            y = torch.empty((rows, self.out_features), dtype=torch.float32, device=x.device)
+            ops.gemm_f32(x, w, y)
+        else:
+            y = ops.gemm_bf16(x, w, out_dtype)
+        if y.dtype != out_dtype:
+            narrow = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+            ops.cast(y, narrow)
+            y = narrow
+        return y

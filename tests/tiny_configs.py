@@ -1,0 +1,54 @@
+"""Tiny configurations of the Qwen3 dense decoder that differ in every size and option."""
+
+import json
+import random
+from pathlib import Path
+
+# A: tied embeddings, group 2, head 16, power-of-two sizes, small page
+TINY_A = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
+    head_dim=16, intermediate_size=128, vocab_size=256, rope_theta=10000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=128,
+    hidden_act="silu", attention_bias=False,
+)
+PAGE_A = 4
+
+# B: untied, one kv head (group 6), head 32 with heads*head_dim != hidden, odd vocabulary
+TINY_B = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=3, hidden_size=96, num_attention_heads=6, num_key_value_heads=1,
+    head_dim=32, intermediate_size=320, vocab_size=503, rope_theta=1000000.0,
+    rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=256,
+    hidden_act="silu", attention_bias=False,
+)
+PAGE_B = 16
+
+# C: windowed layers beside a full one (two cache groups), head 48 (no power of two),
+# as many kv heads as query heads, width 80, vocabulary 331
+TINY_C = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=3, hidden_size=80, num_attention_heads=5, num_key_value_heads=5,
+    head_dim=48, intermediate_size=176, vocab_size=331, rope_theta=500000.0,
+    rms_norm_eps=3e-6, tie_word_embeddings=False, max_position_embeddings=512,
+    hidden_act="silu", attention_bias=False,
+    sliding_window=21, layer_types=["full_attention", "sliding_attention", "sliding_attention"],
+)
+PAGE_C = 8
+
+TINY = {"A": (TINY_A, PAGE_A, 11), "B": (TINY_B, PAGE_B, 22), "C": (TINY_C, PAGE_C, 33)}
+
+
+def make_model_dir(tmp_path: Path, which: str, dtype: str = "float32") -> Path:
+    """Write config.json + model.safetensors of a tiny model (norm weights 1 + N(0, 0.1))."""
+    from rapid_llm_amd.weights import write_random_model
+
+    cfg, _page, seed = TINY[which]
+    out = Path(tmp_path) / f"tiny_{which}_{dtype}"
+    write_random_model(dict(cfg), seed, out, dtype=dtype, norm_std=0.1)
+    return out
+
+
+def random_tokens(n: int, vocab: int, seed: int) -> list[int]:
+    rng = random.Random(seed)
+    return [rng.randrange(vocab) for _ in range(n)]
