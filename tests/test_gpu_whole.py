@@ -8,7 +8,7 @@ from tiny_configs import TINY, make_model_dir, random_tokens
 
 pytestmark = pytest.mark.gpu
 
-F32_TOL = dict(rtol=2e-4, atol=2e-5)
+F32_TOL = dict(rtol=2e-5, atol=3e-6)
 BF16_TOL = dict(rtol=5e-2, atol=3e-2)
 
 
