@@ -1,0 +1,246 @@
+"""Decode and prefill speed of the engine on one MI355X, random weights, synthetic token ids.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16]
+
+A "step" is one decode step of the whole batch through the engine's step function and the
+greedy sampling kernel, tokens fed back.  The default run has the layer sizes of
+Qwen3-8B (BASELINE.json ``configs[2]``), a batch of 8, every request with a 2,048-token
+prompt, context 4,096.  One JSON line is printed: decoded tokens a second (``value``), the
+2,048-token prefill (``prefill``), the decode step against the HBM roofline (``roofline``)
+and decoding at batch 1 and 64 (``points``).
+
+Metric definitions follow rapid_llm's docs/benchmark_models.md:141-149: decode tok/s is
+batch / mean step time; prefill tok/s is prompt tokens / prefill latency; both timed
+between device synchronisations after warm-up.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_GBPS = 8000.0
+PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
+
+
+def load_shape() -> dict:
+    """Layer sizes of BASELINE.json configs[2], parsed from its text."""
+    import re
+
+    with open(os.path.join(ROOT, "BASELINE.json")) as fh:
+        text = json.load(fh)["configs"][2]
+
+    def num(pattern: str) -> int:
+        m = re.search(pattern, text)
+        if m is None:
+            raise SystemExit(f"BASELINE.json configs[2] does not state {pattern!r}")
+        return int(m.group(1).replace(",", ""))
+
+    theta = re.search(r"rope_theta ([0-9.e+]+)", text).group(1)
+    eps = re.search(r"rms_norm_eps ([0-9.e+-]+)", text).group(1)
+    return dict(
+        architectures=["Qwen3ForCausalLM"],
+        model_type="qwen3",
+        num_hidden_layers=num(r"(\d+) layers"),
+        hidden_size=num(r"hidden (\d+)"),
+        num_attention_heads=num(r"(\d+) query heads"),
+        num_key_value_heads=num(r"(\d+) KV heads"),
+        head_dim=num(r"head_dim (\d+)"),
+        intermediate_size=num(r"intermediate (\d+)"),
+        vocab_size=num(r"vocab (\d+)"),
+        rope_theta=float(theta),
+        rms_norm_eps=float(eps),
+        tie_word_embeddings="untied" not in text,
+        max_position_embeddings=40960,
+        context=num(r"context (\d+)"),
+        prompt_len=num(r"one ([\d,]+)-token prompt"),
+    )
+
+
+def weight_bytes(cfg, elem: int) -> int:
+    h, i = cfg.hidden_size, cfg.intermediate_size
+    per_layer = (cfg.q_size + 2 * cfg.kv_size) * h + h * cfg.q_size + 2 * i * h + h * i
+    return (per_layer * cfg.num_hidden_layers + cfg.vocab_size * h) * elem
+
+
+def kv_bytes_per_token(cfg, elem: int) -> int:
+    return 2 * cfg.kv_size * cfg.num_hidden_layers * elem
+
+
+def prefill_flops(cfg, tokens: int) -> float:
+    h, i = cfg.hidden_size, cfg.intermediate_size
+    per_layer = (cfg.q_size + 2 * cfg.kv_size) * h + h * cfg.q_size + 2 * i * h + h * i
+    linear = 2.0 * tokens * per_layer * cfg.num_hidden_layers + 2.0 * cfg.vocab_size * h  # one logits row
+    attn = 2.0 * 2.0 * cfg.q_size * (tokens * (tokens + 1) / 2) * cfg.num_hidden_layers  # causal QK^T and PV
+    return linear + attn
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--points", default="1,64", help="other decode batch sizes to measure ('' for none)")
+    ap.add_argument("--point-steps", type=int, default=32)
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-graph", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
+        return 2
+
+    import torch
+
+    from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
+    from rapid_llm_amd.kernels import ops
+
+    shape = load_shape()
+    context, prompt_len = shape.pop("context"), shape.pop("prompt_len")
+    full_layers = shape["num_hidden_layers"]
+    if args.layers is not None:
+        shape["num_hidden_layers"] = args.layers
+    points = [int(p) for p in args.points.split(",") if p]
+    max_batch = max([args.batch] + points)
+    elem = 2 if args.dtype == "bfloat16" else 4
+
+    engine = EngineConfig(
+        dtype=args.dtype,
+        max_seq_len=context,
+        page_size=16,
+        num_pages=max_batch * (context // 16) + 1,
+        max_num_seqs=max_batch,
+        max_num_batched_tokens=max(8192, prompt_len),
+        use_graph=not args.no_graph,
+        seed=1234,
+    )
+    t0 = time.time()
+    runner = ModelRunner(shape, engine, load_format="random")
+    cfg = runner.config
+    torch.cuda.synchronize()
+    print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    gen = torch.Generator().manual_seed(7)
+    vocab = cfg.vocab_size
+
+    def prompt() -> list[int]:
+        return torch.randint(0, vocab, (prompt_len,), generator=gen).tolist()
+
+    # ---- prefill of one 2,048-token prompt ------------------------------------
+    prefill = None
+    if not args.no_prefill:
+        times = []
+        for i in range(4):
+            toks = prompt()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            runner.step([StepEntry("p", toks, [prompt_len - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            runner.finish("p")
+        sec = statistics.median(times[1:])
+        flops = prefill_flops(cfg, prompt_len)
+        prefill = {
+            "value": round(prompt_len / sec, 1),
+            "tokens": prompt_len,
+            "ms": round(sec * 1e3, 3),
+            "frac": round(flops / sec / (PEAK_TFLOPS[args.dtype] * 1e12), 4),
+        }
+        print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+
+    # ---- decode ----------------------------------------------------------------
+    def decode(batch: int, steps: int, warmup: int) -> tuple[float, float]:
+        """Mean seconds per decode step and the mean context length over the timed steps."""
+        ids = [f"d{i}" for i in range(batch)]
+        last = torch.empty(batch, dtype=torch.int32, device=runner.device)
+        for k, rid in enumerate(ids):  # prompts, one request a step
+            logits = runner.step([StepEntry(rid, prompt(), [prompt_len - 1])])
+            ops.argmax(logits, last[k : k + 1])
+        tokens = last.tolist()
+
+        def one_step():
+            nonlocal tokens
+            logits = runner.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
+            ops.argmax(logits, last)
+            tokens = last.tolist()  # the step's one host synchronisation
+
+        for _ in range(warmup):
+            one_step()
+        torch.cuda.synchronize()
+        ctx_start = runner.tokens_cached(ids[0])
+        t = time.perf_counter()
+        for _ in range(steps):
+            one_step()
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t) / steps
+        mean_ctx = ctx_start + (steps - 1) / 2.0 + 1
+        for rid in ids:
+            runner.finish(rid)
+        return sec, mean_ctx
+
+    sec, mean_ctx = decode(args.batch, args.steps, args.warmup)
+    step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
+    achieved = step_bytes / sec / 1e9
+    result = {
+        "metric": "Qwen3-8B bf16 decode tok/s (batch 8, 2048-token prompts); prefill tok/s at 2048 tokens",
+        "value": round(args.batch / sec, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (uniform random token ids, random N(0,0.02) weights, norm weights 1)",
+        "config": {
+            "model": "Qwen3-8B shape",
+            "layers": cfg.num_hidden_layers,
+            "layers_full": full_layers,
+            "hidden": cfg.hidden_size,
+            "q_heads": cfg.num_attention_heads,
+            "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim,
+            "intermediate": cfg.intermediate_size,
+            "vocab": cfg.vocab_size,
+            "rope_theta": cfg.rope_theta,
+            "rms_norm_eps": cfg.rms_norm_eps,
+            "tied": cfg.tie_word_embeddings,
+            "global_batch": args.batch,
+            "seq_len": prompt_len,
+            "context": context,
+            "page_size": engine.page_size,
+            "graph": engine.use_graph,
+            "parallelism": "single GPU",
+        },
+        "prefill": prefill,
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_GBPS, 4),
+        },
+    }
+    pts = {}
+    for b in points:
+        s, _ = decode(b, args.point_steps, max(2, args.warmup // 2))
+        pts[f"decode_b{b}"] = round(b / s, 2)
+        print(f"[bench] decode batch {b}: {pts[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
+    result["points"] = pts
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

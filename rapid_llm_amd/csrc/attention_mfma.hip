@@ -1,0 +1,561 @@
+// Matrix-core (MFMA) paged attention for bfloat16 on gfx950, compiled for one head size
+// RL_HEAD_DIM (a multiple of 16 up to 256).
+//
+// Both kernels compute the *transposed* products, so that nothing ever has to change
+// layout between the two matrix products:
+//
+//   S^T[keys, rows]  = K[keys, d]   * Q^T[d, rows]      (A = K,   B = Q^T)
+//   O^T[d, rows]    += V^T[d, keys] * P^T[keys, rows]   (A = V^T, B = P^T)
+//
+// with v_mfma_f32_16x16x32_bf16: a wave owns 16 "rows" (queries) as the N dimension.  The
+// result of the first product leaves lane (row r, group g = lane / 16) with the scores of
+// keys 4g..4g+3 of each 16-key block; two such blocks are exactly the B operand of the
+// second product once its contraction slots are labelled (g, j): j < 4 -> key 4g + j of
+// the first block, j >= 4 -> key 4g + j - 4 of the second.  The A operand then needs, for
+// channel d, the values of those same keys: two 8-byte reads of four consecutive positions,
+// which is why the cache stores values transposed (V[page][head][d][slot]).  Softmax state
+// (running maximum and sum) is one scalar per lane, since a lane only ever sees one row.
+//
+// Rows are (token, query head of the kv group) pairs, so grouped-query attention reads each
+// key once for all heads of its group.  Softmax runs in the exp2 domain in float32
+// (rapid_llm/kernels/ops/attention/flashattention2_nopad.py:138-168); P is rounded to
+// bfloat16 for the second product (:162), sums use the unrounded values.
+//
+//   rl_attn_prefill: portions of prompts.  Workgroup = 4 waves x 32 rows; K and V^T tiles of
+//                    64 keys are staged through LDS and shared by the waves.
+//   rl_attn_decode:  single tokens.  Workgroup = (request, kv head, split of the keys); its
+//                    4 waves stride over 32-key steps reading K and V^T straight from
+//                    global memory (nothing is reused), combine through LDS, and a merge
+//                    kernel folds the splits (rapid_llm/kernels/ops/attention/flashdecoding.py:
+//                    115-263 stage 1, :334-407 stage 2).
+#include "common.h"
+
+#ifndef RL_HEAD_DIM
+#error "compile with -DRL_HEAD_DIM=<head size>"
+#endif
+
+#define D RL_HEAD_DIM
+static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int DC = (D + 31) / 32;     // 32-channel chunks of the first product
+constexpr int DB = D / 16;            // 16-channel blocks of the output
+constexpr bool D_TAIL = (D % 32) != 0;  // the last chunk holds 16 channels, the rest is zero
+
+__device__ inline bf16x8 zero8() {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+    return z;
+}
+
+__device__ inline bf16x8 load16(const bf16_t* p) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+
+// two groups of four consecutive bfloat16 -> one operand
+__device__ inline bf16x8 load8x2(const bf16_t* p0, const bf16_t* p1) {
+    struct {
+        uint2 a, b;
+    } v;
+    v.a = *reinterpret_cast<const uint2*>(p0);
+    v.b = *reinterpret_cast<const uint2*>(p1);
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+__device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// maximum over the four lanes (groups) that hold the same row
+__device__ inline float row_max4(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16, RL_WAVE));
+    v = fmaxf(v, __shfl_xor(v, 32, RL_WAVE));
+    return v;
+}
+__device__ inline float row_sum4(float v) {
+    v += __shfl_xor(v, 16, RL_WAVE);
+    v += __shfl_xor(v, 32, RL_WAVE);
+    return v;
+}
+
+// --------------------------------------------------------------------------- //
+// One 32-key step of the online softmax for one block of 16 rows.
+//   s0, s1: raw scores (q . k) of the two 16-key blocks, this lane's keys 4g..4g+3
+//   ok0, ok1: bit i set when key i of the block is visible to this lane's row
+// Updates (m, l), scales the accumulators, returns P^T as the B operand.
+// --------------------------------------------------------------------------- //
+__device__ inline bf16x8 softmax_step(f32x4 s0, f32x4 s1, unsigned ok0, unsigned ok1,
+                                      float scale_log2, float& m, float& l, f32x4* acc) {
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[i] = ((ok0 >> i) & 1u) ? s0[i] * scale_log2 : -INFINITY;
+        x[4 + i] = ((ok1 >> i) & 1u) ? s1[i] * scale_log2 : -INFINITY;
+    }
+    float mx = x[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) mx = fmaxf(mx, x[i]);
+    mx = row_max4(mx);
+    const float m_new = fmaxf(m, mx);
+    // a row that has seen no visible key yet keeps m = -inf; exp2 of (-inf) - 0 is 0
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = exp2f(m - m_safe);
+    float psum = 0.f;
+    bf16x8 p;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float e = exp2f(x[i] - m_safe);
+        psum += e;
+        p[i] = (__bf16)e;
+    }
+    l = l * alpha + psum;  // per-lane partial sum; the four groups are added at the end
+    m = m_new;
+#pragma unroll
+    for (int b = 0; b < DB; ++b) {
+        acc[b][0] *= alpha;
+        acc[b][1] *= alpha;
+        acc[b][2] *= alpha;
+        acc[b][3] *= alpha;
+    }
+    return p;
+}
+
+// =========================================================================== //
+// decode
+// =========================================================================== //
+#define DEC_WAVES 4
+
+__global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, const int* __restrict__ seq_token,
+    const int* __restrict__ positions, const int* __restrict__ token_slot,
+    const int* __restrict__ block_table, int table_stride, int page_size, int nq, int nkv,
+    int window, float scale_log2, int split_chunk, int nsplit) {
+    __shared__ float lds_o[2][D * 16];
+    __shared__ float lds_m[2][16];
+    __shared__ float lds_l[2][16];
+
+    const int G = nq / nkv;
+    const int head_chunks = (G + 15) / 16;
+    const int seq = blockIdx.x;
+    const int hk = blockIdx.y / head_chunks;
+    const int hc = blockIdx.y % head_chunks;
+    const int split = blockIdx.z;
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int col = lane & 15;  // row of the attention problem = query head of the group
+    const int g = lane >> 4;
+
+    const int t = seq_token[seq];
+    const int pos = positions[t];
+    const int* table = block_table + (size_t)token_slot[t] * table_stride;
+    const int kend = pos + 1;
+    const int kstart = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int lo = (kstart & ~31) + split * split_chunk;  // split_chunk is a multiple of 32
+    const int hi = min(kend, lo + split_chunk);
+
+    const int hh = hc * 16 + col;  // head within the group
+    const bool head_ok = hh < G;
+    const int head = hk * G + (head_ok ? hh : 0);
+
+    if (lo >= hi) {
+        // nothing of this request falls into this split: tell the merge to skip it
+        if (nsplit > 1 && wave == 0 && g == 0 && head_ok) {
+            float* ml = part_ml + (((size_t)seq * nq + head) * nsplit + split) * 2;
+            ml[0] = -INFINITY;
+            ml[1] = 0.f;
+        }
+        return;
+    }
+
+    // Q^T as B operand: lane (row col, group g) holds channels 32c + 8g .. + 7
+    bf16x8 qf[DC];
+    {
+        const bf16_t* qrow = q + ((size_t)t * nq + head) * D;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
+            qf[c] = (head_ok && chan_ok) ? load16(qrow + 32 * c + 8 * g) : zero8();
+        }
+    }
+
+    float m = -INFINITY, l = 0.f;
+    f32x4 acc[DB];
+#pragma unroll
+    for (int b = 0; b < DB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    const int last_key = kend - 1;
+    for (int base = lo + 32 * wave; base < hi; base += 32 * DEC_WAVES) {
+        // ---- S^T = K Q^T for two blocks of 16 keys --------------------------------
+        f32x4 s[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int key = min(base + 16 * kb + col, last_key);  // clamped: masked below
+            const int page = table[key / page_size];
+            const bf16_t* krow =
+                k_cache + (((size_t)page * nkv + hk) * page_size + key % page_size) * D;
+            s[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < DC; ++c) {
+                const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
+                const bf16x8 a = chan_ok ? load16(krow + 32 * c + 8 * g) : zero8();
+                s[kb] = mfma(a, qf[c], s[kb]);
+            }
+        }
+        // ---- which of this lane's keys are visible ---------------------------------
+        unsigned ok[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            ok[kb] = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = base + 16 * kb + 4 * g + i;
+                ok[kb] |= (key >= kstart && key < kend) ? (1u << i) : 0u;
+            }
+        }
+        const bf16x8 p = softmax_step(s[0], s[1], ok[0], ok[1], scale_log2, m, l, acc);
+        // ---- O^T += V^T P^T ---------------------------------------------------------
+        const bool partial = (base + 32 > kend) || (base < kstart);
+        const bf16_t* vrow[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            // this lane's four keys of the block; clamped as a group so that the read stays
+            // inside one page of the request (what is read there is zeroed below)
+            const int key = min(base + 16 * kb + 4 * g, last_key & ~3);
+            const int page = table[key / page_size];
+            vrow[kb] = v_cache + (((size_t)page * nkv + hk) * D) * page_size + key % page_size;
+        }
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+            const size_t doff = (size_t)(16 * b + col) * page_size;
+            bf16x8 v = load8x2(vrow[0] + doff, vrow[1] + doff);
+            if (partial) {
+                // 0 * stale data must be 0: a page used before may hold anything
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (!((ok[0] >> i) & 1u)) v[i] = (__bf16)0.f;
+                    if (!((ok[1] >> i) & 1u)) v[4 + i] = (__bf16)0.f;
+                }
+            }
+            acc[b] = mfma(v, p, acc[b]);
+        }
+    }
+
+    // ---- combine the waves: (2,3) -> (0,1), then 1 -> 0, in the accumulators' own layout ----
+    l = row_sum4(l);
+    auto put = [&](int slot) {
+        if (g == 0) {
+            lds_m[slot][col] = m;
+            lds_l[slot][col] = l;
+        }
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lds_o[slot][(16 * b + 4 * g + i) * 16 + col] = acc[b][i];
+    };
+    auto take = [&](int slot) {
+        const float m_o = lds_m[slot][col], l_o = lds_l[slot][col];
+        const float mm = fmaxf(m, m_o);
+        const float ms = (mm == -INFINITY) ? 0.f : mm;  // a wave without keys has m = -inf
+        const float f1 = exp2f(m - ms), f2 = exp2f(m_o - ms);
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                acc[b][i] = acc[b][i] * f1 + lds_o[slot][(16 * b + 4 * g + i) * 16 + col] * f2;
+        l = l * f1 + l_o * f2;
+        m = mm;
+    };
+    if (wave >= 2) put(wave - 2);
+    __syncthreads();
+    if (wave < 2) take(wave);
+    __syncthreads();
+    if (wave == 1) put(0);
+    __syncthreads();
+    if (wave != 0) return;
+    take(0);
+    if (!head_ok) return;
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    if (nsplit == 1) {
+        bf16_t* orow = out + ((size_t)t * nq + head) * D;
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+            struct {
+                bf16_t v[4];
+            } o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o.v[i] = float_to_bf16(acc[b][i] * inv);
+            *reinterpret_cast<uint2*>(orow + 16 * b + 4 * g) = __builtin_bit_cast(uint2, o);
+        }
+    } else {
+        const size_t slot = ((size_t)seq * nq + head) * nsplit + split;
+        float* orow = part_o + slot * D;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+            *reinterpret_cast<float4*>(orow + 16 * b + 4 * g) =
+                make_float4(acc[b][0] * inv, acc[b][1] * inv, acc[b][2] * inv, acc[b][3] * inv);
+        if (g == 0) {
+            part_ml[slot * 2] = m;
+            part_ml[slot * 2 + 1] = l;
+        }
+    }
+}
+
+// merge of the splits: out = sum_s w_s o_s / sum_s w_s with w_s = l_s * 2^(m_s - max m)
+__global__ void attn_merge_kernel(const float* __restrict__ part_o,
+                                  const float* __restrict__ part_ml, bf16_t* __restrict__ out,
+                                  const int* __restrict__ seq_token, int nq, int nsplit) {
+    const int seq = blockIdx.x, head = blockIdx.y;
+    const size_t slot0 = ((size_t)seq * nq + head) * nsplit;
+    float mm = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(slot0 + s) * 2]);
+    float wsum = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float ms = part_ml[(slot0 + s) * 2];
+        if (ms != -INFINITY) wsum += part_ml[(slot0 + s) * 2 + 1] * exp2f(ms - mm);
+    }
+    const int t = seq_token[seq];
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float o = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float ms = part_ml[(slot0 + s) * 2];
+            if (ms == -INFINITY) continue;  // an empty split wrote no output
+            o += part_o[(slot0 + s) * D + d] * (part_ml[(slot0 + s) * 2 + 1] * exp2f(ms - mm));
+        }
+        out[((size_t)t * nq + head) * D + d] = float_to_bf16(o / wsum);
+    }
+}
+
+extern "C" int rl_attn_head_dim() { return D; }
+
+extern "C" int rl_attn_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
+                              float* part_o, float* part_ml, const int* seq_token,
+                              const int* positions, const int* token_slot,
+                              const int* block_table, int table_stride, int page_size,
+                              int num_seqs, int nq, int nkv, int window, float scale,
+                              int split_chunk, int nsplit, hipStream_t stream) {
+    if (num_seqs <= 0) return RL_OK;
+    if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || split_chunk < 32 ||
+        split_chunk % 32 || nsplit < 1 || nsplit > 65535)
+        return RL_ERR_ARG;
+    if (nsplit > 1 && (!part_o || !part_ml)) return RL_ERR_ARG;
+    const int G = nq / nkv;
+    const int head_chunks = (G + 15) / 16;
+    if ((long)nkv * head_chunks > 65535) return RL_ERR_ARG;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    dim3 grid(num_seqs, nkv * head_chunks, nsplit), block(DEC_WAVES * RL_WAVE);
+    hipLaunchKernelGGL(attn_decode_kernel, grid, block, 0, stream, (const bf16_t*)q,
+                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_o,
+                       part_ml, seq_token, positions, token_slot, block_table, table_stride,
+                       page_size, nq, nkv, window, scale_log2, split_chunk, nsplit);
+    if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
+    if (nsplit > 1) {
+        hipLaunchKernelGGL(attn_merge_kernel, dim3(num_seqs, nq), dim3(D < 64 ? 64 : D), 0,
+                           stream, part_o, part_ml, (bf16_t*)out, seq_token, nq, nsplit);
+    }
+    return rl_launch_status();
+}
+
+// =========================================================================== //
+// prefill
+// =========================================================================== //
+#define PF_WAVES 4
+#define PF_NQ 2                          // 16-row blocks per wave
+#define PF_ROWS (PF_WAVES * PF_NQ * 16)  // rows per workgroup
+#define PF_KEYS (D > 192 ? 32 : 64)      // keys per LDS tile (static LDS stays under 64 KB)
+#define PF_THREADS (PF_WAVES * RL_WAVE)
+#define K_LD (D + 8)                     // padded row of the K tile (bfloat16 elements)
+#define V_LD (PF_KEYS + 8)               // padded row of the V^T tile
+
+// tile_info[4 * tile + {0,1,2,3}] = {first token of the request's portion in the flat batch,
+//   tokens of the request already in the cache, tokens in this portion, first row of the tile}
+__global__ __launch_bounds__(PF_WAVES* RL_WAVE) void attn_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out,
+    const int* __restrict__ tile_info, const int* __restrict__ token_slot,
+    const int* __restrict__ block_table, int table_stride, int page_size, int nq, int nkv,
+    int window, float scale_log2) {
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_KEYS * K_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * V_LD];
+
+    const int G = nq / nkv;
+    const int tile = blockIdx.x;
+    const int hk = blockIdx.y;
+    const int tok0 = tile_info[4 * tile + 0];
+    const int start = tile_info[4 * tile + 1];
+    const int qlen = tile_info[4 * tile + 2];
+    const int row0 = tile_info[4 * tile + 3];
+    const int rows = qlen * G;
+    const int seq_end = start + qlen;  // keys at or beyond this were never written
+    const int* table = block_table + (size_t)token_slot[tok0] * table_stride;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (RL_WAVE - 1);
+    const int wave = tid / RL_WAVE;
+    const int col = lane & 15;
+    const int g = lane >> 4;
+
+    // rows of this lane: one per 16-row block
+    int r_tok[PF_NQ], r_head[PF_NQ], r_pos[PF_NQ];
+    bool r_ok[PF_NQ];
+    bf16x8 qf[PF_NQ][DC];
+#pragma unroll
+    for (int n = 0; n < PF_NQ; ++n) {
+        const int row = row0 + (wave * PF_NQ + n) * 16 + col;
+        r_ok[n] = row < rows;
+        const int rr = r_ok[n] ? row : rows - 1;
+        r_tok[n] = tok0 + rr / G;
+        r_head[n] = hk * G + rr % G;
+        r_pos[n] = start + rr / G;
+        const bf16_t* qrow = q + ((size_t)r_tok[n] * nq + r_head[n]) * D;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
+            qf[n][c] = (r_ok[n] && chan_ok) ? load16(qrow + 32 * c + 8 * g) : zero8();
+        }
+    }
+    // keys the tile needs: up to the position of its last row; from the window of its first
+    const int last_row = min(row0 + PF_ROWS, rows) - 1;
+    const int tile_kend = start + last_row / G + 1;
+    const int first_pos = start + row0 / G;
+    const int tile_kstart = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+
+    float m[PF_NQ], l[PF_NQ];
+    f32x4 acc[PF_NQ][DB];
+#pragma unroll
+    for (int n = 0; n < PF_NQ; ++n) {
+        m[n] = -INFINITY;
+        l[n] = 0.f;
+#pragma unroll
+        for (int b = 0; b < DB; ++b) acc[n][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+
+    for (int base = tile_kstart & ~(PF_KEYS - 1); base < tile_kend; base += PF_KEYS) {
+        __syncthreads();  // the previous tile has been consumed
+        // ---- stage K: PF_THREADS / PF_KEYS threads share one key row -------------------
+        {
+            constexpr int TPK = PF_THREADS / PF_KEYS;
+            const int kk = tid / TPK;
+            const int key = min(base + kk, seq_end - 1);  // clamped; masked by position below
+            const int page = table[key / page_size];
+            const bf16_t* krow =
+                k_cache + (((size_t)page * nkv + hk) * page_size + key % page_size) * D;
+            for (int ch = tid % TPK; ch < D / 8; ch += TPK)
+                *reinterpret_cast<uint4*>(&Ks[kk * K_LD + 8 * ch]) =
+                    *reinterpret_cast<const uint4*>(krow + 8 * ch);
+        }
+        // ---- stage V^T: thread -> (group of 4 keys, channel d, d + PF_THREADS / groups, ..) --
+        {
+            constexpr int KG = PF_KEYS / 4;
+            const int kg = tid % KG;
+            const int key = base + 4 * kg;
+            const int keyc = min(key, (seq_end - 1) & ~3);
+            const int page = table[keyc / page_size];
+            const bf16_t* vbase =
+                v_cache + (((size_t)page * nkv + hk) * D) * page_size + keyc % page_size;
+            // keys of the group that may be multiplied: written ones (below seq_end) that no
+            // row's window has left behind (their pages may have been given back already)
+            const int lo_cut = tile_kstart - key;  // keys i < lo_cut are out
+            const int hi_cut = seq_end - key;      // keys i >= hi_cut are out
+            const bool all_in = lo_cut <= 0 && hi_cut >= 4;
+            unsigned keep_x = 0, keep_y = 0;  // never multiply stale data, not even by zero
+            if (0 >= lo_cut && 0 < hi_cut) keep_x |= 0x0000ffffu;
+            if (1 >= lo_cut && 1 < hi_cut) keep_x |= 0xffff0000u;
+            if (2 >= lo_cut && 2 < hi_cut) keep_y |= 0x0000ffffu;
+            if (3 >= lo_cut && 3 < hi_cut) keep_y |= 0xffff0000u;
+            for (int d = tid / KG; d < D; d += PF_THREADS / KG) {
+                uint2 v = *reinterpret_cast<const uint2*>(vbase + (size_t)d * page_size);
+                if (!all_in) {
+                    v.x &= keep_x;
+                    v.y &= keep_y;
+                }
+                *reinterpret_cast<uint2*>(&Vs[d * V_LD + 4 * kg]) = v;
+            }
+        }
+        __syncthreads();
+        // ---- steps of 32 keys -----------------------------------------------------
+#pragma unroll
+        for (int hf = 0; hf < PF_KEYS / 32; ++hf) {
+            const int kb0 = base + 32 * hf;
+            if (kb0 >= tile_kend) break;  // uniform
+            bf16x8 kf[2][DC];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int c = 0; c < DC; ++c) {
+                    const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
+                    kf[kb][c] = chan_ok
+                                    ? load16(&Ks[(32 * hf + 16 * kb + col) * K_LD + 32 * c + 8 * g])
+                                    : zero8();
+                }
+            bf16x8 p[PF_NQ];
+#pragma unroll
+            for (int n = 0; n < PF_NQ; ++n) {
+                f32x4 s[2];
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    s[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int c = 0; c < DC; ++c) s[kb] = mfma(kf[kb][c], qf[n][c], s[kb]);
+                }
+                unsigned ok[2];
+                const int pos = r_pos[n];
+                const int wlo = (window > 0) ? pos - window + 1 : 0;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    ok[kb] = 0;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = kb0 + 16 * kb + 4 * g + i;
+                        ok[kb] |= (key <= pos && key >= wlo) ? (1u << i) : 0u;
+                    }
+                }
+                p[n] = softmax_step(s[0], s[1], ok[0], ok[1], scale_log2, m[n], l[n], acc[n]);
+            }
+#pragma unroll
+            for (int b = 0; b < DB; ++b) {
+                const bf16_t* vr = &Vs[(16 * b + col) * V_LD + 32 * hf + 4 * g];
+                const bf16x8 v = load8x2(vr, vr + 16);
+#pragma unroll
+                for (int n = 0; n < PF_NQ; ++n) acc[n][b] = mfma(v, p[n], acc[n][b]);
+            }
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < PF_NQ; ++n) {
+        const float lt = row_sum4(l[n]);
+        const float inv = lt > 0.f ? 1.f / lt : 0.f;
+        if (!r_ok[n]) continue;
+        bf16_t* orow = out + ((size_t)r_tok[n] * nq + r_head[n]) * D;
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+            struct {
+                bf16_t v[4];
+            } o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o.v[i] = float_to_bf16(acc[n][b][i] * inv);
+            *reinterpret_cast<uint2*>(orow + 16 * b + 4 * g) = __builtin_bit_cast(uint2, o);
+        }
+    }
+}
+
+extern "C" int rl_attn_prefill_rows() { return PF_ROWS; }
+
+extern "C" int rl_attn_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                               const int* tile_info, int num_tiles, const int* token_slot,
+                               const int* block_table, int table_stride, int page_size, int nq,
+                               int nkv, int window, float scale, hipStream_t stream) {
+    if (num_tiles <= 0) return RL_OK;
+    if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535) return RL_ERR_ARG;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    dim3 grid(num_tiles, nkv), block(PF_WAVES * RL_WAVE);
+    hipLaunchKernelGGL(attn_prefill_kernel, grid, block, 0, stream, (const bf16_t*)q,
+                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_info,
+                       token_slot, block_table, table_stride, page_size, nq, nkv, window,
+                       scale_log2);
+    return rl_launch_status();
+}

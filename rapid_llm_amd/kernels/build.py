@@ -42,9 +42,9 @@ CORE_SOURCES = (
 ATTENTION_SOURCES = ("attention_mfma.hip",)
 HEADERS = ("common.h",)
 
-# head sizes built ahead of time by build_all(); any other multiple of 16 up to 256 is
-# compiled when a model first asks for it
-DEFAULT_HEAD_DIMS = (16, 32, 64, 128)
+# head sizes built ahead of time by build_all(): every one the kernels take.  A fresh
+# checkout compiles only the head size of the model it is asked to run.
+DEFAULT_HEAD_DIMS = tuple(range(16, 257, 16))
 
 _HIPCC_FLAGS = (
     "-O3",
@@ -88,9 +88,8 @@ def build_dir() -> Path:
     path = CSRC / "_build"
     try:
         path.mkdir(parents=True, exist_ok=True)
-        probe = path / f".probe-{os.getpid()}"
-        probe.write_bytes(b"")
-        probe.unlink()
+        with tempfile.NamedTemporaryFile(dir=path, prefix=".probe-"):
+            pass
         return path
     except OSError:
         path = Path(tempfile.gettempdir()) / f"rapid_llm_amd-build-{os.getuid()}"
@@ -212,7 +211,7 @@ def build_all(head_dims: tuple[int, ...] = DEFAULT_HEAD_DIMS, force: bool = True
     out = [core_library(force=force)]
     if not all((CSRC / s).is_file() for s in ATTENTION_SOURCES):
         return out
-    with ThreadPoolExecutor(min(4, len(head_dims))) as pool:
+    with ThreadPoolExecutor(min(8, len(head_dims))) as pool:
         out += list(pool.map(lambda d: attention_library(d, force=force), head_dims))
     return out
 

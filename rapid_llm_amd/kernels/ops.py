@@ -44,6 +44,8 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
     lib = _attn.get(head_dim)
     if lib is None:
         lib = build.load(build.attention_library(head_dim))
+        if lib.rl_attn_head_dim() != head_dim:
+            raise KernelError(f"attention library for head size {head_dim} reports {lib.rl_attn_head_dim()}")
         _attn[head_dim] = lib
     return lib
 
@@ -291,6 +293,37 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch
     return torch.matmul(x, w.t())
 
 
+class AttentionPlan:
+    """Per-step launch data of the matrix-core attention kernels for one group size G
+    (query heads per kv head): which requests are single tokens (decode kernel) and how the
+    portions of the others are cut into row tiles (prefill kernel)."""
+
+    __slots__ = ("num_decode", "seq_token", "max_decode_ctx", "num_tiles", "tile_info")
+
+    def __init__(self, ctx, group: int, tile_rows: int) -> None:
+        dec_tokens: list[int] = []
+        tiles: list[int] = []
+        self.max_decode_ctx = 0
+        at = 0
+        for start, n in zip(ctx.h_seq_starts, ctx.h_seq_lens):
+            if n == 1:
+                dec_tokens.append(at)
+                self.max_decode_ctx = max(self.max_decode_ctx, start + 1)
+            else:
+                for row0 in range(0, n * group, tile_rows):
+                    tiles += (at, start, n, row0)
+            at += n
+        self.num_decode = len(dec_tokens)
+        self.num_tiles = len(tiles) // 4
+        device = ctx.token_ids.device
+        packed = torch.tensor(dec_tokens + tiles, dtype=torch.int32).to(device)
+        self.seq_token = packed[: self.num_decode]
+        self.tile_info = packed[self.num_decode :]
+
+
+_TARGET_BLOCKS = 1024  # workgroups a decode launch should reach: a few per compute unit
+
+
 def paged_attention(
     q: torch.Tensor,
     k_cache: torch.Tensor,
@@ -305,8 +338,64 @@ def paged_attention(
     window: int,
     scale: float,
 ) -> None:
-    """Attention of every token of the step over its request's cached keys."""
-    attention_generic(
-        q, k_cache, v_cache, out, ctx.positions, ctx.token_slot, block_table, page_size,
-        nq, nkv, d, window, scale, ctx.max_position,
-    )
+    """Attention of every token of the step over its request's cached keys.
+
+    float32 runs the FMA kernel.  bfloat16 runs the matrix-core kernels: single tokens go
+    to the split-key decode kernel, portions to the tiled prefill kernel."""
+    if q.dtype != torch.bfloat16:
+        attention_generic(
+            q, k_cache, v_cache, out, ctx.positions, ctx.token_slot, block_table, page_size,
+            nq, nkv, d, window, scale, ctx.max_position,
+        )
+        return
+    tokens = q.shape[0]
+    pages = k_cache.shape[0]
+    _need(q, "q", torch.bfloat16, (tokens, nq * d))
+    _need(out, "out", torch.bfloat16, (tokens, nq * d))
+    _need(k_cache, "k_cache", torch.bfloat16, (pages, nkv, page_size, d))
+    _need(v_cache, "v_cache", torch.bfloat16, (pages, nkv, d, page_size))
+    _need(block_table, "block_table", torch.int32)
+    if page_size % 4:
+        raise KernelError(f"the matrix-core attention kernels need a page size that is a multiple of 4, got {page_size}")
+    if ctx.max_position // page_size >= block_table.shape[1]:
+        raise KernelError(
+            f"position {ctx.max_position} needs page {ctx.max_position // page_size} of a block "
+            f"table with {block_table.shape[1]} columns"
+        )
+    lib = attention_lib(d)
+    group = nq // nkv
+    key = ("attention_plan", group)
+    plan = ctx.extra.get(key)
+    if plan is None:
+        plan = AttentionPlan(ctx, group, lib.rl_attn_prefill_rows())
+        ctx.extra[key] = plan
+    if plan.num_tiles:
+        _ok(
+            lib.rl_attn_prefill(
+                _p(q), _p(k_cache), _p(v_cache), _p(out), _p(plan.tile_info), plan.num_tiles,
+                _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv,
+                window, ctypes.c_float(scale), _stream(),
+            ),
+            "rl_attn_prefill",
+        )
+    if plan.num_decode:
+        span = plan.max_decode_ctx
+        if window > 0:
+            span = min(span, window + 31)
+        pairs = plan.num_decode * nkv * ((group + 15) // 16)
+        want = max(1, _TARGET_BLOCKS // pairs)
+        chunk = max(128, -(-(-(-span // want)) // 128) * 128)
+        nsplit = -(-span // chunk)
+        part_o = part_ml = None
+        if nsplit > 1:
+            part_o = torch.empty((plan.num_decode, nq, nsplit, d), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((plan.num_decode, nq, nsplit, 2), dtype=torch.float32, device=q.device)
+        _ok(
+            lib.rl_attn_decode(
+                _p(q), _p(k_cache), _p(v_cache), _p(out), _p(part_o), _p(part_ml),
+                _p(plan.seq_token), _p(ctx.positions), _p(ctx.token_slot), _p(block_table),
+                block_table.stride(0), page_size, plan.num_decode, nq, nkv, window,
+                ctypes.c_float(scale), chunk, nsplit, _stream(),
+            ),
+            "rl_attn_decode",
+        )

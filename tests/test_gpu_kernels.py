@@ -1,0 +1,294 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the tiny models'."""
+
+import math
+import random
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from plain_model import plain_attention, plain_inv_freq, plain_rmsnorm, plain_rope_apply, plain_rope_tables
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _ops():
+    from rapid_llm_amd.kernels import ops
+
+    return ops
+
+
+# --------------------------------------------------------------------------- #
+# a paged cache laid out by hand: pages in shuffled order, everything else NaN
+# --------------------------------------------------------------------------- #
+def _paged_problem(seqs, nq, nkv, d, page, dtype, seed, window=0, spike=None):
+    """``seqs`` = list of (tokens already cached, tokens in this step).  Returns the kernel
+    operands and the expected output from the plain attention."""
+    rng = random.Random(seed)
+    gen = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-(a + n) // page) for a, n in seqs) + 1
+    order = list(range(1, total_pages))
+    rng.shuffle(order)
+    max_pages = max(-(-(a + n) // page) for a, n in seqs) + 2
+    table = torch.zeros((len(seqs) + 3, max_pages), dtype=torch.int32)
+    k_cache = torch.full((total_pages, nkv, page, d), float("nan"))
+    v_cache = torch.full((total_pages, nkv, d, page), float("nan"))
+    slots = list(range(len(seqs) + 3))
+    rng.shuffle(slots)
+    q_rows, positions, token_slot, expect = [], [], [], []
+    for i, (a, n) in enumerate(seqs):
+        t = a + n
+        k = torch.randn((t, nkv, d), generator=gen)
+        v = torch.randn((t, nkv, d), generator=gen)
+        q = torch.randn((n, nq, d), generator=gen)
+        if spike is not None and i == spike[0]:
+            # one far key carries nearly all of the softmax mass of the last query
+            far = spike[1]
+            group = nq // nkv
+            for j in range(nkv):
+                u = q[-1, j * group].clone()
+                q[-1, j * group : (j + 1) * group] = u  # the heads of a group ask alike
+                k[far, j] = u * (30.0 * math.sqrt(d) / float(u @ u))  # score 30 against ~N(0,1)
+            v[far] = 7.0
+        if dtype == torch.bfloat16:
+            q, k, v = (x.bfloat16().float() for x in (q, k, v))
+        slot = slots[i]
+        for p in range(-(-t // page)):
+            pid = order.pop()
+            table[slot, p] = pid
+            lo, hi = p * page, min(t, (p + 1) * page)
+            k_cache[pid, :, : hi - lo, :] = k[lo:hi].transpose(0, 1)
+            v_cache[pid, :, :, : hi - lo] = v[lo:hi].permute(1, 2, 0)
+        qpos = torch.arange(a, t)
+        expect.append(
+            plain_attention(q, k, v, 1.0 / math.sqrt(d), window or None, qpos, torch.arange(t)).reshape(n, nq * d)
+        )
+        q_rows.append(q.reshape(n, nq * d))
+        positions += list(range(a, t))
+        token_slot += [slot] * n
+    ctx = SimpleNamespace(
+        positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+        token_slot=torch.tensor(token_slot, dtype=torch.int32, device=DEV),
+        token_ids=torch.zeros(len(positions), dtype=torch.int32, device=DEV),
+        h_seq_starts=[a for a, _ in seqs],
+        h_seq_lens=[n for _, n in seqs],
+        max_position=max(positions),
+        extra={},
+    )
+    return (
+        torch.cat(q_rows).to(DEV, dtype),
+        k_cache.to(DEV, dtype),
+        v_cache.to(DEV, dtype),
+        table.to(DEV),
+        ctx,
+        torch.cat(expect),
+    )
+
+
+ATTN_CASES = [
+    # nq, nkv, d, page, window, seqs
+    (7, 7, 16, 4, 0, [(0, 5), (37, 1), (3, 2)]),
+    (12, 3, 48, 8, 0, [(0, 130), (200, 1), (64, 33), (0, 1)]),
+    (20, 1, 80, 16, 0, [(300, 1), (5, 70), (0, 2)]),          # 20 heads on one kv head
+    (8, 2, 128, 16, 0, [(700, 1), (0, 257), (511, 1), (100, 29)]),
+    (4, 4, 256, 32, 0, [(90, 1), (0, 75)]),
+    (6, 2, 64, 4, 19, [(0, 90), (45, 1), (200, 1), (30, 31)]),  # window
+    (10, 5, 112, 12, 40, [(333, 1), (77, 50)]),
+]
+
+
+@pytest.mark.parametrize("case", ATTN_CASES, ids=lambda c: f"h{c[0]}kv{c[1]}d{c[2]}p{c[3]}w{c[4]}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_paged_attention(case, dtype):
+    ops = _ops()
+    nq, nkv, d, page, window, seqs = case
+    q, kc, vc, table, ctx, want = _paged_problem(seqs, nq, nkv, d, page, dtype, seed=len(seqs) * 7 + d, window=window)
+    out = torch.full_like(q, float("nan"))
+    ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, window, 1.0 / math.sqrt(d))
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=2e-6)
+    else:
+        torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("far", [3, 257, 640])
+def test_attention_finds_a_far_key(dtype, far):
+    """One key among hundreds holds the mass: a kernel that skips or misplaces its page
+    returns something far from that key's value (7.0 in every channel)."""
+    ops = _ops()
+    nq, nkv, d, page = 8, 2, 128, 16
+    for seqs, who in (([(699, 1), (10, 1)], 0), ([(5, 1), (100, 600)], 1)):
+        q, kc, vc, table, ctx, want = _paged_problem(seqs, nq, nkv, d, page, dtype, seed=far, spike=(who, far))
+        out = torch.empty_like(q)
+        ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, 0, 1.0 / math.sqrt(d))
+        got = out.float().cpu()
+        row = 0 if who == 0 else got.shape[0] - 1
+        assert (want[row] > 6.5).all()  # the construction works in the plain attention
+        torch.testing.assert_close(got[row], want[row], rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+
+
+def test_attention_window_edge():
+    """Keys exactly at and just outside the window's edge: the key one step too far holds a
+    huge value; it must not leak into the result."""
+    ops = _ops()
+    nq, nkv, d, page, window = 4, 2, 64, 8, 33
+    for dtype in (torch.float32, torch.bfloat16):
+        for seqs in ([(100, 1)], [(60, 41)]):
+            q, kc, vc, table, ctx, want = _paged_problem(seqs, nq, nkv, d, page, dtype, seed=5, window=window)
+            out = torch.empty_like(q)
+            ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, window, 1.0 / math.sqrt(d))
+            tol = dict(rtol=1e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+            torch.testing.assert_close(out.float().cpu(), want, **tol)
+
+
+# --------------------------------------------------------------------------- #
+# norms, activation, rotation, cache write, products, embedding, arg-max
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("hidden", [80, 1000, 4096])
+def test_add_rmsnorm(dtype, hidden):
+    ops = _ops()
+    t = 37
+    res = torch.randn(t, hidden)
+    delta = torch.randn(t, hidden).to(dtype)
+    w = 1 + 0.1 * torch.randn(hidden)
+    eps = 3e-5
+    want_res = res + delta.float()
+    want = plain_rmsnorm(want_res, w, eps)
+    r = res.to(DEV)
+    out = torch.empty(t, hidden, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(r, delta.to(DEV), w.to(DEV), out, eps)
+    torch.testing.assert_close(r.cpu(), want_res, rtol=0, atol=0)  # residual updated in place
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=8e-3, atol=8e-3)
+    torch.testing.assert_close(out.float().cpu(), want, **tol)
+    # without a delta, and for chosen rows only
+    rows = torch.tensor([5, 0, 36], dtype=torch.int32)
+    out2 = torch.empty(3, hidden, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(r, None, w.to(DEV), out2, eps, rows.to(DEV))
+    torch.testing.assert_close(out2.float().cpu(), want[rows.long()], **tol)
+    # unit RMS with weight one
+    ones = torch.ones(hidden, device=DEV)
+    out3 = torch.empty(t, hidden, dtype=torch.float32, device=DEV)
+    ops.add_rmsnorm(r, None, ones, out3, 0.0)
+    torch.testing.assert_close(out3.square().mean(-1).cpu(), torch.ones(t), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_swiglu(dtype):
+    ops = _ops()
+    t, inter = 19, 333
+    x = torch.randn(t, 2 * inter).to(dtype)
+    want = torch.nn.functional.silu(x[:, :inter].float()) * x[:, inter:].float()
+    out = torch.empty(t, inter, dtype=dtype, device=DEV)
+    ops.swiglu(x.to(DEV), out)
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=8e-3, atol=8e-3)
+    torch.testing.assert_close(out.float().cpu(), want, **tol)
+    x[:, :inter] = 0  # zero gate => zero
+    ops.swiglu(x.to(DEV), out)
+    assert (out == 0).all()
+
+
+def test_rope_table_matches_plain():
+    ops = _ops()
+    for d, theta in ((16, 1e4), (48, 5e5), (128, 1e6)):
+        cos, sin = ops.rope_table(plain_inv_freq(d, theta).to(DEV), 5000)
+        wc, ws = plain_rope_tables(torch.arange(5000), d, theta)
+        torch.testing.assert_close(cos.cpu(), wc, rtol=0, atol=1e-7)
+        torch.testing.assert_close(sin.cpu(), ws, rtol=0, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(5, 5, 48, 8), (6, 2, 128, 16), (3, 1, 16, 4), (4, 4, 256, 4)])
+def test_qknorm_rope_kvwrite(dtype, shape):
+    ops = _ops()
+    nq, nkv, d, page = shape
+    theta, eps = 77777.0, 2e-5
+    positions = [0, 1, 2, 9, 300, 301, 4000]
+    slots = [2, 2, 2, 0, 1, 1, 3]
+    t = len(positions)
+    qkv = torch.randn(t, (nq + 2 * nkv) * d).to(dtype)
+    qw = 1 + 0.1 * torch.randn(d)
+    kw = 1 + 0.1 * torch.randn(d)
+    max_pages = 4001 // page + 1
+    table = torch.zeros((4, max_pages), dtype=torch.int32)
+    pid = 1
+    for p, s in zip(positions, slots):
+        if table[s, p // page] == 0:
+            table[s, p // page] = pid
+            pid += 1
+    kc = torch.full((pid, nkv, page, d), float("nan"), dtype=dtype, device=DEV)
+    vc = torch.full((pid, nkv, d, page), float("nan"), dtype=dtype, device=DEV)
+    cos, sin = ops.rope_table(plain_inv_freq(d, theta).to(DEV), 4001)
+    q_out = torch.empty(t, nq * d, dtype=dtype, device=DEV)
+    ops.qknorm_rope_kvwrite(
+        qkv.to(DEV), q_out, kc, vc, qw.to(DEV), kw.to(DEV), cos, sin,
+        torch.tensor(positions, dtype=torch.int32, device=DEV),
+        torch.tensor(slots, dtype=torch.int32, device=DEV), table.to(DEV), page, nq, nkv, d, eps, max(positions),
+    )
+    x = qkv.float()
+    q = x[:, : nq * d].view(t, nq, d)
+    k = x[:, nq * d : (nq + nkv) * d].view(t, nkv, d)
+    v = x[:, (nq + nkv) * d :].view(t, nkv, d)
+    pc, ps = plain_rope_tables(torch.tensor(positions), d, theta)
+    want_q = plain_rope_apply(plain_rmsnorm(q, qw, eps), pc, ps).reshape(t, nq * d)
+    want_k = plain_rope_apply(plain_rmsnorm(k, kw, eps), pc, ps)
+    tol = dict(rtol=1e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=8e-3, atol=8e-3)
+    torch.testing.assert_close(q_out.float().cpu(), want_q, **tol)
+    kc, vc = kc.float().cpu(), vc.float().cpu()
+    written_k = torch.zeros_like(kc, dtype=torch.bool)
+    for i, (p, s) in enumerate(zip(positions, slots)):
+        page_id, off = int(table[s, p // page]), p % page
+        torch.testing.assert_close(kc[page_id, :, off, :], want_k[i], **tol)
+        torch.testing.assert_close(vc[page_id, :, :, off], v[i], rtol=0, atol=0)
+        written_k[page_id, :, off, :] = True
+    assert torch.isnan(kc[~written_k]).all()  # nothing else was touched
+
+
+@pytest.mark.parametrize("shape", [(1, 96, 64), (7, 503, 96), (130, 200, 333), (64, 64, 16)])
+def test_gemm_f32(shape):
+    ops = _ops()
+    m, n, k = shape
+    a, w = torch.randn(m, k), torch.randn(n, k)
+    out = torch.empty(m, n, device=DEV)
+    ops.gemm_f32(a.to(DEV), w.to(DEV), out)
+    want = (a.double() @ w.double().T).float()
+    torch.testing.assert_close(out.cpu(), want, rtol=1e-5, atol=1e-5 * math.sqrt(k))
+    # a row's result does not depend on the rows beside it
+    out1 = torch.empty(1, n, device=DEV)
+    ops.gemm_f32(a[m // 2 : m // 2 + 1].to(DEV), w.to(DEV), out1)
+    assert torch.equal(out1[0], out[m // 2])
+
+
+@pytest.mark.parametrize("shape", [(1, 503, 96), (8, 4096, 4096), (64, 1000, 12288), (200, 331, 80), (3, 24, 48)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16out", "f32out"])
+def test_gemm_bf16(shape, out_dtype):
+    ops = _ops()
+    m, n, k = shape
+    a = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    got = ops.gemm_bf16(a.to(DEV), w.to(DEV), out_dtype)
+    want = a.float() @ w.float().T
+    tol = dict(rtol=1e-2, atol=1e-2) if got.dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(got.float().cpu(), want, **tol)
+
+
+def test_embed_and_argmax():
+    ops = _ops()
+    vocab, hidden = 503, 96
+    for dtype in (torch.float32, torch.bfloat16):
+        table = torch.randn(vocab, hidden).to(dtype)
+        ids = torch.tensor([0, 502, 17, 17, 250], dtype=torch.int32)
+        out = torch.empty(5, hidden, device=DEV)
+        ops.embed(ids.to(DEV), table.to(DEV), out)
+        assert torch.equal(out.cpu(), table.float()[ids.long()])
+    logits = torch.randn(9, 151936)
+    logits[3, 777] = logits[3, 90000] = 50.0  # a tie: the lower index wins
+    out = torch.empty(9, dtype=torch.int32, device=DEV)
+    ops.argmax(logits.to(DEV), out)
+    assert out.cpu().tolist() == logits.argmax(-1).tolist()
+    assert int(out[3]) == 777
