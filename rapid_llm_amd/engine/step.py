@@ -141,6 +141,7 @@ class ModelRunner:
         self.device_cache = DeviceCache(self.cache, needs, group_of, self.dtype, self.device)
         self.computed: dict[str, int] = {}
         self.vocab_size = self.spec.vocab_size
+        self._graphs: dict[int, tuple] = {}
 
     # ------------------------------------------------------------------ sizing
     def _decide_num_pages(self, groups) -> int:
@@ -189,7 +190,7 @@ class ModelRunner:
         self.computed.pop(request_id, None)
 
     # ------------------------------------------------------------------ the step
-    def _prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+    def _prepare(self, entries: Sequence[StepEntry]):
         cache = self.cache
         seen = set()
         for e in entries:
@@ -254,14 +255,22 @@ class ModelRunner:
         host[offs[3] : offs[4]] = slots
         host[offs[4] : offs[5]] = starts
         host[offs[5] : offs[6]] = lens
-        dev = torch.from_numpy(host).to(self.device, non_blocking=False)
-        part = [dev[offs[i] : offs[i + 1]] for i in range(len(sizes))]
-
         self.device_cache.refresh()
-        return StepContext(
-            runtime=self.runtime,
+        return host, offs, dict(
             num_tokens=total,
             num_seqs=n_seq,
+            num_logit_rows=n_rows,
+            h_seq_slots=slots,
+            h_seq_starts=starts,
+            h_seq_lens=lens,
+            max_position=max(s + n for s, n in zip(starts, lens)) - 1,
+            max_seq_tokens=max(lens),
+        )
+
+    def _context(self, dev: torch.Tensor, offs, meta: dict) -> StepContext:
+        part = [dev[offs[i] : offs[i + 1]] for i in range(len(offs) - 1)]
+        return StepContext(
+            runtime=self.runtime,
             token_ids=part[0],
             positions=part[1],
             token_slot=part[2],
@@ -270,24 +279,69 @@ class ModelRunner:
             seq_lens=part[5],
             cu_seqlens=part[6],
             logit_rows=part[7],
-            num_logit_rows=n_rows,
             block_tables=self.device_cache.tables,
-            h_seq_slots=slots,
-            h_seq_starts=starts,
-            h_seq_lens=lens,
-            max_position=max(s + n for s, n in zip(starts, lens)) - 1,
-            max_seq_tokens=max(lens),
+            **meta,
         )
+
+    # ------------------------------------------------------------------ decode graphs
+    def _graph_step(self, entries, host, offs, meta) -> torch.Tensor:
+        """A step of single tokens, all wanted: replayed from a HIP graph captured once per
+        batch size.  The graph holds only this package's kernels; its inputs are one static
+        int32 buffer, refreshed by a copy on the same stream before each replay.  Launch
+        decisions that depend on the context length are made for the longest sequence the
+        engine allows, so one capture serves every step."""
+        batch = len(entries)
+        entry = self._graphs.get(batch)
+        if entry is None:
+            static = torch.zeros(len(host), dtype=torch.int32, device=self.device)
+            pinned = torch.empty(len(host), dtype=torch.int32, pin_memory=True)
+            pinned.numpy()[:] = host
+            static.copy_(pinned, non_blocking=True)
+            bound = dict(meta, max_position=self.engine.max_seq_len - 1)
+            ctx = self._context(static, offs, bound)
+            ctx.extra["decode_only_tokens"] = torch.arange(batch, dtype=torch.int32, device=self.device)
+            ctx.extra["context_bound"] = self.engine.max_seq_len
+            # one eager run on a side stream first: kernels get loaded, the allocator warm
+            current = torch.cuda.current_stream()
+            side = torch.cuda.Stream()
+            side.wait_stream(current)
+            with torch.cuda.stream(side):
+                self.model.forward(ctx, self.device_cache.layers)
+            current.wait_stream(side)
+            torch.cuda.synchronize()
+            ctx.extra = {k: v for k, v in ctx.extra.items() if k in ("decode_only_tokens", "context_bound")}
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(ctx, self.device_cache.layers)
+            # the graph's kernel nodes hold raw pointers: everything they point at that was
+            # allocated outside the capture (the static inputs, the index list in ctx.extra)
+            # must live as long as the graph does, so the context is kept with it
+            entry = (graph, static, pinned, logits, ctx)
+            self._graphs[batch] = entry
+        graph, static, pinned, logits, _ctx = entry
+        pinned.numpy()[:] = host
+        static.copy_(pinned, non_blocking=True)
+        graph.replay()
+        return logits
 
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run one batch; returns float32 logits ``[wanted, vocab]`` in the order of the
         entries and of each entry's ``want``.  Raises :class:`OutOfPages`, with nothing
-        changed, when slots or pages do not suffice."""
+        changed, when slots or pages do not suffice.  The returned tensor may be reused by
+        the next step: read it (sample from it, copy it) before stepping again."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
-        ctx = self._prepare(entries)
-        logits = self.model.forward(ctx, self.device_cache.layers)
+        host, offs, meta = self._prepare(entries)
+        if (
+            self.engine.use_graph
+            and len(entries) <= ops.SKINNY_MAX_ROWS
+            and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+        ):
+            logits = self._graph_step(entries, host, offs, meta)
+        else:
+            dev = torch.from_numpy(host).to(self.device, non_blocking=False)
+            logits = self.model.forward(self._context(dev, offs, meta), self.device_cache.layers)
         for e in entries:
             done = self.computed.get(e.request_id, 0) + len(e.tokens)
             self.computed[e.request_id] = done

@@ -38,6 +38,7 @@ CORE_SOURCES = (
     "gemm_f32.hip",
     "attention_generic.hip",
     "sampling.hip",
+    "gemm_bf16.hip",
 )
 ATTENTION_SOURCES = ("attention_mfma.hip",)
 HEADERS = ("common.h",)

@@ -282,15 +282,67 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _ok(core().rl_argmax(_p(logits), _p(out), rows, vocab, _stream()), "rl_argmax")
 
 
+SKINNY_MAX_ROWS = 64  # rows up to which the bandwidth-bound product is used
+SWIGLU_MAX_ROWS = 32
+_MIN_BLOCKS = 512  # workgroups a skinny product should reach before it widens its tiles
+
+
+def _skinny_tiles(rows: int, out_features: int, choices: tuple[int, ...]) -> int:
+    """Weight-row tiles per workgroup: the most the accumulators allow while the launch
+    still has a couple of workgroups per compute unit."""
+    mb = -(-rows // 16)
+    mbv = 1 if mb <= 1 else (2 if mb == 2 else 4)
+    best = None
+    for nt in choices:
+        if nt * mbv > 4:
+            continue
+        if best is None or -(-out_features // (16 * nt)) >= _MIN_BLOCKS:
+            best = nt
+    return best
+
+
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """``x[M,K] @ w[N,K]^T`` with bfloat16 operands and float32 accumulation.  Returns
-    bfloat16, or float32 when ``out_dtype`` is float32 and the kernel used can write it."""
+    """``x[M,K] @ w[N,K]^T`` with bfloat16 operands and float32 accumulation.
+
+    Few rows (decode) run the hand-written bandwidth-bound kernel, which can write float32
+    directly.  Many rows go to the library product, as the reference's dense products do
+    (``F.linear``); its bfloat16 result is returned as is and widened by the caller."""
     _need(x, "x", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
-    if x.shape[1] != w.shape[1]:
+    m, k = x.shape
+    n = w.shape[0]
+    if k != w.shape[1]:
         raise KernelError(f"gemm_bf16 shapes do not agree: x {tuple(x.shape)}, w {tuple(w.shape)}")
-    # the library product, as the reference's dense products are (F.linear)
+    if m <= SKINNY_MAX_ROWS and k % 8 == 0:
+        if out_dtype not in (torch.bfloat16, torch.float32):
+            raise KernelError(f"gemm_bf16 writes bfloat16 or float32, not {out_dtype}")
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        nt = _skinny_tiles(m, n, (1, 2, 4))
+        _ok(
+            core().rl_gemm_skinny(_p(x), _p(w), _p(out), m, n, k, k, k, n, _tag(out_dtype), nt, _stream()),
+            "rl_gemm_skinny",
+        )
+        return out
     return torch.matmul(x, w.t())
+
+
+def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor | None:
+    """``silu(x Wg^T) * (x Wu^T)`` for the packed ``[gate | up]`` matrix in one kernel, for
+    few rows; ``None`` when the shape is not one the fused kernel takes."""
+    m, k = x.shape
+    two_i = w_gate_up.shape[0]
+    if m > SWIGLU_MAX_ROWS or k % 8 or two_i % 2 or x.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16:
+        return None
+    _need(x, "x", torch.bfloat16)
+    _need(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, k))
+    inter = two_i // 2
+    out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
+    nt = _skinny_tiles(m, inter, (1, 2)) * 2  # pairs of (gate, up) tiles
+    _ok(
+        core().rl_gemm_skinny_swiglu(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, _stream()),
+        "rl_gemm_skinny_swiglu",
+    )
+    return out
 
 
 class AttentionPlan:
@@ -301,6 +353,15 @@ class AttentionPlan:
     __slots__ = ("num_decode", "seq_token", "max_decode_ctx", "num_tiles", "tile_info")
 
     def __init__(self, ctx, group: int, tile_rows: int) -> None:
+        fixed = ctx.extra.get("decode_only_tokens")
+        if fixed is not None:
+            # a step of single tokens whose index list is already on the device (graphs)
+            self.num_decode = fixed.numel()
+            self.seq_token = fixed
+            self.max_decode_ctx = max(ctx.h_seq_starts) + 1
+            self.num_tiles = 0
+            self.tile_info = None
+            return
         dec_tokens: list[int] = []
         tiles: list[int] = []
         self.max_decode_ctx = 0
@@ -379,7 +440,8 @@ def paged_attention(
             "rl_attn_prefill",
         )
     if plan.num_decode:
-        span = plan.max_decode_ctx
+        # under a graph the split is laid out for the longest context the engine allows
+        span = ctx.extra.get("context_bound", plan.max_decode_ctx)
         if window > 0:
             span = min(span, window + 31)
         pairs = plan.num_decode * nkv * ((group + 15) // 16)

@@ -46,6 +46,11 @@ class SwiGLU(FeedForward):
         self.down.bind(params[self.name + ".down"])
 
     def forward(self, x, ctx):
+        w = self.gate_up.weight
+        if w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
+            act = ops.gemm_bf16_swiglu(x, w)  # few rows: product and activation in one kernel
+            if act is not None:
+                return self.down(act)
         gu = self.gate_up(x)
         act = torch.empty((x.shape[0], self.intermediate_size), dtype=gu.dtype, device=x.device)
         ops.swiglu(gu, act)

@@ -277,6 +277,19 @@ def test_gemm_bf16(shape, out_dtype):
     torch.testing.assert_close(got.float().cpu(), want, **tol)
 
 
+@pytest.mark.parametrize("shape", [(1, 320, 96), (8, 12288, 4096), (32, 176, 80), (17, 100, 64)])
+def test_gemm_bf16_swiglu_fused(shape):
+    ops = _ops()
+    m, inter, k = shape
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(2 * inter, k) / math.sqrt(k)).bfloat16()
+    got = ops.gemm_bf16_swiglu(x.to(DEV), w.to(DEV))
+    gu = (x.float() @ w.float().T).bfloat16().float()
+    want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    torch.testing.assert_close(got.float().cpu(), want, rtol=2e-2, atol=2e-2)
+    assert ops.gemm_bf16_swiglu(torch.zeros(33, k, dtype=torch.bfloat16, device=DEV), w.to(DEV)) is None
+
+
 def test_embed_and_argmax():
     ops = _ops()
     vocab, hidden = 503, 96
