@@ -245,7 +245,13 @@ class CacheManager:
     def num_free_pages(self, group_id: int | None = None) -> int:
         if group_id is not None:
             return self.pools[group_id].num_free
-        return min(p.num_free for p in self.pools.values())
+        # a model without paged layers is never short of pages
+        return min((p.num_free for p in self.pools.values()), default=1 << 30)
+
+    def capacity_tokens(self) -> int:
+        """Positions one request can hold at most if it has the pool to itself."""
+        usable = min((p.num_usable for p in self.pools.values()), default=None)
+        return self.max_seq_len if usable is None else usable * self.page_size
 
     def check_invariants(self) -> None:
         """No page lost, none held twice: every held page sits in exactly one table cell."""

@@ -23,7 +23,6 @@ class EngineConfig:
     max_num_seqs: int = 32
     max_num_batched_tokens: int = 8192
     max_chunk_size: int = 512  # 0 turns chunked prefill off
-    enable_preemption: bool = False  # evict to admit; eviction under page pressure is always on
     use_graph: bool = True  # replay decode-only steps from a captured HIP graph
     seed: int = 0
 

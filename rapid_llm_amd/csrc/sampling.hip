@@ -48,3 +48,349 @@ extern "C" int rl_argmax(const float* logits, int* out, int rows, int vocab, hip
     hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, stream, logits, out, vocab);
     return rl_launch_status();
 }
+
+// --------------------------------------------------------------------------- //
+// General token selection, one workgroup of 1024 threads per row.
+//
+// In the order of rapid_llm/engine/sampler.py:641-718:
+//   1. repetition penalty over the tokens the request has generated so far, each token once:
+//      a negative logit is multiplied by the penalty, any other divided (:134-179);
+//   2. temperature 0: arg-max, lowest index among equals; done;
+//   3. probabilities softmax(logits / temperature) in float32;
+//   4. top_p == 1: one draw from the whole distribution (:218);
+//      otherwise the pool is the POOL most likely tokens in descending order, a token is
+//      dropped when the mass before it exceeds top_p, but only in a row whose pool reaches
+//      top_p at all (:234-244); the rest is renormalised and one token drawn.
+// The draw is the inverse of the cumulative distribution at u * (kept mass), with u in
+// [0, 1) a counter-based hash of (seed, counter): the same request draws the same tokens
+// whatever else is in the batch and however often it is recomputed.
+//
+// Per-row parameters, 8 int32 words: temperature, top_p, penalty (float bits), seed low,
+// seed high, counter, first and one-past-last index of its generated tokens in `history`.
+// --------------------------------------------------------------------------- //
+#define SMP_THREADS 1024
+#define SMP_WAVES (SMP_THREADS / RL_WAVE)
+#define SMP_POOL 1024  // candidates of nucleus sampling (rapid_llm/engine/sampler.py:186)
+
+__device__ inline uint32_t float_key(float v) {
+    // order-preserving map float -> uint32 (NaN sorts lowest)
+    if (v != v) return 0u;
+    const uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ inline float key_float(uint32_t k) {
+    const uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+    return __uint_as_float(u);
+}
+
+// splitmix64 of (seed + counter * golden ratio); the top 24 bits make u in [0, 1)
+__device__ __host__ inline float sample_uniform(uint32_t seed_lo, uint32_t seed_hi,
+                                                uint32_t counter) {
+    uint64_t z = (((uint64_t)seed_hi << 32) | seed_lo) +
+                 ((uint64_t)counter + 1ull) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+__device__ inline float wave_inclusive_scan(float v) {
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+#pragma unroll
+    for (int off = 1; off < RL_WAVE; off <<= 1) {
+        const float o = __shfl_up(v, off, RL_WAVE);
+        if (lane >= off) v += o;
+    }
+    return v;
+}
+
+__global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
+    const float* __restrict__ logits, const int* __restrict__ row_params,
+    const int* __restrict__ history, int* __restrict__ out, float* __restrict__ out_logprob,
+    int vocab, int bitmap_words) {
+    extern __shared__ uint32_t seen[];  // one bit per token id, when the row has a penalty
+    __shared__ unsigned long long cand[SMP_POOL];
+    __shared__ float cum[SMP_POOL];
+    __shared__ unsigned int hist[256];
+    __shared__ float scratch[16];
+    __shared__ float wave_tot[SMP_WAVES];
+    __shared__ float best_v[SMP_WAVES];
+    __shared__ int best_i[SMP_WAVES];
+    __shared__ unsigned int sh_u[4];
+    __shared__ int sh_i[2];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (RL_WAVE - 1), wave = tid / RL_WAVE;
+    const int* rp = row_params + 8 * blockIdx.x;
+    const float temperature = __int_as_float(rp[0]);
+    const float top_p = __int_as_float(rp[1]);
+    const float penalty = __int_as_float(rp[2]);
+    const bool penalise = bitmap_words > 0 && penalty != 1.0f && rp[7] > rp[6];
+    const bool greedy = !(temperature > 0.f);
+    const float inv_t = greedy ? 1.f : 1.f / temperature;
+    const float* row = logits + (size_t)blockIdx.x * vocab;
+
+    if (penalise) {
+        for (int i = tid; i < bitmap_words; i += SMP_THREADS) seen[i] = 0u;
+        __syncthreads();
+        for (int i = rp[6] + tid; i < rp[7]; i += SMP_THREADS) {
+            const int tok = history[i];
+            if (tok >= 0 && tok < vocab) atomicOr(&seen[tok >> 5], 1u << (tok & 31));
+        }
+        __syncthreads();
+    }
+    // z(i): penalised logit over temperature
+    auto zval = [&](int i) -> float {
+        float x = row[i];
+        if (penalise && ((seen[i >> 5] >> (i & 31)) & 1u)) x = x < 0.f ? x * penalty : x / penalty;
+        return x * inv_t;
+    };
+
+    // ---- maximum and arg-max (lowest index among equals; NaN never wins) -----------------
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = tid; i < vocab; i += SMP_THREADS) {
+        const float v = zval(i);
+        if (v > bv || (v == bv && i < bi)) {
+            bv = v;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = RL_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, RL_WAVE);
+        const int oi = __shfl_xor(bi, off, RL_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if (lane == 0) {
+        best_v[wave] = bv;
+        best_i[wave] = bi;
+    }
+    __syncthreads();
+    bv = best_v[0];
+    bi = best_i[0];
+    for (int w = 1; w < SMP_WAVES; ++w)
+        if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+            bv = best_v[w];
+            bi = best_i[w];
+        }
+    if (bi == 0x7fffffff) bi = 0;  // a row of NaN or -inf
+    const float zmax = bv;
+
+    // ---- sum of exp, in a fixed order: wave w owns a contiguous segment -------------------
+    // (needed for the probabilities and for the logprob of the chosen token)
+    const int seg = ((vocab + SMP_WAVES - 1) / SMP_WAVES + RL_WAVE - 1) / RL_WAVE * RL_WAVE;
+    const int seg_lo = min(vocab, wave * seg), seg_hi = min(vocab, seg_lo + seg);
+    float wsum = 0.f;
+    if (!greedy || out_logprob) {
+        for (int base = seg_lo; base < seg_hi; base += RL_WAVE) {
+            const int i = base + lane;
+            wsum += (i < seg_hi) ? expf(zval(i) - zmax) : 0.f;
+        }
+        wsum = wave_sum(wsum);
+        if (lane == 0) wave_tot[wave] = wsum;
+    }
+    __syncthreads();
+    float total = 0.f;
+    if (!greedy || out_logprob)
+        for (int w = 0; w < SMP_WAVES; ++w) total += wave_tot[w];
+
+    if (greedy) {
+        if (tid == 0) {
+            out[blockIdx.x] = bi;
+            if (out_logprob) out_logprob[blockIdx.x] = -logf(total);  // z - zmax = 0
+        }
+        return;
+    }
+    const float u = sample_uniform((uint32_t)rp[3], (uint32_t)rp[4], (uint32_t)rp[5]);
+
+    if (top_p >= 1.0f) {
+        // ---- one draw from the whole distribution: first i with cumsum(i) >= u * total ----
+        const float target = u * total;
+        float before = 0.f;
+        int owner = SMP_WAVES - 1;
+        for (int w = 0; w < SMP_WAVES; ++w) {
+            if (before + wave_tot[w] >= target && wave_tot[w] > 0.f) {
+                owner = w;
+                break;
+            }
+            before += wave_tot[w];
+        }
+        // rounding may leave the target just beyond the last wave with mass: fall back to it
+        while (owner > 0 && !(wave_tot[owner] > 0.f)) --owner;
+        if (wave != owner) return;
+        float run = 0.f;
+        for (int w = 0; w < owner; ++w) run += wave_tot[w];
+        int chosen = -1, last_mass = -1;
+        for (int base = seg_lo; base < seg_hi && chosen < 0; base += RL_WAVE) {
+            const int i = base + lane;
+            const float e = (i < seg_hi) ? expf(zval(i) - zmax) : 0.f;
+            const float inc = wave_inclusive_scan(e) + run;
+            const unsigned long long hit = __ballot(e > 0.f && inc >= target);
+            const unsigned long long mass = __ballot(e > 0.f);
+            if (mass) last_mass = base + 63 - __clzll(mass);
+            if (hit) chosen = base + __ffsll((long long)hit) - 1;
+            run = __shfl(inc, RL_WAVE - 1, RL_WAVE);
+        }
+        if (chosen < 0) chosen = last_mass >= 0 ? last_mass : bi;
+        if (lane == 0) {
+            out[blockIdx.x] = chosen;
+            if (out_logprob) out_logprob[blockIdx.x] = zval(chosen) - zmax - logf(total);
+        }
+        return;
+    }
+
+    // ---- the pool: the k = min(POOL, vocab) largest z, by radix select on their keys ------
+    const int k = min(SMP_POOL, vocab);
+    uint32_t prefix = 0;
+    int k_rem = k;
+    if (vocab > SMP_POOL) {
+        for (int shift = 24; shift >= 0; shift -= 8) {
+            if (tid < 256) hist[tid] = 0u;
+            __syncthreads();
+            for (int i = tid; i < vocab; i += SMP_THREADS) {
+                const uint32_t key = float_key(zval(i));
+                if (shift == 24 || (key >> (shift + 8)) == prefix)
+                    atomicAdd(&hist[(key >> shift) & 255u], 1u);
+            }
+            __syncthreads();
+            if (tid == 0) {
+                int acc = 0, b = 255;
+                for (; b > 0; --b) {
+                    if (acc + (int)hist[b] >= k_rem) break;
+                    acc += (int)hist[b];
+                }
+                sh_u[0] = (prefix << 8) | (uint32_t)b;
+                sh_i[0] = k_rem - acc;
+                sh_i[1] = (int)hist[b];  // elements sharing the digits chosen so far
+            }
+            __syncthreads();
+            prefix = sh_u[0];
+            k_rem = sh_i[0];
+            __syncthreads();
+        }
+    }
+    const int equal_total = (vocab > SMP_POOL) ? sh_i[1] : 0;
+    // gather: keys above the threshold in any order (they are sorted afterwards); keys equal
+    // to it by ascending index until the pool is full
+    cand[tid] = 0ull;
+    if (tid == 0) sh_u[1] = 0u;
+    __syncthreads();
+    if (vocab <= SMP_POOL) {
+        if (tid < vocab)
+            cand[tid] = ((unsigned long long)float_key(zval(tid)) << 32) | (0xffffffffu - (uint32_t)tid);
+    } else {
+        const bool all_equal_fit = equal_total == k_rem;
+        for (int i = tid; i < vocab; i += SMP_THREADS) {
+            const uint32_t key = float_key(zval(i));
+            if (key > prefix || (all_equal_fit && key == prefix)) {
+                const unsigned int at = atomicAdd(&sh_u[1], 1u);
+                if (at < SMP_POOL)
+                    cand[at] = ((unsigned long long)key << 32) | (0xffffffffu - (uint32_t)i);
+            }
+        }
+        __syncthreads();
+        if (!all_equal_fit) {
+            // more equal keys than places: the lowest indices take them
+            int base_count = 0;
+            const int first_free = k - k_rem;
+            for (int base = 0; base < vocab && base_count < k_rem; base += SMP_THREADS) {
+                const int i = base + tid;
+                const bool eq = i < vocab && float_key(zval(i)) == prefix;
+                const unsigned long long bal = __ballot(eq);
+                if (lane == 0) hist[wave] = (unsigned int)__popcll(bal);
+                __syncthreads();
+                int before = base_count;
+                for (int w = 0; w < wave; ++w) before += (int)hist[w];
+                int tile_total = 0;
+                for (int w = 0; w < SMP_WAVES; ++w) tile_total += (int)hist[w];
+                const int rank = before + __popcll(bal & ((1ull << lane) - 1ull));
+                if (eq && rank < k_rem)
+                    cand[first_free + rank] =
+                        ((unsigned long long)prefix << 32) | (0xffffffffu - (uint32_t)i);
+                base_count += tile_total;
+                __syncthreads();
+            }
+        }
+    }
+    __syncthreads();
+    // ---- bitonic sort, descending (key, then lower index first) -----------------------------
+    for (int size = 2; size <= SMP_POOL; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            if (tid < SMP_POOL / 2) {
+                const int lo = 2 * tid - (tid & (stride - 1));
+                const int hi = lo + stride;
+                const bool desc = (lo & size) == 0;
+                const unsigned long long a = cand[lo], b = cand[hi];
+                if ((a < b) == desc) {
+                    cand[lo] = b;
+                    cand[hi] = a;
+                }
+            }
+            __syncthreads();
+        }
+    }
+    // ---- probabilities of the pool, their cumulative sums, the nucleus ----------------------
+    const float p = (tid < k) ? expf(key_float((uint32_t)(cand[tid] >> 32)) - zmax) / total : 0.f;
+    float inc = wave_inclusive_scan(p);
+    if (lane == RL_WAVE - 1) scratch[wave] = inc;
+    __syncthreads();
+    float off = 0.f;
+    for (int w = 0; w < wave; ++w) off += scratch[w];
+    inc += off;
+    cum[tid] = inc;
+    __syncthreads();
+    const float pool_mass = cum[SMP_POOL - 1];
+    const bool dropped = tid >= k || (pool_mass > top_p && inc - p > top_p);
+    // the kept tokens are a prefix of the pool (the mass before a token never decreases)
+    const unsigned long long kb = __ballot(!dropped);
+    if (lane == 0) hist[wave] = (unsigned int)__popcll(kb);
+    __syncthreads();
+    int n_keep = 0;
+    for (int w = 0; w < SMP_WAVES; ++w) n_keep += (int)hist[w];
+    if (n_keep < 1) n_keep = 1;
+    const float target = u * cum[n_keep - 1];
+    __syncthreads();
+    const unsigned long long below = __ballot(tid < n_keep && cum[tid] < target);
+    if (lane == 0) hist[wave] = (unsigned int)__popcll(below);
+    __syncthreads();
+    if (tid == 0) {
+        int j = 0;
+        for (int w = 0; w < SMP_WAVES; ++w) j += (int)hist[w];
+        if (j > n_keep - 1) j = n_keep - 1;
+        const int chosen = (int)(0xffffffffu - (uint32_t)(cand[j] & 0xffffffffull));
+        out[blockIdx.x] = chosen;
+        if (out_logprob)
+            out_logprob[blockIdx.x] =
+                key_float((uint32_t)(cand[j] >> 32)) - zmax - logf(total);
+    }
+}
+
+// the uniform draw of (seed, counter), for tests and for callers that mirror the draw
+extern "C" float rl_sample_uniform(unsigned int seed_lo, unsigned int seed_hi,
+                                   unsigned int counter) {
+    return sample_uniform(seed_lo, seed_hi, counter);
+}
+
+extern "C" int rl_sample_pool() { return SMP_POOL; }
+
+// history may be null when no row has a penalty.  out_logprob (optional): log-probability
+// of the chosen token under the penalised, temperature-scaled distribution.
+extern "C" int rl_sample(const float* logits, const int* row_params, const int* history, int* out,
+                         float* out_logprob, int rows, int vocab, int any_penalty,
+                         hipStream_t stream) {
+    if (rows <= 0) return RL_OK;
+    if (vocab < 1) return RL_ERR_ARG;
+    int words = 0;
+    if (any_penalty) {
+        words = (vocab + 31) / 32;
+        if ((size_t)words * 4 > 40 * 1024) return RL_ERR_ARG;  // the bitmap lives in LDS
+        if (!history) return RL_ERR_ARG;
+    }
+    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), (size_t)words * 4, stream,
+                       logits, row_params, history, out, out_logprob, vocab, words);
+    return rl_launch_status();
+}

@@ -1,0 +1,83 @@
+"""One generation request, from arrival to completion.
+
+Field names follow the reference's ``Request`` (rapid_llm/engine/batch_planner.py:25-150).
+The tokens a request has to run are ``prompt_token_ids + output_token_ids``;
+``num_computed_tokens`` of them are in the cache.  Whenever a step brings the last of
+them, the logits at that place choose the next token.  A prompt portion, a decoded token
+and the recomputation after an eviction are therefore the same thing: the next
+``n`` uncomputed tokens.
+"""
+
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from enum import Enum
+
+from ..sampling.params import SamplingParams
+
+
+class RequestStatus(str, Enum):
+    WAITING = "waiting"  # holds no slot and no pages
+    RUNNING = "running"  # holds one slot
+    FINISHED = "finished"
+
+
+@dataclass
+class Request:
+    request_id: str
+    prompt: str | None
+    prompt_token_ids: list[int]
+    params: SamplingParams
+    max_new_tokens: int = 0
+    seed: int = 0
+    num_computed_tokens: int = 0
+    arrival_time: float = field(default_factory=time.monotonic)
+    scheduled_time: float | None = None
+    admission_number: int = -1  # order of the latest admission: larger is younger
+    status: RequestStatus = RequestStatus.WAITING
+    output_token_ids: list[int] = field(default_factory=list)
+    output_logprobs: list[float] | None = None
+    text: str = ""
+    delta: str = ""
+    finish_reason: str | None = None  # "eos" | "length" | "repeat" | "abort"
+    first_token_time: float | None = None
+    finish_time: float | None = None
+    num_preemptions: int = 0
+
+    @property
+    def prompt_len(self) -> int:
+        return len(self.prompt_token_ids)
+
+    @property
+    def seq_len(self) -> int:
+        return len(self.prompt_token_ids) + len(self.output_token_ids)
+
+    @property
+    def num_uncomputed(self) -> int:
+        return self.seq_len - self.num_computed_tokens
+
+    @property
+    def is_finished(self) -> bool:
+        return self.status is RequestStatus.FINISHED
+
+    @property
+    def has_room(self) -> bool:
+        return len(self.output_token_ids) < self.max_new_tokens
+
+    @property
+    def prefill_done(self) -> bool:
+        """Everything but the newest token is in the cache: the next step is a decode."""
+        return self.num_uncomputed <= 1 and bool(self.output_token_ids)
+
+    def token_at(self, index: int) -> int:
+        n = len(self.prompt_token_ids)
+        return self.prompt_token_ids[index] if index < n else self.output_token_ids[index - n]
+
+    def tokens(self, start: int, stop: int) -> list[int]:
+        n = len(self.prompt_token_ids)
+        if stop <= n:
+            return self.prompt_token_ids[start:stop]
+        if start >= n:
+            return self.output_token_ids[start - n : stop - n]
+        return self.prompt_token_ids[start:] + self.output_token_ids[: stop - n]

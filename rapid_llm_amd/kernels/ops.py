@@ -282,6 +282,45 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _ok(core().rl_argmax(_p(logits), _p(out), rows, vocab, _stream()), "rl_argmax")
 
 
+def sample(
+    logits: torch.Tensor,
+    row_params: torch.Tensor,
+    history: Optional[torch.Tensor],
+    out: torch.Tensor,
+    out_logprob: Optional[torch.Tensor],
+    any_penalty: bool,
+) -> None:
+    """General token selection (penalty, temperature, nucleus, seeded draw), one row per
+    workgroup.  ``row_params [rows * 8]`` int32 as the kernel documents them."""
+    rows, vocab = logits.shape
+    _need(logits, "logits", torch.float32)
+    _need(row_params, "row_params", torch.int32, (rows * 8,))
+    _need(out, "out", torch.int32, (rows,))
+    if out_logprob is not None:
+        _need(out_logprob, "out_logprob", torch.float32, (rows,))
+    if history is not None:
+        _need(history, "history", torch.int32)
+    if any_penalty and vocab > 40 * 1024 * 8:
+        raise KernelError(
+            f"the repetition penalty keeps one bit per token id in 40 KB of LDS: vocabulary "
+            f"{vocab} is beyond {40 * 1024 * 8}"
+        )
+    _ok(
+        core().rl_sample(
+            _p(logits), _p(row_params), _p(history), _p(out), _p(out_logprob), rows, vocab,
+            int(bool(any_penalty)), _stream(),
+        ),
+        "rl_sample",
+    )
+
+
+def sample_uniform(seed: int, counter: int) -> float:
+    """The kernel's own uniform draw, computed by the library on the host."""
+    fn = core().rl_sample_uniform
+    fn.restype = ctypes.c_float
+    return float(fn(ctypes.c_uint(seed & 0xFFFFFFFF), ctypes.c_uint((seed >> 32) & 0xFFFFFFFF), ctypes.c_uint(counter)))
+
+
 SKINNY_MAX_ROWS = 64  # rows up to which the bandwidth-bound product is used
 SWIGLU_MAX_ROWS = 32
 _MIN_BLOCKS = 512  # workgroups a skinny product should reach before it widens its tiles

@@ -1,0 +1,160 @@
+"""Generation through the entry point: ``LLM.generate`` drives scheduler, step function, cache
+and sampling kernels; the plain implementation re-runs the whole sequence for every token."""
+
+import pytest
+import torch
+
+from plain_model import plain_forward, plain_load
+from plain_sampler import plain_sample
+from rapid_llm_amd.sampling.rng import uniform_draw
+from tiny_configs import TINY, make_model_dir, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+
+def _llm(model_dir, dtype, page, **kw):
+    from rapid_llm_amd import LLM
+
+    body = dict(dtype=dtype, page_size=page, num_pages=200, max_num_seqs=8, use_cuda_graph=False)
+    body.update(kw)
+    return LLM(str(model_dir), **body)
+
+
+def _plain_generate(cfg, w, prompt, n, temperature=0.0, top_p=1.0, seed=0, penalty=1.0):
+    ids, out = list(prompt), []
+    for i in range(n):
+        logits = plain_forward(cfg, w, ids)[-1]
+        tok = plain_sample(logits, temperature, top_p, uniform_draw(seed, i), penalty, out)
+        out.append(tok)
+        ids.append(tok)
+    return out
+
+
+def test_greedy_generation_tiny_a_float32(tmp_path):
+    """BASELINE configuration A: prompts of 1/5/13/29 tokens, 12 greedy tokens each."""
+    from rapid_llm_amd import SamplingParams
+
+    cfg, page, seed = TINY["A"]
+    model_dir = make_model_dir(tmp_path, "A", "float32")
+    pcfg, pw = plain_load(model_dir)
+    prompts = [random_tokens(n, cfg["vocab_size"], seed + n) for n in (1, 5, 13, 29)]
+    llm = _llm(model_dir, "float32", page, max_seq_len=128)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_gen_len=12))
+    for prompt, out in zip(prompts, outs):
+        assert out.outputs[0].token_ids == _plain_generate(pcfg, pw, prompt, 12)
+        assert out.outputs[0].finish_reason == "length" and out.prompt_token_ids == prompt
+    # batched == one by one, and run-to-run equal (tests/engine/test_engine_e2e.py:27-83)
+    for prompt, out in zip(prompts, outs):
+        alone = llm.generate(prompt, SamplingParams(temperature=0.0, max_gen_len=12))
+        assert alone[0].token_ids == out.token_ids
+    llm.scheduler.cache.check_invariants()
+    assert not llm.scheduler.cache.live_requests()
+
+
+def test_sampled_generation_tiny_b_chunked_and_mixed(tmp_path):
+    """BASELINE configuration B: prompts of 2/17/31/64/90/150 tokens in portions of 24 mixed
+    with decodes, then 20 tokens each at temperature 0.8 with a fixed seed."""
+    from rapid_llm_amd import SamplingParams
+
+    cfg, page, seed = TINY["B"]
+    model_dir = make_model_dir(tmp_path, "B", "float32")
+    pcfg, pw = plain_load(model_dir)
+    prompts = [random_tokens(n, cfg["vocab_size"], seed + n) for n in (2, 17, 31, 64, 90, 150)]
+    llm = _llm(model_dir, "float32", page, max_seq_len=256, max_chunk_size=24, max_num_batched_tokens=64,
+               max_num_seqs=4)
+    params = [SamplingParams(temperature=0.8, top_p=0.9, max_gen_len=20, seed=77 + i, logprobs=0)
+              for i in range(len(prompts))]
+    outs = llm.generate(prompts, params)
+    mixed_steps = 0
+    for i, (prompt, out) in enumerate(zip(prompts, outs)):
+        want = _plain_generate(pcfg, pw, prompt, 20, 0.8, 0.9, 77 + i)
+        assert out.token_ids == want, i
+        assert len(out.outputs[0].logprobs) == 20 and all(lp <= 0 for lp in out.outputs[0].logprobs)
+    # the same requests, unchunked and one at a time, draw the same tokens
+    solo = _llm(model_dir, "float32", page, max_seq_len=256, max_chunk_size=0, max_num_batched_tokens=256,
+                max_num_seqs=1)
+    for prompt, p, out in zip(prompts, params, outs):
+        assert solo.generate(prompt, p)[0].token_ids == out.token_ids
+
+
+def test_eviction_changes_nothing(tmp_path):
+    """So few pages that running requests are evicted and recomputed: the tokens are the ones
+    an ample pool gives, greedy and sampled."""
+    from rapid_llm_amd import SamplingParams
+
+    cfg, page, seed = TINY["A"]
+    model_dir = make_model_dir(tmp_path, "A", "float32")
+    prompts = [random_tokens(n, cfg["vocab_size"], seed + n) for n in (9, 14, 6, 11)]
+    params = [SamplingParams(temperature=0.0 if i % 2 else 0.7, top_p=0.95, max_gen_len=30, seed=i,
+                             repetition_penalty=1.15) for i in range(4)]
+    ample = _llm(model_dir, "float32", page, max_seq_len=128).generate(prompts, params)
+    tight = _llm(model_dir, "float32", page, max_seq_len=128, num_pages=24)  # 23 pages of 4: ~2 requests
+    outs = tight.generate(prompts, params)
+    assert tight.scheduler.num_preemptions > 0
+    assert [o.token_ids for o in outs] == [o.token_ids for o in ample]
+    tight.scheduler.cache.check_invariants()
+    assert tight.scheduler.cache.num_free_pages() == 23
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_bfloat16_generation_stays_near_the_plain_choice(tmp_path, which):
+    from rapid_llm_amd import SamplingParams
+
+    cfg, page, seed = TINY[which]
+    model_dir = make_model_dir(tmp_path, which, "bfloat16")
+    pcfg, pw = plain_load(model_dir)
+    prompts = [random_tokens(n, cfg["vocab_size"], seed + n) for n in (3, 20, 45)]
+    for graph in (False, True):
+        llm = _llm(model_dir, "bfloat16", page, max_seq_len=cfg["max_position_embeddings"], use_cuda_graph=graph)
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_gen_len=16))
+        for prompt, out in zip(prompts, outs):
+            ids = list(prompt)
+            for tok in out.token_ids:
+                logits = plain_forward(pcfg, pw, ids)[-1]
+                # bfloat16 may pick another of several nearly equal maxima, never a poor token
+                assert float(logits.max() - logits[tok]) < 0.05, (which, graph)
+                ids.append(tok)
+            assert len(out.token_ids) == 16
+
+
+def test_stop_tokens_and_stream(tmp_path):
+    from rapid_llm_amd import LLM, SamplingParams
+
+    cfg, page, seed = TINY["A"]
+    model_dir = make_model_dir(tmp_path, "A", "float32")
+    prompt = random_tokens(7, cfg["vocab_size"], 5)
+    free = _llm(model_dir, "float32", page, max_seq_len=64).generate(prompt, SamplingParams(temperature=0.0, max_gen_len=10))[0]
+    stop = free.token_ids[4]
+    (model_dir / "generation_config.json").write_text('{"eos_token_id": [%d]}' % stop)
+    llm = _llm(model_dir, "float32", page, max_seq_len=64)
+    out = llm.generate(prompt, SamplingParams(temperature=0.0, max_gen_len=10))[0]
+    first = free.token_ids.index(stop)
+    assert out.token_ids == free.token_ids[:first] and out.outputs[0].finish_reason == "eos"
+    seen = []
+    for batch in llm.stream([prompt, prompt[:3]], SamplingParams(temperature=0.0, max_gen_len=5, ignore_eos=True)):
+        seen.append([len(o.token_ids) for o in batch])
+    assert seen[-1] == [5, 5] or seen[-1] == [5]
+    assert sum(1 for s in seen) >= 5
+
+
+def test_command_line_batch(tmp_path, capsys):
+    from rapid_llm_amd.cli import main
+
+    cfg, page, seed = TINY["B"]
+    model_dir = make_model_dir(tmp_path, "B", "float32")
+    prompts = tmp_path / "prompts.txt"
+    prompts.write_text("[1, 2, 3, 4]\n\n[10, 20]\n")
+    code = main(["batch", "--model-dir", str(model_dir), "--dtype", "float32", "--max-seq-len", "64",
+                 "--temperature", "0", "--max-gen-len", "6", "--repetition-penalty", "1.0",
+                 "--prompts-file", str(prompts), "--show-stats", "--no-cuda-graph"])
+    text = capsys.readouterr().out
+    assert code == 0 and "--- [0] length ---" in text and "--- [1] length ---" in text
+    assert "2 requests, 12 tokens" in text and "throughput" in text
+    pcfg, pw = plain_load(model_dir)
+    assert str(_plain_generate(pcfg, pw, [1, 2, 3, 4], 6)) in text
+
+
+def test_smoke_entry():
+    import __graft_entry__
+
+    __graft_entry__.smoke()

@@ -1,0 +1,321 @@
+"""Each part the model is put together from, alone against its plain formula; and the seams:
+a toy mixer with state of its own and a toy architecture, registered, built and stepped
+without a change to the framework; a run order that names a layer twice; a layer that reads
+another layer's cache."""
+
+import json
+import math
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+from plain_model import (
+    plain_attention,
+    plain_load,
+    plain_rmsnorm,
+    plain_rope_apply,
+    plain_rope_tables,
+    plain_swiglu_mlp,
+)
+from tiny_configs import TINY, make_model_dir, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": dict(rtol=2e-5, atol=2e-6), "bfloat16": dict(rtol=3e-2, atol=2e-2)}
+
+
+def _runner(model_dir, dtype, page, **kw):
+    from rapid_llm_amd import EngineConfig, ModelRunner
+
+    body = dict(dtype=dtype, max_seq_len=128, page_size=page, num_pages=64, max_num_seqs=4, use_graph=False)
+    body.update(kw)
+    return ModelRunner(model_dir, EngineConfig(**body))
+
+
+def _context(runner, entries):
+    host, offs, meta = runner._prepare(entries)
+    dev = torch.from_numpy(host).to(runner.device)
+    return runner._context(dev, offs, meta)
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_parts_alone(tmp_path, which, dtype):
+    from rapid_llm_amd import StepEntry
+
+    cfg, page, seed = TINY[which]
+    model_dir = make_model_dir(tmp_path, which, dtype)
+    _, w = plain_load(model_dir)
+    runner = _runner(model_dir, dtype, page)
+    tdt = runner.dtype
+    tol = TOL[dtype]
+    H, nq, nkv, d = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    eps = cfg["rms_norm_eps"]
+    # two requests in one batch: 11 and 6 tokens
+    lens = (11, 6)
+    entries = [StepEntry(f"p{i}", random_tokens(n, cfg["vocab_size"], seed + i), [n - 1]) for i, n in enumerate(lens)]
+    ctx = _context(runner, entries)
+    T = sum(lens)
+    gen = torch.Generator().manual_seed(seed)
+    model = runner.model
+
+    # ---- embedding: a row gather into the float32 stream --------------------------------
+    emb = model.embed.forward(ctx.token_ids).cpu()
+    ids = [t for e in entries for t in e.tokens]
+    assert emb.dtype == torch.float32
+    torch.testing.assert_close(emb, w["model.embed_tokens.weight"][torch.tensor(ids)], rtol=0, atol=0)
+
+    # ---- norm with the residual add in front of it, whole and on chosen rows -----------------
+    block = model.blocks[1]
+    residual = torch.randn(T, H, generator=gen)
+    delta = torch.randn(T, H, generator=gen).to(tdt)
+    res_dev = residual.cuda()
+    out = block.mixer_norm.forward(res_dev, delta.cuda(), ctx).cpu().float()
+    summed = residual + delta.float()
+    torch.testing.assert_close(res_dev.cpu(), summed, rtol=0, atol=0)  # written in place, in float32
+    torch.testing.assert_close(out, plain_rmsnorm(summed, w["model.layers.1.input_layernorm.weight"], eps), **tol)
+    rows = torch.tensor([T - 1, 2], dtype=torch.int32).cuda()
+    picked = model.final_norm.forward(res_dev, None, ctx, rows=rows).cpu().float()
+    torch.testing.assert_close(picked, plain_rmsnorm(summed[[T - 1, 2]], w["model.norm.weight"], eps), **tol)
+
+    # ---- feed-forward ----------------------------------------------------------------------
+    x = (torch.randn(T, H, generator=gen) * 0.5).to(tdt)
+    p = "model.layers.1.mlp."
+    got = block.feed_forward.forward(x.cuda(), ctx).cpu().float()
+    want = plain_swiglu_mlp(x.float(), w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+    torch.testing.assert_close(got, want, **tol)
+
+    # ---- position tables ---------------------------------------------------------------------
+    cos, sin = plain_rope_tables(torch.arange(128), d, cfg["rope_theta"])
+    rope = block.mixer.position
+    torch.testing.assert_close(rope.cos.cpu(), cos, rtol=0, atol=1e-6)
+    torch.testing.assert_close(rope.sin.cpu(), sin, rtol=0, atol=1e-6)
+
+    # ---- the mixer: projection, head norms, rotation, cache write, attention, projection ----
+    a = "model.layers.1.self_attn."
+    got = block.mixer.forward(x.cuda(), ctx, runner.device_cache.layers[1]).cpu().float()
+    window = cfg.get("sliding_window") if cfg.get("layer_types", ["full_attention"] * 3)[1] == "sliding_attention" else None
+    want, at = [], 0
+    for n in lens:
+        xs = x[at : at + n].float()
+        q = plain_rmsnorm((xs @ w[a + "q_proj.weight"].T).view(n, nq, d), w[a + "q_norm.weight"], eps)
+        k = plain_rmsnorm((xs @ w[a + "k_proj.weight"].T).view(n, nkv, d), w[a + "k_norm.weight"], eps)
+        v = (xs @ w[a + "v_proj.weight"].T).view(n, nkv, d)
+        c, s = plain_rope_tables(torch.arange(n), d, cfg["rope_theta"])
+        o = plain_attention(plain_rope_apply(q, c, s), plain_rope_apply(k, c, s), v, 1 / math.sqrt(d), window)
+        want.append(o.reshape(n, nq * d) @ w[a + "o_proj.weight"].T)
+        at += n
+    torch.testing.assert_close(got, torch.cat(want), **tol)
+
+    # ---- output projection -------------------------------------------------------------------
+    h = torch.randn(3, H, generator=gen).to(tdt)
+    logits = model.output.forward(h.cuda()).cpu()
+    head = w.get("lm_head.weight", w["model.embed_tokens.weight"])
+    assert logits.dtype == torch.float32
+    torch.testing.assert_close(logits, h.float() @ head.T, **tol)
+
+
+# --------------------------------------------------------------------------- #
+# a toy architecture defined here: a mixer with state of its own in layer 0, attention in
+# layer 1, and a run order that visits layer 1 twice
+# --------------------------------------------------------------------------- #
+@dataclass(frozen=True)
+class ToyConfig:
+    hidden: int
+    vocab: int
+    heads: int
+    head_dim: int
+    inter: int
+    decay: float
+    twice: bool = False
+    share: bool = False
+
+    @classmethod
+    def from_dict(cls, data, overrides=None):
+        return cls(data["hidden"], data["vocab"], data["heads"], data["head_dim"], data["inter"],
+                   data["decay"], data.get("twice", False), data.get("share", False))
+
+    def to_dict(self):
+        return dict(architectures=["ToyForCausalLM"], hidden=self.hidden, vocab=self.vocab, heads=self.heads,
+                    head_dim=self.head_dim, inter=self.inter, decay=self.decay, twice=self.twice,
+                    share=self.share, torch_dtype="float32")
+
+
+def _toy_parts():
+    from rapid_llm_amd.parts import MIXERS, CacheNeed, Mixer, ParamSpec, Source
+    from rapid_llm_amd.parts.linear import Linear
+
+    class DecayingSum(Mixer):
+        """``s_t = decay * s_{t-1} + x_t`` per request, output ``W s_t``: no pages, one vector of
+        state per request, carried from step to step in the request's slot."""
+
+        def __init__(self, hidden_size, decay, checkpoint_prefix, position=None, name="mixer"):
+            self.h, self.decay, self.prefix, self.name = hidden_size, decay, checkpoint_prefix, name
+            self.proj = Linear(hidden_size, hidden_size)
+
+        def param_specs(self):
+            return [ParamSpec(self.name + ".w", (self.h, self.h), "matrix", (Source(self.prefix + "w", self.h),))]
+
+        def bind(self, params, runtime):
+            self.proj.bind(params[self.name + ".w"])
+
+        def cache_need(self):
+            return CacheNeed("state", state_shape=(self.h,), state_dtype="float32")
+
+        def forward(self, x, ctx, cache):
+            out = torch.empty_like(x, dtype=torch.float32)
+            at = 0
+            for slot, n in zip(ctx.h_seq_slots, ctx.h_seq_lens):
+                s = cache.state[slot]
+                for t in range(at, at + n):
+                    s = self.decay * s + x[t].float()
+                    out[t] = s
+                cache.state[slot] = s
+                at += n
+            return self.proj(out.to(x.dtype))
+
+    MIXERS.register("toy_decaying_sum", DecayingSum, replace=True)
+
+
+def _toy_spec(cfg: ToyConfig):
+    from rapid_llm_amd.models import LayerSpec, ModelSpec, PartSpec
+
+    def norm(name):
+        return PartSpec("rmsnorm", {"size": cfg.hidden, "eps": 1e-5, "checkpoint_name": name})
+
+    def ff(i):
+        return PartSpec("swiglu", {"hidden_size": cfg.hidden, "intermediate_size": cfg.inter,
+                                   "checkpoint_prefix": f"l{i}.ff."})
+
+    rope = PartSpec("rope_half_split", {"head_dim": cfg.head_dim, "theta": 100.0})
+
+    def attn(i):
+        return PartSpec("gqa_attention", {"hidden_size": cfg.hidden, "num_heads": cfg.heads, "num_kv_heads": 1,
+                                          "head_dim": cfg.head_dim, "checkpoint_prefix": f"l{i}.attn."})
+
+    layers = [
+        LayerSpec(PartSpec("toy_decaying_sum", {"hidden_size": cfg.hidden, "decay": cfg.decay,
+                                                "checkpoint_prefix": "l0.mix."}), ff(0), norm("l0.n1"), norm("l0.n2")),
+        LayerSpec(attn(1), ff(1), norm("l1.n1"), norm("l1.n2"), position=rope),
+    ]
+    if cfg.share:
+        layers.append(LayerSpec(attn(2), ff(2), norm("l2.n1"), norm("l2.n2"), position=rope, share_cache_with=1))
+    order = (0, 1, 0, 1) if cfg.twice else None
+    return ModelSpec(cfg.hidden, cfg.vocab, tuple(layers), norm("final"), "embed", "head", False, run_order=order)
+
+
+def _toy_plain(w, cfg: ToyConfig, toks):
+    """The toy model, whole sequence, in plain torch."""
+    t = len(toks)
+    h = w["embed"][torch.tensor(toks)]
+    pos = torch.arange(t)
+
+    def ffn(i, h):
+        x = plain_rmsnorm(h, w[f"l{i}.n2"], 1e-5)
+        return h + plain_swiglu_mlp(x, w[f"l{i}.ff.gate_proj.weight"], w[f"l{i}.ff.up_proj.weight"],
+                                    w[f"l{i}.ff.down_proj.weight"])
+
+    def toy(h):
+        x = plain_rmsnorm(h, w["l0.n1"], 1e-5)
+        s, rows = torch.zeros(cfg.hidden), []
+        for j in range(t):
+            s = cfg.decay * s + x[j]
+            rows.append(s)
+        return ffn(0, h + torch.stack(rows) @ w["l0.mix.w"].T)
+
+    def kv_of(i, h):
+        x = plain_rmsnorm(h, w[f"l{i}.n1"], 1e-5)
+        c, s = plain_rope_tables(pos, cfg.head_dim, 100.0)
+        k = plain_rope_apply((x @ w[f"l{i}.attn.k_proj.weight"].T).view(t, 1, cfg.head_dim), c, s)
+        return k, (x @ w[f"l{i}.attn.v_proj.weight"].T).view(t, 1, cfg.head_dim)
+
+    def attn(i, h, kv=None):
+        x = plain_rmsnorm(h, w[f"l{i}.n1"], 1e-5)
+        c, s = plain_rope_tables(pos, cfg.head_dim, 100.0)
+        q = plain_rope_apply((x @ w[f"l{i}.attn.q_proj.weight"].T).view(t, cfg.heads, cfg.head_dim), c, s)
+        k, v = kv if kv is not None else kv_of(i, h)
+        o = plain_attention(q, k, v, cfg.head_dim**-0.5).reshape(t, -1)
+        return ffn(i, h + o @ w[f"l{i}.attn.o_proj.weight"].T)
+
+    if cfg.twice:
+        h = attn(1, toy(h))
+        # the second visit of layer 0 starts from fresh state: each place in the order has its own
+        h = attn(1, toy(h))
+    else:
+        h = toy(h)
+        kv = kv_of(1, h)
+        h = attn(1, h)
+        if cfg.share:
+            h = attn(2, h, kv)  # reads the keys and values layer 1 wrote
+    return plain_rmsnorm(h, w["final"], 1e-5) @ w["head"].T
+
+
+@pytest.mark.parametrize("variant", ["plain", "twice", "share"])
+def test_toy_architecture_registers_builds_and_steps(tmp_path, variant):
+    from safetensors.torch import load_file
+
+    from rapid_llm_amd import StepEntry, write_random_model
+    from rapid_llm_amd.config import register_architecture, unregister_architecture
+    from rapid_llm_amd.parts import MIXERS
+
+    _toy_parts()
+    register_architecture("ToyForCausalLM", ToyConfig, _toy_spec, replace=True)
+    try:
+        cfg = ToyConfig(hidden=48, vocab=97, heads=3, head_dim=16, inter=80, decay=0.8,
+                        twice=variant == "twice", share=variant == "share")
+        folder = write_random_model(cfg.to_dict(), 3, tmp_path / "toy", dtype="float32")
+        weights = load_file(str(folder / "model.safetensors"))
+        if variant == "share":  # the sharing layer's own k/v projections exist but are never used
+            assert "l2.attn.k_proj.weight" in weights
+        runner = _runner(folder, "float32", 8)
+        needs = runner.model.cache_needs()
+        assert needs[0].kind == "state" and needs[1].kind == "kv"
+        if variant == "share":
+            assert needs[2].share_with == 1 and not runner.device_cache.layers[2].owns_pages
+            assert runner.device_cache.layers[2].k is runner.device_cache.layers[1].k
+        if variant == "twice":
+            assert len(runner.device_cache.layers) == 4
+            assert runner.device_cache.layers[0].state is not runner.device_cache.layers[2].state
+        reqs = {f"t{i}": random_tokens(n, cfg.vocab, 40 + i) for i, n in enumerate((19, 33, 7))}
+        want = {rid: _toy_plain(weights, cfg, toks) for rid, toks in reqs.items()}
+        # whole, then cut: portions and single tokens of the three requests interleaved
+        for cut in ("whole", "cut"):
+            got = {rid: [] for rid in reqs}
+            if cut == "whole":
+                for rid, toks in reqs.items():
+                    got[rid].append(runner.step([StepEntry(rid, toks, list(range(len(toks))))]).cpu())
+            else:
+                done = {rid: 0 for rid in reqs}
+                sizes = [5, 1, 2, 9, 1, 3]
+                k = 0
+                while any(done[r] < len(reqs[r]) for r in reqs):
+                    entries = []
+                    for rid, toks in reqs.items():
+                        if done[rid] >= len(toks):
+                            continue
+                        n = min(sizes[k % len(sizes)], len(toks) - done[rid])
+                        k += 1
+                        entries.append(StepEntry(rid, toks[done[rid] : done[rid] + n], list(range(n))))
+                        done[rid] += n
+                    logits = runner.step(entries).cpu()
+                    at = 0
+                    for e in entries:
+                        got[e.request_id].append(logits[at : at + len(e.tokens)])
+                        at += len(e.tokens)
+            for rid in reqs:
+                torch.testing.assert_close(torch.cat(got[rid]), want[rid], rtol=2e-5, atol=3e-6)
+                runner.finish(rid)  # the slot's state is cleared for whoever takes it next
+        runner.cache.check_invariants()
+    finally:
+        unregister_architecture("ToyForCausalLM")
+        MIXERS.unregister("toy_decaying_sum")
+
+
+def test_unknown_part_kinds_are_named():
+    from rapid_llm_amd.models import CausalLM, LayerSpec, ModelSpec, PartSpec
+
+    norm = PartSpec("rmsnorm", {"size": 8, "eps": 1e-5, "checkpoint_name": "n"})
+    bad = ModelSpec(8, 10, (LayerSpec(PartSpec("no_such_mixer"), PartSpec("swiglu"), norm, norm),), norm, "e", "o", False)
+    with pytest.raises(ValueError, match="unknown mixer kind 'no_such_mixer'; known: .*gqa_attention"):
+        CausalLM(bad)

@@ -1,0 +1,135 @@
+"""The sampling kernels against the plain sampler: arg-max, temperature, nucleus with its
+pool of 1024, repetition penalty, seeded draws; at vocabularies from 3 to 151,936."""
+
+import pytest
+import torch
+
+from plain_sampler import plain_logprob, plain_sample
+from rapid_llm_amd.sampling.rng import uniform_draw
+
+pytestmark = pytest.mark.gpu
+
+
+def _sampler():
+    from rapid_llm_amd.sampling.sampler import RowSampling, Sampler
+
+    return Sampler("cuda"), RowSampling
+
+
+def _acceptable(logits, row, u):
+    """Tokens the plain sampler picks for draws within rounding of ``u``: the kernel sums
+    its probabilities in float32 in another order."""
+    return {
+        plain_sample(logits, row.temperature, row.top_p, min(max(u + d, 0.0), 0.9999999),
+                     row.repetition_penalty, list(row.generated))
+        for d in (0.0, -3e-6, 3e-6)
+    }
+
+
+def test_uniform_draw_matches_the_kernel():
+    from rapid_llm_amd.kernels import ops
+
+    for seed, counter in [(0, 0), (1, 0), (0, 1), (2**63 + 12345, 99), (2**64 - 1, 2**32 - 1)]:
+        assert ops.sample_uniform(seed, counter) == uniform_draw(seed, counter)
+    draws = [uniform_draw(42, i) for i in range(4000)]
+    assert 0.0 <= min(draws) and max(draws) < 1.0 and abs(sum(draws) / 4000 - 0.5) < 0.02
+
+
+@pytest.mark.parametrize("vocab", [3, 64, 503, 1024, 1025, 4099, 151936])
+def test_rows_of_every_kind_match_the_plain_sampler(vocab):
+    sampler, Row = _sampler()
+    gen = torch.Generator().manual_seed(vocab)
+    rows, logit_rows = [], []
+    kinds = [
+        dict(temperature=0.0, top_p=1.0),
+        dict(temperature=0.0, top_p=0.9, repetition_penalty=1.3),
+        dict(temperature=0.8, top_p=1.0),
+        dict(temperature=0.8, top_p=0.9),
+        dict(temperature=1.5, top_p=0.5, repetition_penalty=1.2),
+        dict(temperature=0.3, top_p=0.1),
+        dict(temperature=2.5, top_p=0.999),
+        dict(temperature=1.0, top_p=0.95, repetition_penalty=0.8),
+    ]
+    for i in range(24):
+        kind = kinds[i % len(kinds)]
+        scale = (1.0, 4.0, 0.2)[i % 3]
+        logit_rows.append(torch.randn(vocab, generator=gen) * scale)
+        generated = torch.randint(0, vocab, (17,), generator=gen).tolist() + [int(logit_rows[-1].argmax())]
+        rows.append(Row(seed=1000 + i, counter=i * 7, generated=generated, **kind))
+    logits = torch.stack(logit_rows).cuda()
+    ids, logprobs = sampler.sample(logits, rows, want_logprobs=True)
+    ids, logprobs = ids.tolist(), logprobs.tolist()
+    for i, row in enumerate(rows):
+        u = uniform_draw(row.seed, row.counter)
+        assert ids[i] in _acceptable(logit_rows[i], row, u), (vocab, i, row)
+        want = plain_logprob(logit_rows[i], ids[i], row.temperature, row.repetition_penalty, list(row.generated))
+        assert abs(logprobs[i] - want) < 2e-4 * max(1.0, abs(want)), (vocab, i)
+
+
+def test_greedy_batch_takes_the_argmax_kernel_and_lowest_index_wins():
+    sampler, Row = _sampler()
+    logits = torch.randn(9, 7001)
+    logits[3, 100] = logits[3, 4000] = 50.0  # equal maxima: the lower index
+    logits[5, :] = 1.25
+    ids, lp = sampler.sample(logits.cuda(), [Row() for _ in range(9)])
+    assert lp is None
+    want = logits.argmax(-1).tolist()
+    want[3], want[5] = 100, 0
+    assert ids.tolist() == want
+    # the general kernel's greedy rows agree
+    ids2, _ = sampler.sample(logits.cuda(), [Row() for _ in range(9)], want_logprobs=True)
+    assert ids2.tolist() == want
+
+
+def test_reference_vectors():
+    sampler, Row = _sampler()
+    # rapid_llm tests/engine/test_sampler.py:61-63
+    ids, _ = sampler.sample(torch.tensor([[0.1, 0.9, 0.0], [0.5, 0.1, 0.4]]).cuda(), [Row(), Row()])
+    assert ids.tolist() == [1, 0]
+    # :66-72 a nucleus of 0.1 keeps only the dominant token, whatever the draw
+    logits = torch.log(torch.tensor([[0.7, 0.2, 0.1]])).cuda().repeat(64, 1)
+    ids, _ = sampler.sample(logits, [Row(temperature=1.0, top_p=0.1, seed=5, counter=c) for c in range(64)])
+    assert set(ids.tolist()) == {0}
+    # :229-266 the penalty divides positive and multiplies negative logits, once per token
+    logits = torch.tensor([[4.0, -4.0, 3.9], [4.0, 3.0, -9.0]]).cuda()
+    ids, _ = sampler.sample(logits, [Row(repetition_penalty=2.0, generated=[0, 0, 1]),
+                                     Row(repetition_penalty=1.2, generated=[0, 0, 0, 0])])
+    assert ids.tolist() == [2, 0]  # row 0: 4/2 < 3.9; row 1: 4/1.2 = 3.33 > 3 (applied once, not four times)
+
+
+def test_draws_follow_the_distribution_and_the_seed():
+    sampler, Row = _sampler()
+    probs = torch.tensor([0.05, 0.5, 0.25, 0.2])
+    n = 4096
+    logits = torch.log(probs)[None].repeat(n, 1).cuda()
+    for top_p, want in ((1.0, probs), (0.8, torch.tensor([0.0, 0.5, 0.25, 0.2]) / 0.95)):
+        ids, _ = sampler.sample(logits, [Row(temperature=1.0, top_p=top_p, seed=9, counter=c) for c in range(n)])
+        freq = torch.bincount(ids.cpu().long(), minlength=4).float() / n
+        assert float((freq - want).abs().max()) < 0.03, (top_p, freq)
+        again, _ = sampler.sample(logits, [Row(temperature=1.0, top_p=top_p, seed=9, counter=c) for c in range(n)])
+        assert torch.equal(ids, again)
+        other, _ = sampler.sample(logits, [Row(temperature=1.0, top_p=top_p, seed=10, counter=c) for c in range(n)])
+        assert not torch.equal(ids, other)
+
+
+def test_pool_never_leaks_and_flat_rows_keep_the_whole_pool():
+    sampler, Row = _sampler()
+    vocab = 5000
+    flat = torch.zeros(256, vocab).cuda()  # more equal logits than the pool has places
+    ids, _ = sampler.sample(flat, [Row(temperature=1.0, top_p=0.999, seed=3, counter=c) for c in range(256)])
+    assert max(ids.tolist()) < 1024 and len(set(ids.tolist())) > 100  # the lowest indices fill the pool
+    gen = torch.Generator().manual_seed(0)
+    logits = torch.randn(64, vocab, generator=gen) * 0.01  # nearly flat: the pool never reaches top_p
+    pool = [set(r.topk(1024).indices.tolist()) for r in logits]
+    ids, _ = sampler.sample(logits.cuda(), [Row(temperature=1.0, top_p=0.9, seed=4, counter=c) for c in range(64)])
+    assert all(t in pool[i] for i, t in enumerate(ids.tolist()))
+
+
+def test_penalty_needs_a_vocabulary_the_bitmap_holds():
+    from rapid_llm_amd.kernels.ops import KernelError
+
+    sampler, Row = _sampler()
+    logits = torch.zeros(1, 400_000).cuda()
+    sampler.sample(logits, [Row(temperature=1.0, top_p=0.9)])  # no penalty: fine
+    with pytest.raises(KernelError, match="beyond"):
+        sampler.sample(logits, [Row(temperature=1.0, repetition_penalty=1.1, generated=[1])])

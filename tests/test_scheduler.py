@@ -1,0 +1,299 @@
+"""The scheduler's decisions, with a scripted step function in place of the model (CPU only).
+
+The pattern is the reference's ``_ScriptedExecutor`` (tests/engine/test_scheduler.py:46-74,
+tests/engine/test_batch_planner.py:156-610)."""
+
+import pytest
+
+from rapid_llm_amd.cache import CacheManager, GroupSpec
+from rapid_llm_amd.config import EngineConfig
+from rapid_llm_amd.engine.request import RequestStatus
+from rapid_llm_amd.engine.scheduler import Scheduler, detect_repetition
+from rapid_llm_amd.sampling import SamplingParams
+
+EOS = 99
+
+
+class ScriptedExecutor:
+    """Checks that every step is runnable from what the plan reserved, records its shape,
+    and "samples" token ``f(request, index of the output token)``."""
+
+    def __init__(self, num_pages, page, seqs, max_len, window=0, token=None):
+        self.cache = CacheManager([GroupSpec(0, window, (0,))], num_pages, page, seqs, max_len)
+        self.token = token or (lambda rid, i: 1000 + i)
+        self.steps = []
+        self.computed = {}
+        self.fed = {}
+
+    def execute(self, entries, rows, want_logprobs=False):
+        shape, out = [], []
+        k = 0
+        for e in entries:
+            assert self.cache.has(e.request_id), "an entry without a slot"
+            start = self.computed.get(e.request_id, 0)
+            assert self.cache.reserved(e.request_id) >= start + len(e.tokens), "pages were not reserved"
+            self.computed[e.request_id] = start + len(e.tokens)
+            self.fed.setdefault(e.request_id, []).extend(e.tokens)
+            shape.append((e.request_id, len(e.tokens), bool(e.want)))
+            if e.want:
+                assert list(e.want) == [len(e.tokens) - 1]
+                out.append(self.token(e.request_id, rows[k].counter))
+                k += 1
+        assert k == len(rows)
+        self.steps.append(shape)
+        self.cache.check_invariants()
+        return out, ([-1.0] * len(out) if want_logprobs else None)
+
+    def finish(self, request_id):
+        self.cache.release(request_id)
+        self.computed.pop(request_id, None)
+        self.fed.pop(request_id, None)
+
+
+def _make(num_pages=64, page=4, seqs=4, max_len=128, token=None, **cfg):
+    ex = ScriptedExecutor(num_pages, page, seqs, max_len, token=token)
+    config = EngineConfig(max_seq_len=max_len, page_size=page, num_pages=num_pages, max_num_seqs=seqs,
+                          **{"max_num_batched_tokens": 64, "max_chunk_size": 16, **cfg})
+    return Scheduler(ex, config, stop_token_ids=[EOS]), ex
+
+
+GREEDY = SamplingParams(temperature=0.0, max_gen_len=4)
+
+
+def test_submission_rules():
+    s, _ = _make(max_len=32)
+    with pytest.raises(ValueError, match="empty"):
+        s.add_request([], GREEDY)
+    with pytest.raises(ValueError, match="no room"):
+        s.add_request(list(range(32)), GREEDY)
+    with pytest.raises(ValueError, match="tokenizer"):
+        s.add_request("text", GREEDY)
+    r = s.add_request(list(range(30)), SamplingParams(temperature=0.0, max_gen_len=10))
+    assert r.max_new_tokens == 2  # capped by the context (batch_planner.py:403-427)
+    assert s.add_request([1], SamplingParams(temperature=0.0)).max_new_tokens == 31
+    s.add_request([1], GREEDY, request_id="mine")
+    with pytest.raises(ValueError, match="already in use"):
+        s.add_request([1], GREEDY, request_id="mine")
+    tiny, _ = _make(num_pages=3, page=4, max_len=128)
+    with pytest.raises(ValueError, match="does not fit the cache pool"):
+        tiny.add_request(list(range(8)), GREEDY)
+
+
+def test_prompt_is_cut_into_portions_and_sampled_with_the_last():
+    s, ex = _make()
+    r = s.add_request(list(range(37)), GREEDY)
+    s.run_to_completion()
+    # 16 + 16 + 5 (sampled), then three decode steps; the 4th token is never fed
+    assert ex.steps == [[("req-0", 16, False)], [("req-0", 16, False)], [("req-0", 5, True)],
+                        [("req-0", 1, True)], [("req-0", 1, True)], [("req-0", 1, True)]]
+    assert r.output_token_ids == [1000, 1001, 1002, 1003] and r.finish_reason == "length"
+    assert r.status is RequestStatus.FINISHED and not ex.cache.live_requests()
+
+
+def test_decodes_run_beside_portions_under_one_budget():
+    s, ex = _make(max_num_batched_tokens=20, max_chunk_size=16)
+    s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=8))
+    s.step()  # a: whole prompt, sampled
+    s.add_request(list(range(40)), GREEDY)
+    s.step()
+    assert ex.steps[1] == [("req-0", 1, True), ("req-1", 16, False)]  # decode first, then the portion
+    s.add_request(list(range(30)), GREEDY)
+    s.step()
+    # budget 20: 1 decode + 16 of req-1 + 3 left for the newcomer's first portion
+    assert ex.steps[2] == [("req-0", 1, True), ("req-1", 16, False), ("req-2", 3, False)]
+    for shape in ex.steps:
+        assert sum(n for _, n, _ in shape) <= 20
+    s.run_to_completion()
+    assert all(r.finish_reason == "length" for r in s._requests.values())
+
+
+def test_first_come_first_served_and_slot_limit():
+    s, ex = _make(seqs=2)
+    rs = [s.add_request([7] * 5, GREEDY) for _ in range(5)]
+    s.step()
+    assert [rid for rid, _, _ in ex.steps[0]] == ["req-0", "req-1"]  # two slots
+    s.run_to_completion()
+    first_step = {}
+    for i, shape in enumerate(ex.steps):
+        for rid, _, _ in shape:
+            first_step.setdefault(rid, i)
+    order = [first_step[r.request_id] for r in rs]
+    assert order == sorted(order)  # nobody overtakes
+    assert ex.cache.num_free_slots == 2
+    for shape in ex.steps:
+        assert len(shape) <= 2
+
+
+def test_chunking_off_runs_whole_prompts_only():
+    s, ex = _make(max_chunk_size=0, max_num_batched_tokens=128, max_len=128)
+    s.add_request(list(range(100)), GREEDY)
+    s.add_request(list(range(50)), GREEDY)
+    s.step()
+    assert ex.steps[0] == [("req-0", 100, True)]  # the second does not fit whole: it waits
+    s.step()
+    assert ex.steps[1] == [("req-0", 1, True), ("req-1", 50, True)]
+
+
+def test_eos_is_not_counted_and_finishes():
+    s, ex = _make(token=lambda rid, i: EOS if i == 2 else 5)
+    r = s.add_request([1, 2], SamplingParams(temperature=0.0, max_gen_len=10))
+    keep = s.add_request([1, 2], SamplingParams(temperature=0.0, max_gen_len=5, ignore_eos=True))
+    s.run_to_completion()
+    assert r.output_token_ids == [5, 5] and r.finish_reason == "eos"  # scheduler.py:1430-1436
+    assert keep.output_token_ids == [5, 5, EOS, 5, 5] and keep.finish_reason == "length"
+
+
+def test_length_cap_is_exact_at_the_context_limit():
+    s, ex = _make(max_len=16)
+    r = s.add_request(list(range(10)), SamplingParams(temperature=0.0))
+    s.run_to_completion()
+    assert len(r.output_token_ids) == 6 and r.seq_len == 16 and r.finish_reason == "length"
+    assert ex.cache.num_free_pages() == 63
+
+
+def test_abort_frees_everything():
+    s, ex = _make()
+    a = s.add_request(list(range(20)), GREEDY)
+    b = s.add_request(list(range(20)), GREEDY)
+    s.step()
+    s.abort(a.request_id)
+    s.abort(b.request_id)
+    s.abort("nobody")
+    assert a.finish_reason == b.finish_reason == "abort"
+    assert not s.has_unfinished_requests() and not ex.cache.live_requests()
+    ex.cache.check_invariants()
+
+
+def test_when_pages_run_out_the_youngest_is_evicted_and_recomputed():
+    # 7 usable pages of 4: two requests of 8 prompt tokens + 12 outputs need 5 pages each
+    s, ex = _make(num_pages=8, page=4, token=lambda rid, i: (hash(rid) % 50) * 100 + i)
+    params = SamplingParams(temperature=0.0, max_gen_len=12)
+    a = s.add_request(list(range(8)), params)
+    b = s.add_request(list(range(50, 58)), params)
+    steps = 0
+    while s.has_unfinished_requests():
+        s.step()
+        steps += 1
+        assert steps < 200, "livelock"
+    assert s.num_preemptions >= 1 and b.num_preemptions >= 1 and a.num_preemptions == 0
+    for r in (a, b):
+        base = (hash(r.request_id) % 50) * 100
+        assert r.output_token_ids == [base + i for i in range(12)]  # nothing lost, nothing doubled
+        assert r.finish_reason == "length"
+    # the evicted request ran its own outputs again as if they were prompt
+    evictions = [i for i, shape in enumerate(ex.steps) if any(rid == "req-1" and n > 1 for rid, n, _ in shape)]
+    assert len(evictions) >= 2
+    assert ex.cache.num_free_pages() == 7 and ex.cache.num_free_slots == 4
+    ex.cache.check_invariants()
+
+
+def test_evicted_request_returns_to_the_front_of_the_queue():
+    s, ex = _make(num_pages=8, page=4, seqs=4)
+    params = SamplingParams(temperature=0.0, max_gen_len=12)
+    a = s.add_request(list(range(8)), params)
+    b = s.add_request(list(range(8)), params)
+    while s.num_preemptions == 0:
+        s.step()
+    late = s.add_request([1, 2, 3], params)
+    assert s.waiting[0] is b and s.waiting[1] is late  # batch_planner.py:987-1023
+    s.run_to_completion()
+    assert len(b.output_token_ids) == 12 and len(late.output_token_ids) == 12
+
+
+def test_a_request_alone_in_a_pool_too_small_ends_with_length():
+    s, ex = _make(num_pages=4, page=4)  # 12 positions
+    r = s.add_request(list(range(6)), SamplingParams(temperature=0.0, max_gen_len=50))
+    s.run_to_completion()
+    assert r.finish_reason == "length" and r.seq_len == 13  # the 13th token had no page to be fed into
+    assert ex.cache.num_free_pages() == 3
+
+
+def test_requests_stuck_in_their_prompts_do_not_deadlock():
+    # both prompts fit alone but not together: neither can grow, nobody decodes
+    s, ex = _make(num_pages=11, page=4, max_chunk_size=8, max_num_batched_tokens=16)
+    params = SamplingParams(temperature=0.0, max_gen_len=2)
+    a = s.add_request(list(range(36)), params)
+    b = s.add_request(list(range(36)), params)
+    steps = 0
+    while s.has_unfinished_requests():
+        s.step()
+        steps += 1
+        assert steps < 100
+    assert len(a.output_token_ids) == 2 and len(b.output_token_ids) == 2
+    assert b.num_preemptions >= 1 and a.num_preemptions == 0
+    ex.cache.check_invariants()
+
+
+def test_slot_and_page_conservation_over_many_rounds():
+    import random
+
+    rng = random.Random(3)
+    s, ex = _make(num_pages=20, page=4, seqs=3, max_num_batched_tokens=24, max_chunk_size=8)
+    done = []
+    for round_ in range(30):
+        for _ in range(rng.randrange(0, 3)):
+            n = rng.randrange(1, 30)
+            done.append(s.add_request([rng.randrange(90) for _ in range(n)],
+                                      SamplingParams(temperature=0.0, max_gen_len=rng.randrange(1, 20))))
+        for _ in range(rng.randrange(1, 6)):
+            s.step()
+            assert len(s.running) <= 3
+    s.run_to_completion()
+    assert all(r.is_finished and len(r.output_token_ids) == r.max_new_tokens for r in done)
+    assert ex.cache.num_free_pages() == 19 and ex.cache.num_free_slots == 3
+    # what was fed is the request's own sequence, in order (checked while it was live)
+
+
+def test_fed_tokens_are_the_requests_own_sequence():
+    s, ex = _make(num_pages=8, page=4, token=lambda rid, i: 200 + i)
+    a = s.add_request(list(range(10)), SamplingParams(temperature=0.0, max_gen_len=9))
+    b = s.add_request(list(range(30, 40)), SamplingParams(temperature=0.0, max_gen_len=9))
+    while s.has_unfinished_requests():
+        s.step()
+        for r in s.running:
+            fed = ex.fed.get(r.request_id, [])
+            whole = r.prompt_token_ids + r.output_token_ids
+            assert fed == whole[: len(fed)] and len(fed) == r.num_computed_tokens
+    assert s.num_preemptions >= 1
+
+
+def test_seeds_are_per_request_and_stable():
+    s1, _ = _make(seed=5)
+    s2, _ = _make(seed=5)
+    s3, _ = _make(seed=6)
+    a = [s1.add_request([1], GREEDY).seed for _ in range(3)]
+    b = [s2.add_request([1], GREEDY).seed for _ in range(3)]
+    c = [s3.add_request([1], GREEDY).seed for _ in range(3)]
+    assert a == b and len(set(a)) == 3 and a != c
+    assert s1.add_request([1], SamplingParams(seed=77)).seed == 77
+
+
+def test_logprobs_are_collected_when_asked():
+    s, _ = _make()
+    r = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=3, logprobs=0))
+    q = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=3))
+    s.run_to_completion()
+    assert r.output_logprobs == [-1.0, -1.0, -1.0] and q.output_logprobs is None
+
+
+def test_repetition_breaker():
+    assert not detect_repetition(list(range(200)))
+    loop = list(range(32)) * 5
+    assert detect_repetition(loop)
+    assert not detect_repetition(loop[:100])
+    s, _ = _make(max_len=512, num_pages=200, token=lambda rid, i: i % 8)
+    r = s.add_request([1], SamplingParams(temperature=0.0, stop_on_repeat=True))
+    free = s.add_request([1], SamplingParams(temperature=0.0, max_gen_len=300))
+    s.run_to_completion()
+    assert r.finish_reason == "repeat" and len(r.output_token_ids) < 200
+    assert free.finish_reason == "length" and len(free.output_token_ids) == 300
+
+
+def test_sampling_params_validation():
+    SamplingParams()
+    for bad in (dict(temperature=-1), dict(top_p=0), dict(top_p=1.5), dict(max_gen_len=0),
+                dict(repetition_penalty=0), dict(logprobs=-1), dict(logprobs=5), dict(prompt_logprobs=1),
+                dict(seed=-3)):
+        with pytest.raises(ValueError):
+            SamplingParams(**bad)
+    assert SamplingParams(temperature=0).is_greedy and not SamplingParams().is_greedy
