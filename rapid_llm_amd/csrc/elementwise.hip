@@ -66,18 +66,95 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __rest
         o[i] = from_float<T>(res[i] * rrms * weight[i]);
 }
 
+// The same with four elements per thread and load: a row of up to 16 * blockDim elements
+// stays in registers between the two passes, so a row costs one round trip to memory.  With
+// few rows (decode) the kernel's time is that latency, not bandwidth.
+template <typename T>
+struct alignas(sizeof(T) * 4) Vec4 {
+    T v[4];
+};
+
+template <typename T, int CHUNKS>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                       const float* __restrict__ weight, T* __restrict__ out,
+                                       const int* __restrict__ rows, int hidden, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int row = rows ? rows[r] : r;
+    float4* res = reinterpret_cast<float4*>(residual + (size_t)row * hidden);
+    const Vec4<T>* dl = delta ? reinterpret_cast<const Vec4<T>*>(delta + (size_t)row * hidden) : nullptr;
+    const int nvec = hidden >> 2;
+    float4 val[CHUNKS];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) {
+            float4 v = res[i];
+            if (dl) {
+                const Vec4<T> d = dl[i];
+                v.x += to_float(d.v[0]);
+                v.y += to_float(d.v[1]);
+                v.z += to_float(d.v[2]);
+                v.w += to_float(d.v[3]);
+                res[i] = v;
+            }
+            val[c] = v;
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float rrms = rsqrtf(ss / (float)hidden + eps);
+    Vec4<T>* o = reinterpret_cast<Vec4<T>*>(out + (size_t)r * hidden);
+    const float4* w4 = reinterpret_cast<const float4*>(weight);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) {
+            const float4 w = w4[i];
+            Vec4<T> y;
+            y.v[0] = from_float<T>(val[c].x * rrms * w.x);
+            y.v[1] = from_float<T>(val[c].y * rrms * w.y);
+            y.v[2] = from_float<T>(val[c].z * rrms * w.z);
+            y.v[3] = from_float<T>(val[c].w * rrms * w.w);
+            o[i] = y;
+        }
+    }
+}
+
+template <typename T>
+static void launch_add_rmsnorm(float* residual, const T* delta, const float* weight, T* out,
+                               const int* rows, int out_rows, int hidden, float eps,
+                               hipStream_t stream) {
+    dim3 grid(out_rows);
+    if (hidden % 4 == 0 && hidden <= 16 * 1024) {
+        const int nvec = hidden / 4;
+        // one chunk per thread while the block stays within 1024 threads, then up to four
+        int threads = ((nvec + RL_WAVE - 1) / RL_WAVE) * RL_WAVE;
+        if (threads <= 1024) {
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, 1>), grid, dim3(threads), 0, stream,
+                               residual, delta, weight, out, rows, hidden, eps);
+        } else {
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, 4>), grid, dim3(1024), 0, stream,
+                               residual, delta, weight, out, rows, hidden, eps);
+        }
+        return;
+    }
+    int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+    hipLaunchKernelGGL(add_rmsnorm_kernel<T>, grid, dim3(threads), 0, stream, residual, delta,
+                       weight, out, rows, hidden, eps);
+}
+
 extern "C" int rl_add_rmsnorm(float* residual, const void* delta, const float* weight, void* out,
                               const int* rows, int out_rows, int hidden, float eps, int act_type,
                               hipStream_t stream) {
     if (out_rows <= 0) return RL_OK;
-    int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
-    dim3 grid(out_rows), block(threads);
     if (act_type == RL_F32)
-        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, stream, residual,
-                           (const float*)delta, weight, (float*)out, rows, hidden, eps);
+        launch_add_rmsnorm<float>(residual, (const float*)delta, weight, (float*)out, rows,
+                                  out_rows, hidden, eps, stream);
     else if (act_type == RL_BF16)
-        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, residual,
-                           (const bf16_t*)delta, weight, (bf16_t*)out, rows, hidden, eps);
+        launch_add_rmsnorm<bf16_t>(residual, (const bf16_t*)delta, weight, (bf16_t*)out, rows,
+                                   out_rows, hidden, eps, stream);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -103,19 +180,58 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
     }
 }
 
-extern "C" int rl_swiglu(const void* gate_up, void* out, int tokens, int inter, int act_type,
-                         hipStream_t stream) {
-    if (tokens <= 0) return RL_OK;
+// eight elements per thread (16-byte loads for bfloat16) when the width allows it
+template <typename T>
+struct alignas(sizeof(T) * 8) Vec8 {
+    T v[8];
+};
+
+template <typename T>
+__global__ void swiglu_vec_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter,
+                                  size_t total_vec) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    const int per_row = inter >> 3;
+    for (; idx < total_vec; idx += step) {
+        const size_t t = idx / per_row;
+        const int j = (int)(idx - t * per_row) << 3;
+        const T* row = gate_up + t * 2 * (size_t)inter;
+        const Vec8<T> g = *reinterpret_cast<const Vec8<T>*>(row + j);
+        const Vec8<T> u = *reinterpret_cast<const Vec8<T>*>(row + inter + j);
+        Vec8<T> y;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float gf = to_float(g.v[i]);
+            y.v[i] = from_float<T>(gf / (1.f + expf(-gf)) * to_float(u.v[i]));
+        }
+        *reinterpret_cast<Vec8<T>*>(out + t * (size_t)inter + j) = y;
+    }
+}
+
+template <typename T>
+static void launch_swiglu(const T* gate_up, T* out, int tokens, int inter, hipStream_t stream) {
+    if (inter % 8 == 0) {
+        const size_t total = (size_t)tokens * (inter / 8);
+        size_t blocks = (total + 255) / 256;
+        if (blocks > 65536) blocks = 65536;
+        hipLaunchKernelGGL(swiglu_vec_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           gate_up, out, inter, total);
+        return;
+    }
     const size_t total = (size_t)tokens * inter;
     size_t blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
-    dim3 grid((unsigned)blocks), block(256);
+    hipLaunchKernelGGL(swiglu_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, gate_up, out,
+                       inter, total);
+}
+
+extern "C" int rl_swiglu(const void* gate_up, void* out, int tokens, int inter, int act_type,
+                         hipStream_t stream) {
+    if (tokens <= 0) return RL_OK;
     if (act_type == RL_F32)
-        hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (const float*)gate_up,
-                           (float*)out, inter, total);
+        launch_swiglu<float>((const float*)gate_up, (float*)out, tokens, inter, stream);
     else if (act_type == RL_BF16)
-        hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gate_up,
-                           (bf16_t*)out, inter, total);
+        launch_swiglu<bf16_t>((const bf16_t*)gate_up, (bf16_t*)out, tokens, inter, stream);
     else
         return RL_ERR_ARG;
     return rl_launch_status();
@@ -186,7 +302,8 @@ extern "C" int rl_rope_table(const float* inv_freq, float* cos_out, float* sin_o
 
 // --------------------------------------------------------------------------- //
 // Fused per-head RMSNorm (optional) + half-split rotation (optional) of q and k, and the
-// write of k and v into the paged cache.  One wave per (token, head).
+// write of k and v into the paged cache.  One wave per (token, head); a workgroup of four
+// waves takes four heads of a token.
 //
 // qkv row layout: [q heads | k heads | v heads], heads adjacent (rapid_llm/modules/linear.py:
 // 236-251).  Norm over head_dim before the rotation (rapid_llm/models/base.py:134-140).
@@ -223,7 +340,7 @@ __global__ void qknorm_rope_kvwrite_kernel(
         off = pos % page_size;
     }
 
-    for (int head = wave; head < total_heads; head += nwaves) {
+    for (int head = blockIdx.y * nwaves + wave; head < total_heads; head += nwaves * gridDim.y) {
         const T* x = row + (size_t)head * d;
         if (head >= nq + nkv) {
             // value head: copy into the transposed page
@@ -296,7 +413,9 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
     if (d % 2 || d > 256) return RL_ERR_ARG;
     // only a rotation over the whole head is implemented (pairs i, i + d/2)
     if (cos_tab && rotary_half != d / 2) return RL_ERR_ARG;
-    dim3 grid(tokens), block(256);
+    const int total_heads = nq + 2 * nkv;
+    const int head_groups = (total_heads + 3) / 4;
+    dim3 grid(tokens, head_groups > 65535 ? 65535 : head_groups), block(256);
     if (act_type == RL_F32)
         hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<float>, grid, block, 0, stream,
                            (const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,

@@ -1,5 +1,5 @@
 // Bandwidth-bound bfloat16 product for few rows (decode): out[M,N] = X[M,K] * W[N,K]^T with
-// M <= 64, float32 accumulation on the matrix cores, optionally fused with SwiGLU.
+// M <= 16, float32 accumulation on the matrix cores, optionally fused with SwiGLU.
 //
 // Every weight byte is read once, in long contiguous runs: a workgroup owns NT tiles of 16
 // weight rows and its 8 waves interleave over K in steps of 128 elements, so that at any
@@ -43,92 +43,91 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
     *p = float_to_bf16(v);
 }
 
-// MB: blocks of 16 rows of X (M <= 16 MB); NT: tiles of 16 weight rows per workgroup.
-// SWIGLU: tiles 2j / 2j+1 are gate rows / up rows; N is then the width I of the result.
-template <int MB, int NT, typename OutT, bool SWIGLU>
+// NT: tiles of 16 weight rows per workgroup.  M <= 16: the rows of X are the 16 columns of
+// one matrix instruction.  SWIGLU: tiles 2j / 2j+1 are gate rows / up rows; N is then the
+// width I of the result.
+//
+// Measured on MI355X (graph replays, weights rotated through 800 MB so that nothing stays in
+// cache): a plain 16-byte-per-lane read kernel reaches 6.2-6.5 TB/s on 1.2 GB and 5 TB/s on
+// 32 MB (launch and ramp are about 2 us); this kernel reaches 6.2 TB/s on the vocabulary
+// matrix and 3.7-4.7 TB/s on the 33-100 MB matrices of a layer at one row.  Deeper unrolling,
+// non-temporal loads, more waves and staggered K offsets did not help; fewer instructions in
+// the loop did, hence the unpredicated main loop with clamped row pointers.
+template <int NT, typename OutT, bool SWIGLU>
 __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, OutT* __restrict__ out, int M,
     int N, int K, int ldx, int ldw, int ldo) {
-    __shared__ float red[GW][NT * MB * 256];
+    __shared__ float red[GW][NT * 256];
 
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
     const int r16 = lane & 15;
     const int g = lane >> 4;
 
-    // weight rows of this lane, one per tile (row >= limit: zeros)
+    // weight row of this lane in each tile; rows beyond the matrix read the last row and
+    // their results are dropped in the epilogue
     const bf16_t* wrow[NT];
-    bool wok[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         int row;
         if (SWIGLU) {
-            const int n = (blockIdx.x * (NT / 2) + nt / 2) * 16 + r16;
-            wok[nt] = n < N;
+            const int n = min((blockIdx.x * (NT / 2) + nt / 2) * 16 + r16, N - 1);
             row = (nt & 1) ? N + n : n;
         } else {
-            row = (blockIdx.x * NT + nt) * 16 + r16;
-            wok[nt] = row < N;
+            row = min((blockIdx.x * NT + nt) * 16 + r16, N - 1);
         }
-        wrow[nt] = W + (size_t)(wok[nt] ? row : 0) * ldw;
+        wrow[nt] = W + (size_t)row * ldw + 32 * g;
     }
-    const bf16_t* xrow[MB];
-    bool xok[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        const int m = mb * 16 + r16;
-        xok[mb] = m < M;
-        xrow[mb] = X + (size_t)(xok[mb] ? m : 0) * ldx;
-    }
+    const bool xok = r16 < M;
+    const bf16_t* xrow = X + (size_t)(xok ? r16 : 0) * ldx + 32 * g;
 
-    f32x4 acc[NT][MB];
+    f32x4 acc[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[nt][mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // the loop bound is the same for every lane of a wave: matrix instructions need them all
-    for (int kw = wave * KSTEP; kw < K; kw += GW * KSTEP) {
-        const int k0 = kw + 32 * g;
-        bf16x8 a[NT][4], x[MB][4];
-        // K is a multiple of 8: a piece is either whole or absent
+    // whole chunks of 128: no predicates.  The bound is the same for every lane of a wave.
+    const int kfull = K & ~(KSTEP - 1);
+    for (int kw = wave * KSTEP; kw < kfull; kw += GW * KSTEP) {
+        bf16x8 a[NT][4], x[4];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                a[nt][j] = (wok[nt] && k0 + 8 * j < K) ? ld16(wrow[nt] + k0 + 8 * j) : z8();
+            for (int j = 0; j < 4; ++j) a[nt][j] = ld16(wrow[nt] + kw + 8 * j);
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                x[mb][j] = (xok[mb] && k0 + 8 * j < K) ? ld16(xrow[mb] + k0 + 8 * j) : z8();
+        for (int j = 0; j < 4; ++j) x[j] = xok ? ld16(xrow + kw + 8 * j) : z8();
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], x[j], acc[nt], 0, 0, 0);
+    }
+    // the last, partial chunk (K is a multiple of 8: a piece is whole or absent)
+    if (kfull < K && wave == (kfull / KSTEP) % GW) {
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-                    acc[nt][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], x[mb][j],
-                                                                          acc[nt][mb], 0, 0, 0);
+        for (int j = 0; j < 4; ++j) {
+            const bool ok = kfull + 32 * g + 8 * j < K;
+            const bf16x8 xv = (ok && xok) ? ld16(xrow + kfull + 8 * j) : z8();
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const bf16x8 av = ok ? ld16(wrow[nt] + kfull + 8 * j) : z8();
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, xv, acc[nt], 0, 0, 0);
+            }
+        }
     }
 
     // partial tiles of the waves -> LDS; lane-major so that reads below are conflict-free
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                red[wave][((nt * MB + mb) * 4 + i) * 64 + lane] = acc[nt][mb][i];
+        for (int i = 0; i < 4; ++i) red[wave][(nt * 4 + i) * 64 + lane] = acc[nt][i];
     __syncthreads();
 
-    // thread -> (tile pair / tile, block of X rows, lane of the tile); sums the waves in order
+    // thread -> (tile pair / tile, lane of the tile); sums the waves in order
     constexpr int OUT_TILES = SWIGLU ? NT / 2 : NT;
-    for (int e = threadIdx.x; e < OUT_TILES * MB * 64; e += GW * RL_WAVE) {
+    for (int e = threadIdx.x; e < OUT_TILES * 64; e += GW * RL_WAVE) {
         const int ln = e & 63;
-        const int mb = (e >> 6) % MB;
-        const int ot = (e >> 6) / MB;
-        const int m = mb * 16 + (ln & 15);
+        const int ot = e >> 6;
+        const int m = ln & 15;
         const int nbase = (blockIdx.x * OUT_TILES + ot) * 16 + 4 * (ln >> 4);
         if (m >= M) continue;
 #pragma unroll
@@ -140,8 +139,8 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
                 float gate = 0.f, up = 0.f;
 #pragma unroll
                 for (int w = 0; w < GW; ++w) {
-                    gate += red[w][(((2 * ot) * MB + mb) * 4 + i) * 64 + ln];
-                    up += red[w][(((2 * ot + 1) * MB + mb) * 4 + i) * 64 + ln];
+                    gate += red[w][((2 * ot) * 4 + i) * 64 + ln];
+                    up += red[w][((2 * ot + 1) * 4 + i) * 64 + ln];
                 }
                 // the activation reads its operands rounded to bfloat16, as the unfused
                 // path does where the product's result is stored before the activation
@@ -151,34 +150,32 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
             } else {
                 v = 0.f;
 #pragma unroll
-                for (int w = 0; w < GW; ++w) v += red[w][((ot * MB + mb) * 4 + i) * 64 + ln];
+                for (int w = 0; w < GW; ++w) v += red[w][(ot * 4 + i) * 64 + ln];
             }
             store_out<OutT>(out + (size_t)m * ldo + n, v);
         }
     }
 }
 
-template <int MB, int NT, typename OutT, bool SWIGLU>
+template <int NT, typename OutT, bool SWIGLU>
 static int launch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
                   int ldw, int ldo, hipStream_t stream) {
     constexpr int rows_per_block = (SWIGLU ? NT / 2 : NT) * 16;
     dim3 grid((N + rows_per_block - 1) / rows_per_block), block(GW * RL_WAVE);
-    hipLaunchKernelGGL((gemm_skinny_kernel<MB, NT, OutT, SWIGLU>), grid, block, 0, stream, X, W,
-                       out, M, N, K, ldx, ldw, ldo);
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, OutT, SWIGLU>), grid, block, 0, stream, X, W, out,
+                       M, N, K, ldx, ldw, ldo);
     return rl_launch_status();
 }
 
 template <typename OutT, bool SWIGLU>
 static int dispatch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
                     int ldw, int ldo, int nt, hipStream_t stream) {
-    const int mb = (M + 15) / 16;
-#define RL_CASE(MBV, NTV)                                                                      \
-    if (mb <= MBV && nt == NTV)                                                                \
-        return launch<MBV, NTV, OutT, SWIGLU>(X, W, out, M, N, K, ldx, ldw, ldo, stream);
+#define RL_CASE(NTV)                                                                           \
+    if (nt == NTV) return launch<NTV, OutT, SWIGLU>(X, W, out, M, N, K, ldx, ldw, ldo, stream);
     if (SWIGLU) {
-        RL_CASE(1, 2) RL_CASE(1, 4) RL_CASE(2, 2)
+        RL_CASE(2) RL_CASE(4)
     } else {
-        RL_CASE(1, 1) RL_CASE(1, 2) RL_CASE(1, 4) RL_CASE(2, 1) RL_CASE(2, 2) RL_CASE(4, 1)
+        RL_CASE(1) RL_CASE(2)
     }
 #undef RL_CASE
     return RL_ERR_ARG;
@@ -189,7 +186,7 @@ extern "C" int rl_gemm_skinny(const void* X, const void* W, void* out, int M, in
                               int ldx, int ldw, int ldo, int out_type, int nt,
                               hipStream_t stream) {
     if (M <= 0 || N <= 0) return RL_OK;
-    if (M > 64 || K < 8 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < N)
+    if (M > 16 || K < 8 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < N)
         return RL_ERR_ARG;
     if (out_type == RL_F32)
         return dispatch<float, false>((const bf16_t*)X, (const bf16_t*)W, (float*)out, M, N, K,
@@ -204,7 +201,7 @@ extern "C" int rl_gemm_skinny(const void* X, const void* W, void* out, int M, in
 extern "C" int rl_gemm_skinny_swiglu(const void* X, const void* W, void* out, int M, int I, int K,
                                      int ldx, int ldw, int ldo, int nt, hipStream_t stream) {
     if (M <= 0 || I <= 0) return RL_OK;
-    if (M > 32 || K < 8 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < I)
+    if (M > 16 || K < 8 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < I)
         return RL_ERR_ARG;
     return dispatch<bf16_t, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx,
                                   ldw, ldo, nt, stream);

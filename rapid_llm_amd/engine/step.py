@@ -325,17 +325,18 @@ class ModelRunner:
         return logits
 
     @torch.no_grad()
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], use_graph: bool | None = None) -> torch.Tensor:
         """Run one batch; returns float32 logits ``[wanted, vocab]`` in the order of the
         entries and of each entry's ``want``.  Raises :class:`OutOfPages`, with nothing
         changed, when slots or pages do not suffice.  The returned tensor may be reused by
-        the next step: read it (sample from it, copy it) before stepping again."""
+        the next step: read it (sample from it, copy it) before stepping again.
+        ``use_graph`` overrides the engine's setting for this one step."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         host, offs, meta = self._prepare(entries)
         if (
-            self.engine.use_graph
-            and len(entries) <= ops.SKINNY_MAX_ROWS
+            (self.engine.use_graph if use_graph is None else use_graph)
+            and len(entries) <= ops.GRAPH_MAX_ROWS
             and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
         ):
             logits = self._graph_step(entries, host, offs, meta)

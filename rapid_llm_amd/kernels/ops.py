@@ -321,30 +321,23 @@ def sample_uniform(seed: int, counter: int) -> float:
     return float(fn(ctypes.c_uint(seed & 0xFFFFFFFF), ctypes.c_uint((seed >> 32) & 0xFFFFFFFF), ctypes.c_uint(counter)))
 
 
-SKINNY_MAX_ROWS = 64  # rows up to which the bandwidth-bound product is used
-SWIGLU_MAX_ROWS = 32
-_MIN_BLOCKS = 512  # workgroups a skinny product should reach before it widens its tiles
+SKINNY_MAX_ROWS = 16  # rows up to which the hand-written bandwidth-bound product is used
+GRAPH_MAX_ROWS = 64  # decode batches up to this size are replayed from HIP graphs
+_MIN_BLOCKS = 512  # workgroups a skinny product should keep when it widens its tiles
 
 
-def _skinny_tiles(rows: int, out_features: int, choices: tuple[int, ...]) -> int:
-    """Weight-row tiles per workgroup: the most the accumulators allow while the launch
-    still has a couple of workgroups per compute unit."""
-    mb = -(-rows // 16)
-    mbv = 1 if mb <= 1 else (2 if mb == 2 else 4)
-    best = None
-    for nt in choices:
-        if nt * mbv > 4:
-            continue
-        if best is None or -(-out_features // (16 * nt)) >= _MIN_BLOCKS:
-            best = nt
-    return best
+def _skinny_tiles(rows: int, out_features: int) -> int:
+    """Weight-row tiles per workgroup: two where the launch still has a couple of workgroups
+    per compute unit and more than a few rows share each weight tile (measured: 5% on the
+    widest matrices at 8 rows, a loss everywhere else)."""
+    return 2 if rows > 4 and -(-out_features // 32) >= _MIN_BLOCKS else 1
 
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     """``x[M,K] @ w[N,K]^T`` with bfloat16 operands and float32 accumulation.
 
-    Few rows (decode) run the hand-written bandwidth-bound kernel, which can write float32
-    directly.  Many rows go to the library product, as the reference's dense products do
+    Up to 16 rows (decode) run the hand-written bandwidth-bound kernel, which can write
+    float32 directly.  More rows go to the library product, as the reference's dense products do
     (``F.linear``); its bfloat16 result is returned as is and widened by the caller."""
     _need(x, "x", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
@@ -356,7 +349,7 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch
         if out_dtype not in (torch.bfloat16, torch.float32):
             raise KernelError(f"gemm_bf16 writes bfloat16 or float32, not {out_dtype}")
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-        nt = _skinny_tiles(m, n, (1, 2, 4))
+        nt = _skinny_tiles(m, n)
         _ok(
             core().rl_gemm_skinny(_p(x), _p(w), _p(out), m, n, k, k, k, n, _tag(out_dtype), nt, _stream()),
             "rl_gemm_skinny",
@@ -370,13 +363,13 @@ def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor |
     few rows; ``None`` when the shape is not one the fused kernel takes."""
     m, k = x.shape
     two_i = w_gate_up.shape[0]
-    if m > SWIGLU_MAX_ROWS or k % 8 or two_i % 2 or x.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16:
+    if m > SKINNY_MAX_ROWS or k % 8 or two_i % 2 or x.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16:
         return None
     _need(x, "x", torch.bfloat16)
     _need(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, k))
     inter = two_i // 2
     out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
-    nt = _skinny_tiles(m, inter, (1, 2)) * 2  # pairs of (gate, up) tiles
+    nt = _skinny_tiles(m, inter) * 2  # pairs of (gate, up) tiles
     _ok(
         core().rl_gemm_skinny_swiglu(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, _stream()),
         "rl_gemm_skinny_swiglu",

@@ -63,3 +63,42 @@ def test_graph_replays_match_eager(tmp_path, which, dtype):
         for rid in live:
             r.finish(rid)
         r.cache.check_invariants()
+
+
+@pytest.mark.parametrize("batch", [17, 40])
+def test_graph_of_a_batch_beyond_the_skinny_product(tmp_path, batch):
+    """More than 16 rows: the bfloat16 products are the library's.  Their graph replays are
+    checked one by one against eager steps of a second engine, with eager work between."""
+    from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
+
+    cfg, page, seed = TINY["B"]
+    model_dir = make_model_dir(tmp_path, "B", "bfloat16")
+    make = lambda graph: ModelRunner(
+        model_dir,
+        EngineConfig(dtype="bfloat16", max_seq_len=64, page_size=page, num_pages=batch * 4 + 8,
+                     max_num_seqs=batch + 1, use_graph=graph),
+    )
+    eager, graph = make(False), make(True)
+    vocab = cfg["vocab_size"]
+    nxt = {}
+    for i in range(batch):
+        prompt = random_tokens(3 + i % 9, vocab, seed + i)
+        a = eager.step([StepEntry(f"b{i}", prompt, [len(prompt) - 1])]).clone()
+        b = graph.step([StepEntry(f"b{i}", prompt, [len(prompt) - 1])]).clone()
+        torch.testing.assert_close(a, b, rtol=2e-2, atol=2e-2)
+        nxt[f"b{i}"] = int(a[0].argmax())
+    for step in range(12):
+        entries = [StepEntry(rid, [tok], [0]) for rid, tok in nxt.items()]
+        a = eager.step(entries).clone()
+        b = graph.step(entries).clone()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(a, b, rtol=2e-2, atol=2e-2)
+        if step % 4 == 1:  # eager work of the program's own between replays
+            extra = random_tokens(5, vocab, step)
+            graph.step([StepEntry("x", extra, [4])])
+            graph.finish("x")
+            eager.step([StepEntry("x", extra, [4])])
+            eager.finish("x")
+        for k, rid in enumerate(nxt):
+            nxt[rid] = int(a[k].argmax())
+    assert batch in graph._graphs

@@ -150,7 +150,7 @@ def test_attention_window_edge():
 # norms, activation, rotation, cache write, products, embedding, arg-max
 # --------------------------------------------------------------------------- #
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("hidden", [80, 1000, 4096])
+@pytest.mark.parametrize("hidden", [80, 333, 1000, 4096, 5120, 16384, 20000])
 def test_add_rmsnorm(dtype, hidden):
     ops = _ops()
     t = 37
@@ -181,7 +181,12 @@ def test_add_rmsnorm(dtype, hidden):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_swiglu(dtype):
     ops = _ops()
-    t, inter = 19, 333
+    _swiglu_case(dtype, 19, 333)  # odd width: one element per thread
+    _swiglu_case(dtype, 70, 12288)  # eight per thread
+
+
+def _swiglu_case(dtype, t, inter):
+    ops = _ops()
     x = torch.randn(t, 2 * inter).to(dtype)
     want = torch.nn.functional.silu(x[:, :inter].float()) * x[:, inter:].float()
     out = torch.empty(t, inter, dtype=dtype, device=DEV)
@@ -264,7 +269,7 @@ def test_gemm_f32(shape):
     assert torch.equal(out1[0], out[m // 2])
 
 
-@pytest.mark.parametrize("shape", [(1, 503, 96), (8, 4096, 4096), (64, 1000, 12288), (200, 331, 80), (3, 24, 48)])
+@pytest.mark.parametrize("shape", [(1, 503, 96), (8, 4096, 4096), (16, 300, 1000), (64, 1000, 12288), (17, 6144, 4096), (200, 331, 80), (3, 24, 48)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16out", "f32out"])
 def test_gemm_bf16(shape, out_dtype):
     ops = _ops()
@@ -277,7 +282,7 @@ def test_gemm_bf16(shape, out_dtype):
     torch.testing.assert_close(got.float().cpu(), want, **tol)
 
 
-@pytest.mark.parametrize("shape", [(1, 320, 96), (8, 12288, 4096), (32, 176, 80), (17, 100, 64)])
+@pytest.mark.parametrize("shape", [(1, 320, 96), (8, 12288, 4096), (16, 176, 80), (13, 100, 64), (5, 24, 200)])
 def test_gemm_bf16_swiglu_fused(shape):
     ops = _ops()
     m, inter, k = shape
