@@ -127,7 +127,60 @@ __device__ inline bf16x8 softmax_step(f32x4 s0, f32x4 s1, unsigned ok0, unsigned
 // decode
 // =========================================================================== //
 #define DEC_WAVES 4
+#define DEC_MAX_PAGES 1024  // pages one split may span (their ids are staged in LDS)
 
+// Keys of one 32-key step as the two matrix products see them.  Tile row i of key block kb
+// is the physical key  base + 8 (i / 4) + 4 kb + (i % 4),  so that lane (row, g) leaves the
+// first product with the scores of the eight *consecutive* keys base + 8g .. base + 8g + 7:
+// exactly its contraction slots of the second product, whose A operand (values, stored
+// transposed) is then one 16-byte read of those eight positions of a channel.
+struct DecodeFrags {
+    bf16x8 k[2][DC];
+    bf16x8 v[DB];
+};
+
+template <bool V16>
+__device__ inline void decode_load(DecodeFrags& f, const bf16_t* __restrict__ k_cache,
+                                   const bf16_t* __restrict__ v_cache, const int* pages,
+                                   int page0, int page_size, int nkv, int hk, int base,
+                                   int last_key, int col, int g) {
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+        const int key = min(base + 8 * (col >> 2) + 4 * kb + (col & 3), last_key);  // masked later
+        const int page = pages[key / page_size - page0];
+        const bf16_t* krow =
+            k_cache + (((size_t)page * nkv + hk) * page_size + key % page_size) * D;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
+            f.k[kb][c] = chan_ok ? load16(krow + 32 * c + 8 * g) : zero8();
+        }
+    }
+    if (V16) {
+        // eight positions of one page row; clamped as a group so that the read stays inside
+        // the request's last page (what is read there is zeroed before use)
+        const int key = min(base + 8 * g, last_key & ~7);
+        const int page = pages[key / page_size - page0];
+        const bf16_t* vrow = v_cache + (((size_t)page * nkv + hk) * D) * page_size + key % page_size;
+#pragma unroll
+        for (int b = 0; b < DB; ++b) f.v[b] = load16(vrow + (size_t)(16 * b + col) * page_size);
+    } else {
+        const bf16_t* vrow[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int key = min(base + 8 * g + 4 * h, last_key & ~3);
+            const int page = pages[key / page_size - page0];
+            vrow[h] = v_cache + (((size_t)page * nkv + hk) * D) * page_size + key % page_size;
+        }
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+            const size_t doff = (size_t)(16 * b + col) * page_size;
+            f.v[b] = load8x2(vrow[0] + doff, vrow[1] + doff);
+        }
+    }
+}
+
+template <bool V16>
 __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out, float* __restrict__ part_o,
@@ -138,6 +191,7 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
     __shared__ float lds_o[2][D * 16];
     __shared__ float lds_m[2][16];
     __shared__ float lds_l[2][16];
+    __shared__ int lds_pages[DEC_MAX_PAGES + 2];
 
     const int G = nq / nkv;
     const int head_chunks = (G + 15) / 16;
@@ -171,7 +225,14 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
         }
         return;
     }
-
+    // page ids of the split, once: the loop's loads then depend on nothing but LDS
+    const int last_key = kend - 1;
+    const int page0 = lo / page_size;
+    {
+        const int npages = last_key / page_size - page0 + 1;  // <= DEC_MAX_PAGES + 1 (host)
+        for (int i = threadIdx.x; i < npages && i < DEC_MAX_PAGES + 2; i += DEC_WAVES * RL_WAVE)
+            lds_pages[i] = table[page0 + i];
+    }
     // Q^T as B operand: lane (row col, group g) holds channels 32c + 8g .. + 7
     bf16x8 qf[DC];
     {
@@ -182,57 +243,49 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
             qf[c] = (head_ok && chan_ok) ? load16(qrow + 32 * c + 8 * g) : zero8();
         }
     }
+    __syncthreads();
 
     float m = -INFINITY, l = 0.f;
     f32x4 acc[DB];
 #pragma unroll
     for (int b = 0; b < DB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    const int last_key = kend - 1;
-    for (int base = lo + 32 * wave; base < hi; base += 32 * DEC_WAVES) {
+    // the loads of the next step are issued before this step's arithmetic
+    DecodeFrags cur, nxt;
+    int base = lo + 32 * wave;
+    if (base < hi)
+        decode_load<V16>(cur, k_cache, v_cache, lds_pages, page0, page_size, nkv, hk, base,
+                         last_key, col, g);
+    for (; base < hi; base += 32 * DEC_WAVES) {
+        const int next = base + 32 * DEC_WAVES;
+        if (next < hi)
+            decode_load<V16>(nxt, k_cache, v_cache, lds_pages, page0, page_size, nkv, hk, next,
+                             last_key, col, g);
         // ---- S^T = K Q^T for two blocks of 16 keys --------------------------------
         f32x4 s[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-            const int key = min(base + 16 * kb + col, last_key);  // clamped: masked below
-            const int page = table[key / page_size];
-            const bf16_t* krow =
-                k_cache + (((size_t)page * nkv + hk) * page_size + key % page_size) * D;
             s[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < DC; ++c) {
-                const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
-                const bf16x8 a = chan_ok ? load16(krow + 32 * c + 8 * g) : zero8();
-                s[kb] = mfma(a, qf[c], s[kb]);
-            }
+            for (int c = 0; c < DC; ++c) s[kb] = mfma(cur.k[kb][c], qf[c], s[kb]);
         }
-        // ---- which of this lane's keys are visible ---------------------------------
+        // ---- which of this lane's keys (base + 8g + 4kb + i) are visible ------------
         unsigned ok[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             ok[kb] = 0;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int key = base + 16 * kb + 4 * g + i;
+                const int key = base + 8 * g + 4 * kb + i;
                 ok[kb] |= (key >= kstart && key < kend) ? (1u << i) : 0u;
             }
         }
         const bf16x8 p = softmax_step(s[0], s[1], ok[0], ok[1], scale_log2, m, l, acc);
         // ---- O^T += V^T P^T ---------------------------------------------------------
         const bool partial = (base + 32 > kend) || (base < kstart);
-        const bf16_t* vrow[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            // this lane's four keys of the block; clamped as a group so that the read stays
-            // inside one page of the request (what is read there is zeroed below)
-            const int key = min(base + 16 * kb + 4 * g, last_key & ~3);
-            const int page = table[key / page_size];
-            vrow[kb] = v_cache + (((size_t)page * nkv + hk) * D) * page_size + key % page_size;
-        }
 #pragma unroll
         for (int b = 0; b < DB; ++b) {
-            const size_t doff = (size_t)(16 * b + col) * page_size;
-            bf16x8 v = load8x2(vrow[0] + doff, vrow[1] + doff);
+            bf16x8 v = cur.v[b];
             if (partial) {
                 // 0 * stale data must be 0: a page used before may hold anything
 #pragma unroll
@@ -243,6 +296,7 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
             }
             acc[b] = mfma(v, p, acc[b]);
         }
+        cur = nxt;
     }
 
     // ---- combine the waves: (2,3) -> (0,1), then 1 -> 0, in the accumulators' own layout ----
@@ -342,16 +396,24 @@ extern "C" int rl_attn_decode(const void* q, const void* k_cache, const void* v_
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || split_chunk < 32 ||
         split_chunk % 32 || nsplit < 1 || nsplit > 65535)
         return RL_ERR_ARG;
+    // a split's pages are staged in LDS (its keys may start up to 31 before a page's first)
+    if ((split_chunk + 31) / page_size + 1 > DEC_MAX_PAGES) return RL_ERR_ARG;
     if (nsplit > 1 && (!part_o || !part_ml)) return RL_ERR_ARG;
     const int G = nq / nkv;
     const int head_chunks = (G + 15) / 16;
     if ((long)nkv * head_chunks > 65535) return RL_ERR_ARG;
     const float scale_log2 = scale * 1.4426950408889634f;
     dim3 grid(num_seqs, nkv * head_chunks, nsplit), block(DEC_WAVES * RL_WAVE);
-    hipLaunchKernelGGL(attn_decode_kernel, grid, block, 0, stream, (const bf16_t*)q,
-                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_o,
-                       part_ml, seq_token, positions, token_slot, block_table, table_stride,
-                       page_size, nq, nkv, window, scale_log2, split_chunk, nsplit);
+    if (page_size % 8 == 0)
+        hipLaunchKernelGGL(attn_decode_kernel<true>, grid, block, 0, stream, (const bf16_t*)q,
+                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_o,
+                           part_ml, seq_token, positions, token_slot, block_table, table_stride,
+                           page_size, nq, nkv, window, scale_log2, split_chunk, nsplit);
+    else
+        hipLaunchKernelGGL(attn_decode_kernel<false>, grid, block, 0, stream, (const bf16_t*)q,
+                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_o,
+                           part_ml, seq_token, positions, token_slot, block_table, table_stride,
+                           page_size, nq, nkv, window, scale_log2, split_chunk, nsplit);
     if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
     if (nsplit > 1) {
         hipLaunchKernelGGL(attn_merge_kernel, dim3(num_seqs, nq), dim3(D < 64 ? 64 : D), 0,

@@ -141,7 +141,7 @@ class ModelRunner:
         self.device_cache = DeviceCache(self.cache, needs, group_of, self.dtype, self.device)
         self.computed: dict[str, int] = {}
         self.vocab_size = self.spec.vocab_size
-        self._graphs: dict[int, tuple] = {}
+        self._graphs: dict[tuple[int, int], tuple] = {}
 
     # ------------------------------------------------------------------ sizing
     def _decide_num_pages(self, groups) -> int:
@@ -288,19 +288,25 @@ class ModelRunner:
         """A step of single tokens, all wanted: replayed from a HIP graph captured once per
         batch size.  The graph holds only this package's kernels; its inputs are one static
         int32 buffer, refreshed by a copy on the same stream before each replay.  Launch
-        decisions that depend on the context length are made for the longest sequence the
-        engine allows, so one capture serves every step."""
+        decisions that depend on the context length are made for the bucket's longest context,
+        so one capture serves every step of that bucket."""
         batch = len(entries)
-        entry = self._graphs.get(batch)
+        # one graph per batch size and context bucket (the next power of two): the split of
+        # the keys over workgroups is fixed at capture and should fit the contexts it serves
+        bound = 512
+        while bound <= meta["max_position"]:
+            bound *= 2
+        bound = min(bound, self.engine.max_seq_len)
+        key = (batch, bound)
+        entry = self._graphs.get(key)
         if entry is None:
             static = torch.zeros(len(host), dtype=torch.int32, device=self.device)
             pinned = torch.empty(len(host), dtype=torch.int32, pin_memory=True)
             pinned.numpy()[:] = host
             static.copy_(pinned, non_blocking=True)
-            bound = dict(meta, max_position=self.engine.max_seq_len - 1)
-            ctx = self._context(static, offs, bound)
+            ctx = self._context(static, offs, dict(meta, max_position=bound - 1))
             ctx.extra["decode_only_tokens"] = torch.arange(batch, dtype=torch.int32, device=self.device)
-            ctx.extra["context_bound"] = self.engine.max_seq_len
+            ctx.extra["context_bound"] = bound
             # one eager run on a side stream first: kernels get loaded, the allocator warm
             current = torch.cuda.current_stream()
             side = torch.cuda.Stream()
@@ -317,7 +323,7 @@ class ModelRunner:
             # allocated outside the capture (the static inputs, the index list in ctx.extra)
             # must live as long as the graph does, so the context is kept with it
             entry = (graph, static, pinned, logits, ctx)
-            self._graphs[batch] = entry
+            self._graphs[key] = entry
         graph, static, pinned, logits, _ctx = entry
         pinned.numpy()[:] = host
         static.copy_(pinned, non_blocking=True)

@@ -414,7 +414,12 @@ class AttentionPlan:
         self.tile_info = packed[self.num_decode :]
 
 
-_TARGET_BLOCKS = 1024  # workgroups a decode launch should reach: a few per compute unit
+# Workgroups a decode launch should reach before it stops splitting the keys, and the fewest
+# keys a split is worth (measured at 2,048 keys, 8 kv heads: 1 request 256 keys a split,
+# 8 requests 512, 64 requests no split; finer splits only add merge work).
+_TARGET_BLOCKS = 256
+_MIN_SPLIT_KEYS = 256
+_MAX_SPLIT_PAGES = 1024  # page ids of one split are staged in LDS
 
 
 def paged_attention(
@@ -478,7 +483,8 @@ def paged_attention(
             span = min(span, window + 31)
         pairs = plan.num_decode * nkv * ((group + 15) // 16)
         want = max(1, _TARGET_BLOCKS // pairs)
-        chunk = max(128, -(-(-(-span // want)) // 128) * 128)
+        chunk = max(_MIN_SPLIT_KEYS, -(-(-(-span // want)) // 128) * 128)
+        chunk = min(chunk, max(32, ((_MAX_SPLIT_PAGES - 1) * page_size - 31) // 32 * 32))
         nsplit = -(-span // chunk)
         part_o = part_ml = None
         if nsplit > 1:
