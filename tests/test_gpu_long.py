@@ -1,0 +1,92 @@
+"""Long decoding (one token a step up to the model's last position, across pages, key splits,
+graph buckets and window trims) and the first tokens of a sequence, against the plain
+implementation."""
+
+import pytest
+import torch
+
+from plain_model import plain_forward, plain_load
+from tiny_configs import TINY, make_model_dir, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = dict(rtol=2e-5, atol=3e-6)
+BF16_TOL = dict(rtol=5e-2, atol=3e-2)
+
+
+def _runner(model_dir, dtype, page, max_seq_len, graph=False, num_pages=None, seqs=4):
+    from rapid_llm_amd import EngineConfig, ModelRunner
+
+    pages = num_pages or (seqs * (max_seq_len // page + 1) + 1)
+    return ModelRunner(
+        model_dir,
+        EngineConfig(dtype=dtype, max_seq_len=max_seq_len, page_size=page, num_pages=pages,
+                     max_num_seqs=seqs, use_graph=graph),
+    )
+
+
+@pytest.mark.parametrize("which", ["B", "C"])
+@pytest.mark.parametrize("dtype,graph", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
+def test_long_decoding(tmp_path, which, dtype, graph):
+    from rapid_llm_amd import StepEntry
+
+    cfg, page, seed = TINY[which]
+    model_dir = make_model_dir(tmp_path, which, dtype)
+    pcfg, pw = plain_load(model_dir)
+    limit = cfg["max_position_embeddings"]
+    # two requests decode side by side, one from a 5-token prompt, one from a 70-token prompt
+    toks = {"s": random_tokens(limit, cfg["vocab_size"], seed + 1), "l": random_tokens(limit - 40, cfg["vocab_size"], seed + 2)}
+    want = {rid: plain_forward(pcfg, pw, t) for rid, t in toks.items()}
+    runner = _runner(model_dir, dtype, page, limit, graph)
+    got = {rid: [] for rid in toks}
+    done = {"s": 5, "l": 70}
+    for rid in toks:
+        got[rid].append(runner.step([StepEntry(rid, toks[rid][: done[rid]], list(range(done[rid])))]).cpu())
+    while any(done[r] < len(toks[r]) for r in toks):
+        entries = [StepEntry(r, [toks[r][done[r]]], [0]) for r in toks if done[r] < len(toks[r])]
+        logits = runner.step(entries).cpu()
+        for k, e in enumerate(entries):
+            got[e.request_id].append(logits[k : k + 1])
+            done[e.request_id] += 1
+    tol = F32_TOL if dtype == "float32" else BF16_TOL
+    for rid in toks:
+        out = torch.cat(got[rid])
+        assert torch.isfinite(out).all()
+        torch.testing.assert_close(out, want[rid], **tol)
+        runner.finish(rid)
+    if graph:
+        assert len({key[1] for key in runner._graphs}) >= 1
+    if which == "C":  # windowed layers gave pages back while decoding
+        assert runner.cache.num_free_pages(1) == runner.cache.pools[1].num_usable
+    runner.cache.check_invariants()
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens(tmp_path, which, dtype):
+    """Positions 0, 1, 2: a one-token prompt, its first decoded tokens, a two-token prompt cut
+    into 1 + 1, and four one-token prompts in one batch."""
+    from rapid_llm_amd import StepEntry
+
+    cfg, page, seed = TINY[which]
+    model_dir = make_model_dir(tmp_path, which, dtype)
+    pcfg, pw = plain_load(model_dir)
+    runner = _runner(model_dir, dtype, page, 64)
+    tol = F32_TOL if dtype == "float32" else BF16_TOL
+    toks = random_tokens(4, cfg["vocab_size"], seed)
+    want = plain_forward(pcfg, pw, toks)
+    rows = [runner.step([StepEntry("a", toks[:1], [0])]).cpu()]
+    for t in toks[1:]:
+        rows.append(runner.step([StepEntry("a", [t], [0])]).cpu())
+    torch.testing.assert_close(torch.cat(rows), want, **tol)
+    first = runner.step([StepEntry("b", toks[:1], [0])]).cpu()
+    second = runner.step([StepEntry("b", toks[1:2], [0])]).cpu()
+    torch.testing.assert_close(torch.cat([first, second]), want[:2], **tol)
+    runner.finish("a")
+    runner.finish("b")
+    singles = random_tokens(4, cfg["vocab_size"], seed + 9)
+    batch = runner.step([StepEntry(f"s{i}", [t], [0]) for i, t in enumerate(singles)]).cpu()
+    for i, t in enumerate(singles):
+        torch.testing.assert_close(batch[i : i + 1], plain_forward(pcfg, pw, [t]), **tol)
+        runner.finish(f"s{i}")
+    runner.cache.check_invariants()
