@@ -425,14 +425,22 @@ extern "C" int rl_attn_decode(const void* q, const void* k_cache, const void* v_
 // =========================================================================== //
 // prefill
 // =========================================================================== //
+#ifndef RL_PF_NQ
+#define RL_PF_NQ 2
+#endif
 #define PF_WAVES 4
-#define PF_NQ 2                          // 16-row blocks per wave
+#define PF_NQ RL_PF_NQ                   // 16-row blocks per wave
 #define PF_ROWS (PF_WAVES * PF_NQ * 16)  // rows per workgroup
-#define PF_KEYS (D > 192 ? 32 : 64)      // keys per LDS tile (static LDS stays under 64 KB)
+#define PF_KEYS 64                       // keys per LDS tile and per softmax step
 #define PF_THREADS (PF_WAVES * RL_WAVE)
 #define K_LD (D + 8)                     // padded row of the K tile (bfloat16 elements)
 #define V_LD (PF_KEYS + 8)               // padded row of the V^T tile
 
+// Softmax is the arithmetic that competes with the matrix cores here, so a step covers 64
+// keys (one maximum, one rescale and one sum for 16 scores per lane), scores are masked only
+// in tiles that the diagonal, a window's edge or the end of the sequence crosses, and the
+// accumulators are rescaled only when some row's maximum moved.
+//
 // tile_info[4 * tile + {0,1,2,3}] = {first token of the request's portion in the flat batch,
 //   tokens of the request already in the cache, tokens in this portion, first row of the tile}
 __global__ __launch_bounds__(PF_WAVES* RL_WAVE) void attn_prefill_kernel(
@@ -485,6 +493,11 @@ __global__ __launch_bounds__(PF_WAVES* RL_WAVE) void attn_prefill_kernel(
     const int tile_kend = start + last_row / G + 1;
     const int first_pos = start + row0 / G;
     const int tile_kstart = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+    // positions of this wave's rows (rows ascend with the position)
+    const int w_first = min(row0 + wave * PF_NQ * 16, rows - 1);
+    const int w_last = min(row0 + (wave + 1) * PF_NQ * 16, rows) - 1;
+    const int wave_min_pos = start + w_first / G;
+    const int wave_max_pos = start + (w_last > w_first ? w_last : w_first) / G;
 
     float m[PF_NQ], l[PF_NQ];
     f32x4 acc[PF_NQ][DB];
@@ -539,51 +552,84 @@ __global__ __launch_bounds__(PF_WAVES* RL_WAVE) void attn_prefill_kernel(
             }
         }
         __syncthreads();
-        // ---- steps of 32 keys -----------------------------------------------------
+        if (base > wave_max_pos) continue;  // every key of the tile is ahead of this wave's rows
+        // masks are needed where the diagonal or a window's edge crosses the tile
+        const bool need_mask =
+            (base + PF_KEYS - 1 > wave_min_pos) || (window > 0 && base < wave_max_pos - window + 1);
+
+        // ---- S^T = K Q^T: tile row i of key block (hf, kb) is key 32 hf + 8 (i / 4) + 4 kb + i % 4,
+        // so that a lane ends up with the scores of keys 32 hf + 8 g .. + 7 (see DecodeFrags)
+        f32x4 s[PF_NQ][4];
 #pragma unroll
-        for (int hf = 0; hf < PF_KEYS / 32; ++hf) {
-            const int kb0 = base + 32 * hf;
-            if (kb0 >= tile_kend) break;  // uniform
-            bf16x8 kf[2][DC];
+        for (int hb = 0; hb < 4; ++hb) {
+            const int krow = 32 * (hb >> 1) + 8 * (col >> 2) + 4 * (hb & 1) + (col & 3);
+            bf16x8 kf[DC];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int c = 0; c < DC; ++c) {
-                    const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
-                    kf[kb][c] = chan_ok
-                                    ? load16(&Ks[(32 * hf + 16 * kb + col) * K_LD + 32 * c + 8 * g])
-                                    : zero8();
-                }
-            bf16x8 p[PF_NQ];
+            for (int c = 0; c < DC; ++c) {
+                const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
+                kf[c] = chan_ok ? load16(&Ks[krow * K_LD + 32 * c + 8 * g]) : zero8();
+            }
 #pragma unroll
             for (int n = 0; n < PF_NQ; ++n) {
-                f32x4 s[2];
+                s[n][hb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    s[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                for (int c = 0; c < DC; ++c) s[n][hb] = mfma(kf[c], qf[n][c], s[n][hb]);
+            }
+        }
+        // ---- softmax of 64 keys per row ---------------------------------------------------
+        bf16x8 p[PF_NQ][2];
 #pragma unroll
-                    for (int c = 0; c < DC; ++c) s[kb] = mfma(kf[kb][c], qf[n][c], s[kb]);
-                }
-                unsigned ok[2];
+        for (int n = 0; n < PF_NQ; ++n) {
+            float x[16];
+#pragma unroll
+            for (int hb = 0; hb < 4; ++hb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) x[4 * hb + i] = s[n][hb][i];
+            if (need_mask) {
                 const int pos = r_pos[n];
                 const int wlo = (window > 0) ? pos - window + 1 : 0;
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    ok[kb] = 0;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int key = kb0 + 16 * kb + 4 * g + i;
-                        ok[kb] |= (key <= pos && key >= wlo) ? (1u << i) : 0u;
-                    }
+                for (int e = 0; e < 16; ++e) {
+                    const int key = base + 32 * (e >> 3) + 8 * g + (e & 7);
+                    if (!(key <= pos && key >= wlo)) x[e] = -INFINITY;
                 }
-                p[n] = softmax_step(s[0], s[1], ok[0], ok[1], scale_log2, m[n], l[n], acc[n]);
             }
+            float mx = x[0];
 #pragma unroll
-            for (int b = 0; b < DB; ++b) {
-                const bf16_t* vr = &Vs[(16 * b + col) * V_LD + 32 * hf + 4 * g];
-                const bf16x8 v = load8x2(vr, vr + 16);
+            for (int e = 1; e < 16; ++e) mx = fmaxf(mx, x[e]);
+            mx = row_max4(mx) * scale_log2;  // the scale is positive: max commutes with it
+            const float m_new = fmaxf(m[n], mx);
+            // a row that has seen no visible key yet keeps m = -inf; exp2 of (-inf) - 0 is 0
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+            if (__any(m_new > m[n])) {
+                const float alpha = __builtin_amdgcn_exp2f(m[n] - m_safe);
+                l[n] *= alpha;
 #pragma unroll
-                for (int n = 0; n < PF_NQ; ++n) acc[n][b] = mfma(v, p[n], acc[n][b]);
+                for (int b = 0; b < DB; ++b) {
+                    acc[n][b][0] *= alpha;
+                    acc[n][b][1] *= alpha;
+                    acc[n][b][2] *= alpha;
+                    acc[n][b][3] *= alpha;
+                }
+                m[n] = m_new;
+            }
+            float psum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float pe = __builtin_amdgcn_exp2f(fmaf(x[e], scale_log2, -m_safe));
+                psum += pe;
+                p[n][e >> 3][e & 7] = (__bf16)pe;
+            }
+            l[n] += psum;  // per-lane partial sum; the four groups are added at the end
+        }
+        // ---- O^T += V^T P^T -------------------------------------------------------------------
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const bf16x8 v = load16(&Vs[(16 * b + col) * V_LD + 32 * hf + 8 * g]);
+#pragma unroll
+                for (int n = 0; n < PF_NQ; ++n) acc[n][b] = mfma(v, p[n][hf], acc[n][b]);
             }
         }
     }

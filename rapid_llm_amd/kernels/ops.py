@@ -395,7 +395,7 @@ class AttentionPlan:
             self.tile_info = None
             return
         dec_tokens: list[int] = []
-        tiles: list[int] = []
+        tile_list: list[tuple[int, int, int, int]] = []
         self.max_decode_ctx = 0
         at = 0
         for start, n in zip(ctx.h_seq_starts, ctx.h_seq_lens):
@@ -404,8 +404,12 @@ class AttentionPlan:
                 self.max_decode_ctx = max(self.max_decode_ctx, start + 1)
             else:
                 for row0 in range(0, n * group, tile_rows):
-                    tiles += (at, start, n, row0)
+                    tile_list.append((at, start, n, row0))
             at += n
+        # tiles with the most keys first: workgroups are handed out in this order, and the
+        # short ones then fill the gaps the long ones leave
+        tile_list.sort(key=lambda t: -(t[1] + min(t[2], (t[3] + tile_rows) // group)))
+        tiles = [v for t in tile_list for v in t]
         self.num_decode = len(dec_tokens)
         self.num_tiles = len(tiles) // 4
         device = ctx.token_ids.device
