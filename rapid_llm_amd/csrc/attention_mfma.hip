@@ -443,7 +443,11 @@ extern "C" int rl_attn_decode(const void* q, const void* k_cache, const void* v_
 //
 // tile_info[4 * tile + {0,1,2,3}] = {first token of the request's portion in the flat batch,
 //   tokens of the request already in the cache, tokens in this portion, first row of the tile}
-__global__ __launch_bounds__(PF_WAVES* RL_WAVE) void attn_prefill_kernel(
+// Two waves per SIMD at most: the accumulators then live in ordinary vector registers, which
+// the rescale and the epilogue read directly (at the default budget of 128 the compiler parks
+// them in accumulation registers and moves them back and forth around every rescale).
+__global__ __launch_bounds__(PF_WAVES* RL_WAVE) __attribute__((amdgpu_waves_per_eu(1, 2))) void
+attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out,
     const int* __restrict__ tile_info, const int* __restrict__ token_slot,
@@ -509,29 +513,57 @@ __global__ __launch_bounds__(PF_WAVES* RL_WAVE) void attn_prefill_kernel(
         for (int b = 0; b < DB; ++b) acc[n][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
 
-    for (int base = tile_kstart & ~(PF_KEYS - 1); base < tile_kend; base += PF_KEYS) {
-        __syncthreads();  // the previous tile has been consumed
-        // ---- stage K: PF_THREADS / PF_KEYS threads share one key row -------------------
+    // The next tile's keys and values travel from memory into registers while this tile is
+    // multiplied; they reach LDS after the barrier that ends this tile's reads.
+    constexpr int TPK = PF_THREADS / PF_KEYS;  // threads sharing one key row
+    constexpr int KCH = (D / 8 + TPK - 1) / TPK;
+    constexpr int KG = PF_KEYS / 4;  // groups of four keys
+    constexpr int VCH = (D + PF_THREADS / KG - 1) / (PF_THREADS / KG);
+    uint4 kreg[KCH];
+    uint2 vreg[VCH];
+    auto stage_load = [&](int base) {
         {
-            constexpr int TPK = PF_THREADS / PF_KEYS;
             const int kk = tid / TPK;
             const int key = min(base + kk, seq_end - 1);  // clamped; masked by position below
             const int page = table[key / page_size];
             const bf16_t* krow =
                 k_cache + (((size_t)page * nkv + hk) * page_size + key % page_size) * D;
-            for (int ch = tid % TPK; ch < D / 8; ch += TPK)
-                *reinterpret_cast<uint4*>(&Ks[kk * K_LD + 8 * ch]) =
-                    *reinterpret_cast<const uint4*>(krow + 8 * ch);
+#pragma unroll
+            for (int i = 0; i < KCH; ++i) {
+                const int ch = tid % TPK + i * TPK;
+                if (ch < D / 8) kreg[i] = *reinterpret_cast<const uint4*>(krow + 8 * ch);
+            }
         }
-        // ---- stage V^T: thread -> (group of 4 keys, channel d, d + PF_THREADS / groups, ..) --
         {
-            constexpr int KG = PF_KEYS / 4;
             const int kg = tid % KG;
-            const int key = base + 4 * kg;
-            const int keyc = min(key, (seq_end - 1) & ~3);
+            const int keyc = min(base + 4 * kg, (seq_end - 1) & ~3);
             const int page = table[keyc / page_size];
             const bf16_t* vbase =
                 v_cache + (((size_t)page * nkv + hk) * D) * page_size + keyc % page_size;
+#pragma unroll
+            for (int i = 0; i < VCH; ++i) {
+                const int d = tid / KG + i * (PF_THREADS / KG);
+                if (d < D) vreg[i] = *reinterpret_cast<const uint2*>(vbase + (size_t)d * page_size);
+            }
+        }
+    };
+    auto stage_store = [&](int base) {
+        {
+            // key kk of the tile goes to the LDS row from which the first product reads it:
+            // row 32 hf + 16 kb + i holds key 32 hf + 8 (i / 4) + 4 kb + i % 4, so that the
+            // sixteen lanes of an operand read consecutive rows (no bank conflicts)
+            const int kk = tid / TPK;
+            const int r = kk & 31;
+            const int lrow = (kk & 32) + 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
+#pragma unroll
+            for (int i = 0; i < KCH; ++i) {
+                const int ch = tid % TPK + i * TPK;
+                if (ch < D / 8) *reinterpret_cast<uint4*>(&Ks[lrow * K_LD + 8 * ch]) = kreg[i];
+            }
+        }
+        {
+            const int kg = tid % KG;
+            const int key = base + 4 * kg;
             // keys of the group that may be multiplied: written ones (below seq_end) that no
             // row's window has left behind (their pages may have been given back already)
             const int lo_cut = tile_kstart - key;  // keys i < lo_cut are out
@@ -542,16 +574,28 @@ __global__ __launch_bounds__(PF_WAVES* RL_WAVE) void attn_prefill_kernel(
             if (1 >= lo_cut && 1 < hi_cut) keep_x |= 0xffff0000u;
             if (2 >= lo_cut && 2 < hi_cut) keep_y |= 0x0000ffffu;
             if (3 >= lo_cut && 3 < hi_cut) keep_y |= 0xffff0000u;
-            for (int d = tid / KG; d < D; d += PF_THREADS / KG) {
-                uint2 v = *reinterpret_cast<const uint2*>(vbase + (size_t)d * page_size);
-                if (!all_in) {
-                    v.x &= keep_x;
-                    v.y &= keep_y;
+#pragma unroll
+            for (int i = 0; i < VCH; ++i) {
+                const int d = tid / KG + i * (PF_THREADS / KG);
+                if (d < D) {
+                    uint2 v = vreg[i];
+                    if (!all_in) {
+                        v.x &= keep_x;
+                        v.y &= keep_y;
+                    }
+                    *reinterpret_cast<uint2*>(&Vs[d * V_LD + 4 * kg]) = v;
                 }
-                *reinterpret_cast<uint2*>(&Vs[d * V_LD + 4 * kg]) = v;
             }
         }
+    };
+
+    const int first_base = tile_kstart & ~(PF_KEYS - 1);
+    if (first_base < tile_kend) stage_load(first_base);
+    for (int base = first_base; base < tile_kend; base += PF_KEYS) {
+        __syncthreads();  // the previous tile has been consumed
+        stage_store(base);
         __syncthreads();
+        if (base + PF_KEYS < tile_kend) stage_load(base + PF_KEYS);
         if (base > wave_max_pos) continue;  // every key of the tile is ahead of this wave's rows
         // masks are needed where the diagonal or a window's edge crosses the tile
         const bool need_mask =
@@ -562,7 +606,7 @@ __global__ __launch_bounds__(PF_WAVES* RL_WAVE) void attn_prefill_kernel(
         f32x4 s[PF_NQ][4];
 #pragma unroll
         for (int hb = 0; hb < 4; ++hb) {
-            const int krow = 32 * (hb >> 1) + 8 * (col >> 2) + 4 * (hb & 1) + (col & 3);
+            const int krow = 16 * hb + col;  // see stage_store for the key it holds
             bf16x8 kf[DC];
 #pragma unroll
             for (int c = 0; c < DC; ++c) {

@@ -202,9 +202,11 @@ def attention_library(head_dim: int, force: bool = False) -> Path:
             f"the matrix-core attention kernels take head sizes in steps of 16 up to 256, "
             f"got {head_dim}"
         )
-    return compile_library(
-        f"attn_d{head_dim}", ATTENTION_SOURCES, (f"-DRL_HEAD_DIM={head_dim}",), force=force
-    )
+    # matrix instructions take their accumulators from ordinary vector registers: the softmax
+    # rescales them every step, and moving them to and from accumulation registers costs more
+    # vector instructions than the rescale itself
+    flags = (f"-DRL_HEAD_DIM={head_dim}", "-mllvm", "-amdgpu-mfma-vgpr-form=1")
+    return compile_library(f"attn_d{head_dim}", ATTENTION_SOURCES, flags, force=force)
 
 
 def build_all(head_dims: tuple[int, ...] = DEFAULT_HEAD_DIMS, force: bool = True) -> list[Path]:
