@@ -180,14 +180,36 @@ __device__ inline void decode_load(DecodeFrags& f, const bf16_t* __restrict__ k_
     }
 }
 
-template <bool V16>
+// What the fused variant needs beside the attention's own operands: the per-head norm
+// weights (null: no norm), the rotation tables (null: no rotation), and whether this layer
+// writes its keys and values.  `counters` (optional, one int per (request, kv head, chunk of
+// 16 heads), zero between launches) turns on the merge inside the kernel.
+struct DecodeExtra {
+    const float* q_norm_w;
+    const float* k_norm_w;
+    const float* cos_tab;
+    const float* sin_tab;
+    bf16_t* k_write;
+    bf16_t* v_write;
+    float eps;
+    int qkv_stride;  // elements between the rows of `q` (fused: the packed q|k|v row)
+    int* counters;
+};
+
+// FUSED: `q` holds raw packed [q | k | v] rows.  The workgroup norms and rotates the query
+// heads of its kv head itself (rapid_llm/models/base.py:134-140), and the workgroup whose
+// split holds the token's own position norms, rotates and writes the new key and value
+// before anyone reads them (rapid_llm/modules/attention.py:126-138), so that a decode step
+// needs no separate kernel for that.  Needs D % 64 == 0: a lane then holds both channels of
+// every rotation pair.
+template <bool V16, bool FUSED>
 __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const int* __restrict__ seq_token,
     const int* __restrict__ positions, const int* __restrict__ token_slot,
     const int* __restrict__ block_table, int table_stride, int page_size, int nq, int nkv,
-    int window, float scale_log2, int split_chunk, int nsplit) {
+    int window, float scale_log2, int split_chunk, int nsplit, DecodeExtra ex) {
     __shared__ float lds_o[2][D * 16];
     __shared__ float lds_m[2][16];
     __shared__ float lds_l[2][16];
@@ -215,126 +237,214 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
     const int hh = hc * 16 + col;  // head within the group
     const bool head_ok = hh < G;
     const int head = hk * G + (head_ok ? hh : 0);
-
-    if (lo >= hi) {
-        // nothing of this request falls into this split: tell the merge to skip it
-        if (nsplit > 1 && wave == 0 && g == 0 && head_ok) {
-            float* ml = part_ml + (((size_t)seq * nq + head) * nsplit + split) * 2;
-            ml[0] = -INFINITY;
-            ml[1] = 0.f;
-        }
-        return;
-    }
-    // page ids of the split, once: the loop's loads then depend on nothing but LDS
-    const int last_key = kend - 1;
-    const int page0 = lo / page_size;
-    {
-        const int npages = last_key / page_size - page0 + 1;  // <= DEC_MAX_PAGES + 1 (host)
-        for (int i = threadIdx.x; i < npages && i < DEC_MAX_PAGES + 2; i += DEC_WAVES * RL_WAVE)
-            lds_pages[i] = table[page0 + i];
-    }
-    // Q^T as B operand: lane (row col, group g) holds channels 32c + 8g .. + 7
-    bf16x8 qf[DC];
-    {
-        const bf16_t* qrow = q + ((size_t)t * nq + head) * D;
-#pragma unroll
-        for (int c = 0; c < DC; ++c) {
-            const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
-            qf[c] = (head_ok && chan_ok) ? load16(qrow + 32 * c + 8 * g) : zero8();
-        }
-    }
-    __syncthreads();
+    const size_t slot_index = ((size_t)seq * nq + head) * nsplit + split;
 
     float m = -INFINITY, l = 0.f;
     f32x4 acc[DB];
 #pragma unroll
     for (int b = 0; b < DB; ++b) acc[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // the loads of the next step are issued before this step's arithmetic
-    DecodeFrags cur, nxt;
-    int base = lo + 32 * wave;
-    if (base < hi)
-        decode_load<V16>(cur, k_cache, v_cache, lds_pages, page0, page_size, nkv, hk, base,
-                         last_key, col, g);
-    for (; base < hi; base += 32 * DEC_WAVES) {
-        const int next = base + 32 * DEC_WAVES;
-        if (next < hi)
-            decode_load<V16>(nxt, k_cache, v_cache, lds_pages, page0, page_size, nkv, hk, next,
-                             last_key, col, g);
-        // ---- S^T = K Q^T for two blocks of 16 keys --------------------------------
-        f32x4 s[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            s[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int c = 0; c < DC; ++c) s[kb] = mfma(cur.k[kb][c], qf[c], s[kb]);
+    if (lo < hi) {  // the same for every thread of the workgroup
+        // page ids of the split, once: the loop's loads then depend on nothing but LDS
+        const int last_key = kend - 1;
+        const int page0 = lo / page_size;
+        {
+            const int npages = last_key / page_size - page0 + 1;
+            for (int i = threadIdx.x; i < npages && i < DEC_MAX_PAGES + 2; i += DEC_WAVES * RL_WAVE)
+                lds_pages[i] = table[page0 + i];
         }
-        // ---- which of this lane's keys (base + 8g + 4kb + i) are visible ------------
-        unsigned ok[2];
+        const bf16_t* qrow = q + (size_t)t * ex.qkv_stride + (size_t)head * D;
+        // Q^T as B operand: lane (row col, group g) holds channels 32c + 8g .. + 7
+        bf16x8 qf[DC];
+        if (FUSED) {
+            float x[DC][8];
+            float ss = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            ok[kb] = 0;
+            for (int c = 0; c < DC; ++c) {
+                const bf16x8 raw = head_ok ? load16(qrow + 32 * c + 8 * g) : zero8();
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = base + 8 * g + 4 * kb + i;
-                ok[kb] |= (key >= kstart && key < kend) ? (1u << i) : 0u;
-            }
-        }
-        const bf16x8 p = softmax_step(s[0], s[1], ok[0], ok[1], scale_log2, m, l, acc);
-        // ---- O^T += V^T P^T ---------------------------------------------------------
-        const bool partial = (base + 32 > kend) || (base < kstart);
-#pragma unroll
-        for (int b = 0; b < DB; ++b) {
-            bf16x8 v = cur.v[b];
-            if (partial) {
-                // 0 * stale data must be 0: a page used before may hold anything
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    if (!((ok[0] >> i) & 1u)) v[i] = (__bf16)0.f;
-                    if (!((ok[1] >> i) & 1u)) v[4 + i] = (__bf16)0.f;
+                for (int j = 0; j < 8; ++j) {
+                    x[c][j] = (float)raw[j];
+                    ss += x[c][j] * x[c][j];
                 }
             }
-            acc[b] = mfma(v, p, acc[b]);
+            if (ex.q_norm_w) {
+                const float rrms = rsqrtf(row_sum4(ss) / (float)D + ex.eps);
+#pragma unroll
+                for (int c = 0; c < DC; ++c)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) x[c][j] *= rrms * ex.q_norm_w[32 * c + 8 * g + j];
+            }
+            if (ex.cos_tab) {
+                constexpr int HC = DC / 2;  // chunk c pairs with chunk c + HC, same lane and slot
+#pragma unroll
+                for (int c = 0; c < HC; ++c)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int i = 32 * c + 8 * g + j;
+                        const float cs = ex.cos_tab[(size_t)pos * (D / 2) + i];
+                        const float sn = ex.sin_tab[(size_t)pos * (D / 2) + i];
+                        const float a = x[c][j], bb = x[c + HC][j];
+                        x[c][j] = a * cs - bb * sn;
+                        x[c + HC][j] = bb * cs + a * sn;
+                    }
+            }
+#pragma unroll
+            for (int c = 0; c < DC; ++c)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) qf[c][j] = (__bf16)x[c][j];
+            // the token's own key and value: written by the split that holds its position
+            // (with more than 16 heads on a kv head every chunk of heads writes the same bytes:
+            // each reads them back after its own barrier only)
+            if (ex.k_write && pos >= lo && pos < hi) {
+                const size_t page = (size_t)table[pos / page_size];
+                const int off = pos % page_size;
+                const bf16_t* krow = q + (size_t)t * ex.qkv_stride + (size_t)(nq + hk) * D;
+                const bf16_t* vrow = q + (size_t)t * ex.qkv_stride + (size_t)(nq + nkv + hk) * D;
+                if (wave == 0) {
+                    // lane handles the pairs (i, i + D/2) for i = lane, lane + 64
+                    constexpr int half = D / 2;
+                    float x1[2], x2[2];
+                    float ks = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 2; ++r) {
+                        const int i = lane + r * RL_WAVE;
+                        x1[r] = x2[r] = 0.f;
+                        if (i < half) {
+                            x1[r] = bf16_to_float(krow[i]);
+                            x2[r] = bf16_to_float(krow[i + half]);
+                            ks += x1[r] * x1[r] + x2[r] * x2[r];
+                        }
+                    }
+                    float rrms = 1.f;
+                    if (ex.k_norm_w) rrms = rsqrtf(wave_sum(ks) / (float)D + ex.eps);
+                    bf16_t* dst = ex.k_write + ((page * nkv + hk) * page_size + off) * D;
+#pragma unroll
+                    for (int r = 0; r < 2; ++r) {
+                        const int i = lane + r * RL_WAVE;
+                        if (i < half) {
+                            float a = x1[r], bb = x2[r];
+                            if (ex.k_norm_w) {
+                                a = a * rrms * ex.k_norm_w[i];
+                                bb = bb * rrms * ex.k_norm_w[i + half];
+                            }
+                            if (ex.cos_tab) {
+                                const float cs = ex.cos_tab[(size_t)pos * half + i];
+                                const float sn = ex.sin_tab[(size_t)pos * half + i];
+                                const float ra = a * cs - bb * sn;
+                                bb = bb * cs + a * sn;
+                                a = ra;
+                            }
+                            dst[i] = float_to_bf16(a);
+                            dst[i + half] = float_to_bf16(bb);
+                        }
+                    }
+                } else if (wave == 1) {
+                    bf16_t* dst = ex.v_write + ((page * nkv + hk) * D) * page_size + off;
+                    for (int i = lane; i < D; i += RL_WAVE) dst[(size_t)i * page_size] = vrow[i];
+                }
+                __threadfence_block();  // the loop below reads them back from the cache
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < DC; ++c) {
+                const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
+                qf[c] = (head_ok && chan_ok) ? load16(qrow + 32 * c + 8 * g) : zero8();
+            }
         }
-        cur = nxt;
-    }
+        __syncthreads();
 
-    // ---- combine the waves: (2,3) -> (0,1), then 1 -> 0, in the accumulators' own layout ----
-    l = row_sum4(l);
-    auto put = [&](int slot) {
-        if (g == 0) {
-            lds_m[slot][col] = m;
-            lds_l[slot][col] = l;
+        // the loads of the next step are issued before this step's arithmetic
+        DecodeFrags cur, nxt;
+        int base = lo + 32 * wave;
+        if (base < hi)
+            decode_load<V16>(cur, k_cache, v_cache, lds_pages, page0, page_size, nkv, hk, base,
+                             last_key, col, g);
+        for (; base < hi; base += 32 * DEC_WAVES) {
+            const int next = base + 32 * DEC_WAVES;
+            if (next < hi)
+                decode_load<V16>(nxt, k_cache, v_cache, lds_pages, page0, page_size, nkv, hk, next,
+                                 last_key, col, g);
+            // ---- S^T = K Q^T for two blocks of 16 keys --------------------------------
+            f32x4 s[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                s[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < DC; ++c) s[kb] = mfma(cur.k[kb][c], qf[c], s[kb]);
+            }
+            // ---- which of this lane's keys (base + 8g + 4kb + i) are visible ------------
+            unsigned ok[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                ok[kb] = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = base + 8 * g + 4 * kb + i;
+                    ok[kb] |= (key >= kstart && key < kend) ? (1u << i) : 0u;
+                }
+            }
+            const bf16x8 p = softmax_step(s[0], s[1], ok[0], ok[1], scale_log2, m, l, acc);
+            // ---- O^T += V^T P^T ---------------------------------------------------------
+            const bool partial = (base + 32 > kend) || (base < kstart);
+#pragma unroll
+            for (int b = 0; b < DB; ++b) {
+                bf16x8 v = cur.v[b];
+                if (partial) {
+                    // 0 * stale data must be 0: a page used before may hold anything
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        if (!((ok[0] >> i) & 1u)) v[i] = (__bf16)0.f;
+                        if (!((ok[1] >> i) & 1u)) v[4 + i] = (__bf16)0.f;
+                    }
+                }
+                acc[b] = mfma(v, p, acc[b]);
+            }
+            cur = nxt;
         }
+
+        // ---- combine the waves: (2,3) -> (0,1), then 1 -> 0, in the accumulators' own layout --
+        l = row_sum4(l);
+        auto put = [&](int slot) {
+            if (g == 0) {
+                lds_m[slot][col] = m;
+                lds_l[slot][col] = l;
+            }
 #pragma unroll
-        for (int b = 0; b < DB; ++b)
+            for (int b = 0; b < DB; ++b)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) lds_o[slot][(16 * b + 4 * g + i) * 16 + col] = acc[b][i];
-    };
-    auto take = [&](int slot) {
-        const float m_o = lds_m[slot][col], l_o = lds_l[slot][col];
-        const float mm = fmaxf(m, m_o);
-        const float ms = (mm == -INFINITY) ? 0.f : mm;  // a wave without keys has m = -inf
-        const float f1 = exp2f(m - ms), f2 = exp2f(m_o - ms);
+                for (int i = 0; i < 4; ++i)
+                    lds_o[slot][(16 * b + 4 * g + i) * 16 + col] = acc[b][i];
+        };
+        auto take = [&](int slot) {
+            const float m_o = lds_m[slot][col], l_o = lds_l[slot][col];
+            const float mm = fmaxf(m, m_o);
+            const float ms = (mm == -INFINITY) ? 0.f : mm;  // a wave without keys has m = -inf
+            const float f1 = exp2f(m - ms), f2 = exp2f(m_o - ms);
 #pragma unroll
-        for (int b = 0; b < DB; ++b)
+            for (int b = 0; b < DB; ++b)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                acc[b][i] = acc[b][i] * f1 + lds_o[slot][(16 * b + 4 * g + i) * 16 + col] * f2;
-        l = l * f1 + l_o * f2;
-        m = mm;
-    };
-    if (wave >= 2) put(wave - 2);
-    __syncthreads();
-    if (wave < 2) take(wave);
-    __syncthreads();
-    if (wave == 1) put(0);
-    __syncthreads();
-    if (wave != 0) return;
-    take(0);
-    if (!head_ok) return;
+                for (int i = 0; i < 4; ++i)
+                    acc[b][i] =
+                        acc[b][i] * f1 + lds_o[slot][(16 * b + 4 * g + i) * 16 + col] * f2;
+            l = l * f1 + l_o * f2;
+            m = mm;
+        };
+        if (wave >= 2) put(wave - 2);
+        __syncthreads();
+        if (wave < 2) take(wave);
+        __syncthreads();
+        if (wave == 1) put(0);
+        __syncthreads();
+        if (wave != 0) return;
+        take(0);
+    } else if (wave != 0) {
+        return;
+    }
+    // ---- wave 0: this split's result (m = -inf, l = 0 if the split holds no key) -------------
     const float inv = l > 0.f ? 1.f / l : 0.f;
     if (nsplit == 1) {
+        if (!head_ok) return;
         bf16_t* orow = out + ((size_t)t * nq + head) * D;
 #pragma unroll
         for (int b = 0; b < DB; ++b) {
@@ -345,17 +455,64 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
             for (int i = 0; i < 4; ++i) o.v[i] = float_to_bf16(acc[b][i] * inv);
             *reinterpret_cast<uint2*>(orow + 16 * b + 4 * g) = __builtin_bit_cast(uint2, o);
         }
-    } else {
-        const size_t slot = ((size_t)seq * nq + head) * nsplit + split;
-        float* orow = part_o + slot * D;
+        return;
+    }
+    if (head_ok) {
+        float* orow = part_o + slot_index * D;
+        if (l > 0.f) {
 #pragma unroll
-        for (int b = 0; b < DB; ++b)
-            *reinterpret_cast<float4*>(orow + 16 * b + 4 * g) =
-                make_float4(acc[b][0] * inv, acc[b][1] * inv, acc[b][2] * inv, acc[b][3] * inv);
-        if (g == 0) {
-            part_ml[slot * 2] = m;
-            part_ml[slot * 2 + 1] = l;
+            for (int b = 0; b < DB; ++b)
+                *reinterpret_cast<float4*>(orow + 16 * b + 4 * g) = make_float4(
+                    acc[b][0] * inv, acc[b][1] * inv, acc[b][2] * inv, acc[b][3] * inv);
         }
+        if (g == 0) {
+            part_ml[slot_index * 2] = m;
+            part_ml[slot_index * 2 + 1] = l;
+        }
+    }
+    if (!ex.counters) return;  // a separate kernel merges
+    // ---- the split that finishes last merges them all, in the order of the splits ------------
+    __threadfence();
+    int ticket = 0;
+    int* counter = ex.counters + (size_t)seq * gridDim.y + blockIdx.y;
+    if (lane == 0) ticket = atomicAdd(counter, 1);
+    ticket = __shfl(ticket, 0, RL_WAVE);
+    if (ticket != nsplit - 1) return;
+    __threadfence();
+    if (lane == 0) *counter = 0;  // ready for the next launch
+    if (!head_ok) return;
+    const size_t slot0 = ((size_t)seq * nq + head) * nsplit;
+    float mm = -INFINITY;
+    for (int sp = 0; sp < nsplit; ++sp) mm = fmaxf(mm, part_ml[(slot0 + sp) * 2]);
+    float wsum = 0.f;
+    f32x4 o[DB];
+#pragma unroll
+    for (int b = 0; b < DB; ++b) o[b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < nsplit; ++sp) {
+        const float ms = part_ml[(slot0 + sp) * 2];
+        if (ms == -INFINITY) continue;  // an empty split wrote no output
+        const float w = part_ml[(slot0 + sp) * 2 + 1] * exp2f(ms - mm);
+        wsum += w;
+        const float* prow = part_o + (slot0 + sp) * D;
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+            const float4 v = *reinterpret_cast<const float4*>(prow + 16 * b + 4 * g);
+            o[b][0] += v.x * w;
+            o[b][1] += v.y * w;
+            o[b][2] += v.z * w;
+            o[b][3] += v.w * w;
+        }
+    }
+    const float winv = wsum > 0.f ? 1.f / wsum : 0.f;
+    bf16_t* orow = out + ((size_t)t * nq + head) * D;
+#pragma unroll
+    for (int b = 0; b < DB; ++b) {
+        struct {
+            bf16_t v[4];
+        } r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r.v[i] = float_to_bf16(o[b][i] * winv);
+        *reinterpret_cast<uint2*>(orow + 16 * b + 4 * g) = __builtin_bit_cast(uint2, r);
     }
 }
 
@@ -386,12 +543,19 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o,
 
 extern "C" int rl_attn_head_dim() { return D; }
 
+// `counters`: null, or zeroed ints, one per (request, kv head, chunk of 16 heads): the merge
+// then runs inside the decode kernel (the counters are zero again when it ends; launches that
+// share them must not overlap).  Fused form (`fused` != 0): `q` is the packed [q | k | v]
+// row, norm weights and rotation tables may be null, `k_write` / `v_write` null for a layer
+// that writes no cache.
 extern "C" int rl_attn_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
-                              float* part_o, float* part_ml, const int* seq_token,
+                              float* part_o, float* part_ml, int* counters, const int* seq_token,
                               const int* positions, const int* token_slot,
                               const int* block_table, int table_stride, int page_size,
                               int num_seqs, int nq, int nkv, int window, float scale,
-                              int split_chunk, int nsplit, hipStream_t stream) {
+                              int split_chunk, int nsplit, int fused, const float* q_norm_w,
+                              const float* k_norm_w, const float* cos_tab, const float* sin_tab,
+                              void* k_write, void* v_write, float eps, hipStream_t stream) {
     if (num_seqs <= 0) return RL_OK;
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || split_chunk < 32 ||
         split_chunk % 32 || nsplit < 1 || nsplit > 65535)
@@ -399,28 +563,51 @@ extern "C" int rl_attn_decode(const void* q, const void* k_cache, const void* v_
     // a split's pages are staged in LDS (its keys may start up to 31 before a page's first)
     if ((split_chunk + 31) / page_size + 1 > DEC_MAX_PAGES) return RL_ERR_ARG;
     if (nsplit > 1 && (!part_o || !part_ml)) return RL_ERR_ARG;
+    if (fused && (D % 64 != 0 || (cos_tab && !sin_tab) || (k_write && !v_write))) return RL_ERR_ARG;
     const int G = nq / nkv;
     const int head_chunks = (G + 15) / 16;
     if ((long)nkv * head_chunks > 65535) return RL_ERR_ARG;
     const float scale_log2 = scale * 1.4426950408889634f;
+    DecodeExtra ex;
+    ex.q_norm_w = fused ? q_norm_w : nullptr;
+    ex.k_norm_w = fused ? k_norm_w : nullptr;
+    ex.cos_tab = fused ? cos_tab : nullptr;
+    ex.sin_tab = fused ? sin_tab : nullptr;
+    ex.k_write = fused ? (bf16_t*)k_write : nullptr;
+    ex.v_write = fused ? (bf16_t*)v_write : nullptr;
+    ex.eps = eps;
+    ex.qkv_stride = fused ? (nq + 2 * nkv) * D : nq * D;
+    ex.counters = nsplit > 1 ? counters : nullptr;
     dim3 grid(num_seqs, nkv * head_chunks, nsplit), block(DEC_WAVES * RL_WAVE);
-    if (page_size % 8 == 0)
-        hipLaunchKernelGGL(attn_decode_kernel<true>, grid, block, 0, stream, (const bf16_t*)q,
-                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_o,
-                           part_ml, seq_token, positions, token_slot, block_table, table_stride,
-                           page_size, nq, nkv, window, scale_log2, split_chunk, nsplit);
-    else
-        hipLaunchKernelGGL(attn_decode_kernel<false>, grid, block, 0, stream, (const bf16_t*)q,
-                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, part_o,
-                           part_ml, seq_token, positions, token_slot, block_table, table_stride,
-                           page_size, nq, nkv, window, scale_log2, split_chunk, nsplit);
+#define RL_DECODE(V16, FUSED)                                                                  \
+    hipLaunchKernelGGL((attn_decode_kernel<V16, FUSED>), grid, block, 0, stream,               \
+                       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,       \
+                       (bf16_t*)out, part_o, part_ml, seq_token, positions, token_slot,        \
+                       block_table, table_stride, page_size, nq, nkv, window, scale_log2,      \
+                       split_chunk, nsplit, ex)
+    if (fused) {
+        if constexpr (D % 64 == 0) {
+            if (page_size % 8 == 0)
+                RL_DECODE(true, true);
+            else
+                RL_DECODE(false, true);
+        }
+    } else {
+        if (page_size % 8 == 0)
+            RL_DECODE(true, false);
+        else
+            RL_DECODE(false, false);
+    }
+#undef RL_DECODE
     if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
-    if (nsplit > 1) {
+    if (nsplit > 1 && !ex.counters) {
         hipLaunchKernelGGL(attn_merge_kernel, dim3(num_seqs, nq), dim3(D < 64 ? 64 : D), 0,
                            stream, part_o, part_ml, (bf16_t*)out, seq_token, nq, nsplit);
     }
     return rl_launch_status();
 }
+
+extern "C" int rl_attn_decode_fusable() { return D % 64 == 0 ? 1 : 0; }
 
 // =========================================================================== //
 // prefill

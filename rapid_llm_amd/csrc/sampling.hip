@@ -42,9 +42,97 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict_
     }
 }
 
-extern "C" int rl_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+// Wide rows in two stages, so that a handful of rows still fills the chip: stage one finds
+// the best (value, index) of each slice of a row, stage two the best of the slices.  Ties
+// keep the lower index in both, so the result is the one-stage kernel's.
+#define ARGMAX_SLICE 4096
+
+__global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restrict__ logits,
+                                                           float* __restrict__ part_v,
+                                                           int* __restrict__ part_i, int vocab,
+                                                           int slices) {
+    __shared__ float best_v[4];
+    __shared__ int best_i[4];
+    const float* row = logits + (size_t)blockIdx.y * vocab;
+    const int lo = blockIdx.x * ARGMAX_SLICE;
+    const int hi = min(vocab, lo + ARGMAX_SLICE);
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+        const float v = row[i];
+        if (v > bv || (v == bv && i < bi)) {
+            bv = v;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = RL_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, RL_WAVE);
+        const int oi = __shfl_xor(bi, off, RL_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    const int lane = threadIdx.x & (RL_WAVE - 1), wave = threadIdx.x / RL_WAVE;
+    if (lane == 0) {
+        best_v[wave] = bv;
+        best_i[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+                bv = best_v[w];
+                bi = best_i[w];
+            }
+        part_v[(size_t)blockIdx.y * slices + blockIdx.x] = bv;
+        part_i[(size_t)blockIdx.y * slices + blockIdx.x] = bi;
+    }
+}
+
+__global__ __launch_bounds__(RL_WAVE) void argmax_merge_kernel(const float* __restrict__ part_v,
+                                                              const int* __restrict__ part_i,
+                                                              int* __restrict__ out, int slices) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int s = threadIdx.x; s < slices; s += RL_WAVE) {
+        const float v = part_v[(size_t)blockIdx.x * slices + s];
+        const int i = part_i[(size_t)blockIdx.x * slices + s];
+        if (v > bv || (v == bv && i < bi)) {
+            bv = v;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = RL_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, RL_WAVE);
+        const int oi = __shfl_xor(bi, off, RL_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+}
+
+extern "C" int rl_argmax_slices(int vocab) { return (vocab + ARGMAX_SLICE - 1) / ARGMAX_SLICE; }
+
+// part_v / part_i: [rows, rl_argmax_slices(vocab)] scratch of the caller; without it (null)
+// the one-stage kernel runs.
+extern "C" int rl_argmax(const float* logits, int* out, float* part_v, int* part_i, int rows,
+                         int vocab, hipStream_t stream) {
     if (rows <= 0) return RL_OK;
     if (vocab < 1) return RL_ERR_ARG;
+    const int slices = (vocab + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
+    if (part_v && part_i && slices > 1 && rows <= 65535) {
+        hipLaunchKernelGGL(argmax_slices_kernel, dim3(slices, rows), dim3(256), 0, stream, logits,
+                           part_v, part_i, vocab, slices);
+        if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
+        hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(RL_WAVE), 0, stream, part_v,
+                           part_i, out, slices);
+        return rl_launch_status();
+    }
     hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, stream, logits, out, vocab);
     return rl_launch_status();
 }

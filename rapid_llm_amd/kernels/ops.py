@@ -279,7 +279,13 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     rows, vocab = logits.shape
     _need(logits, "logits", torch.float32)
     _need(out, "out", torch.int32, (rows,))
-    _ok(core().rl_argmax(_p(logits), _p(out), rows, vocab, _stream()), "rl_argmax")
+    lib = core()
+    slices = lib.rl_argmax_slices(vocab)
+    part_v = part_i = None
+    if slices > 1 and rows * 4 < slices * 16:  # few wide rows: two stages fill the chip
+        part_v = torch.empty((rows, slices), dtype=torch.float32, device=logits.device)
+        part_i = torch.empty((rows, slices), dtype=torch.int32, device=logits.device)
+    _ok(lib.rl_argmax(_p(logits), _p(out), _p(part_v), _p(part_i), rows, vocab, _stream()), "rl_argmax")
 
 
 def sample(
@@ -466,11 +472,7 @@ def paged_attention(
         )
     lib = attention_lib(d)
     group = nq // nkv
-    key = ("attention_plan", group)
-    plan = ctx.extra.get(key)
-    if plan is None:
-        plan = AttentionPlan(ctx, group, lib.rl_attn_prefill_rows())
-        ctx.extra[key] = plan
+    plan = attention_plan(ctx, group, d)
     if plan.num_tiles:
         _ok(
             lib.rl_attn_prefill(
@@ -481,25 +483,135 @@ def paged_attention(
             "rl_attn_prefill",
         )
     if plan.num_decode:
-        # under a graph the split is laid out for the longest context the engine allows
-        span = ctx.extra.get("context_bound", plan.max_decode_ctx)
-        if window > 0:
-            span = min(span, window + 31)
-        pairs = plan.num_decode * nkv * ((group + 15) // 16)
-        want = max(1, _TARGET_BLOCKS // pairs)
-        chunk = max(_MIN_SPLIT_KEYS, -(-(-(-span // want)) // 128) * 128)
-        chunk = min(chunk, max(32, ((_MAX_SPLIT_PAGES - 1) * page_size - 31) // 32 * 32))
-        nsplit = -(-span // chunk)
-        part_o = part_ml = None
-        if nsplit > 1:
-            part_o = torch.empty((plan.num_decode, nq, nsplit, d), dtype=torch.float32, device=q.device)
-            part_ml = torch.empty((plan.num_decode, nq, nsplit, 2), dtype=torch.float32, device=q.device)
-        _ok(
-            lib.rl_attn_decode(
-                _p(q), _p(k_cache), _p(v_cache), _p(out), _p(part_o), _p(part_ml),
-                _p(plan.seq_token), _p(ctx.positions), _p(ctx.token_slot), _p(block_table),
-                block_table.stride(0), page_size, plan.num_decode, nq, nkv, window,
-                ctypes.c_float(scale), chunk, nsplit, _stream(),
-            ),
-            "rl_attn_decode",
+        _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_size, nq, nkv, d,
+                       window, scale, None)
+
+
+def attention_plan(ctx, group: int, d: int) -> AttentionPlan:
+    """The step's launch data for one group size, made once and kept with the step."""
+    key = ("attention_plan", group)
+    plan = ctx.extra.get(key)
+    if plan is None:
+        plan = AttentionPlan(ctx, group, attention_lib(d).rl_attn_prefill_rows())
+        ctx.extra[key] = plan
+    return plan
+
+
+_MERGE_COUNTERS: dict[torch.device, torch.Tensor] = {}
+_NUM_MERGE_COUNTERS = 1 << 16
+
+
+def _merge_counters(device: torch.device) -> torch.Tensor:
+    """Zeroed ints the decode kernel's in-kernel merge counts finished splits with.  Every
+    launch leaves them zero again, so one buffer per device serves all layers of a stream."""
+    buf = _MERGE_COUNTERS.get(device)
+    if buf is None:
+        buf = torch.zeros(_NUM_MERGE_COUNTERS, dtype=torch.int32, device=device)
+        _MERGE_COUNTERS[device] = buf
+    return buf
+
+
+def _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_size, nq, nkv, d,
+                   window, scale, fused) -> None:
+    """Split-key decode attention of the step's single tokens.  ``fused`` is ``None`` (``q``
+    holds finished queries) or ``(q_norm_w, k_norm_w, cos, sin, k_write, v_write, eps)`` with
+    ``q`` the packed [q | k | v] rows."""
+    group = nq // nkv
+    # under a graph the split is laid out for the longest context of the graph's bucket
+    span = ctx.extra.get("context_bound", plan.max_decode_ctx)
+    if window > 0:
+        span = min(span, window + 31)
+    chunks = (group + 15) // 16
+    pairs = plan.num_decode * nkv * chunks
+    want = max(1, _TARGET_BLOCKS // pairs)
+    chunk = max(_MIN_SPLIT_KEYS, -(-(-(-span // want)) // 128) * 128)
+    chunk = min(chunk, max(32, ((_MAX_SPLIT_PAGES - 1) * page_size - 31) // 32 * 32))
+    nsplit = -(-span // chunk)
+    part_o = part_ml = counters = None
+    if nsplit > 1:
+        part_o = torch.empty((plan.num_decode, nq, nsplit, d), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((plan.num_decode, nq, nsplit, 2), dtype=torch.float32, device=q.device)
+        if pairs <= _NUM_MERGE_COUNTERS:
+            counters = _merge_counters(q.device)
+    qn = kn = cos = sin = kw = vw = None
+    eps = 0.0
+    if fused is not None:
+        qn, kn, cos, sin, kw, vw, eps = fused
+    _ok(
+        lib.rl_attn_decode(
+            _p(q), _p(k_cache), _p(v_cache), _p(out), _p(part_o), _p(part_ml), _p(counters),
+            _p(plan.seq_token), _p(ctx.positions), _p(ctx.token_slot), _p(block_table),
+            block_table.stride(0), page_size, plan.num_decode, nq, nkv, window,
+            ctypes.c_float(scale), chunk, nsplit, int(fused is not None), _p(qn), _p(kn), _p(cos),
+            _p(sin), _p(kw), _p(vw), ctypes.c_float(eps), _stream(),
+        ),
+        "rl_attn_decode",
+    )
+
+
+def decode_attention_fusable(ctx, x_dtype: torch.dtype, group: int, d: int, rotary_half: int) -> bool:
+    """Whether the step is one the fused decode kernel takes: bfloat16, single tokens only,
+    a head size whose rotation pairs stay within a lane, rotation over the whole head or none."""
+    if x_dtype != torch.bfloat16 or d % 64 or rotary_half not in (0, d // 2):
+        return False
+    plan = attention_plan(ctx, group, d)
+    return plan.num_tiles == 0 and plan.num_decode > 0
+
+
+def decode_attention_fused(
+    qkv: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    out: torch.Tensor,
+    ctx,
+    block_table: torch.Tensor,
+    page_size: int,
+    nq: int,
+    nkv: int,
+    d: int,
+    window: int,
+    scale: float,
+    q_norm_w: Optional[torch.Tensor],
+    k_norm_w: Optional[torch.Tensor],
+    cos: Optional[torch.Tensor],
+    sin: Optional[torch.Tensor],
+    eps: float,
+    write_cache: bool,
+) -> None:
+    """Per-head norm, rotation, cache write and split-key attention of a step of single
+    tokens in one kernel (the merge of the splits included).  Same result as
+    ``qknorm_rope_kvwrite`` followed by ``paged_attention`` up to rounding."""
+    tokens = qkv.shape[0]
+    pages = k_cache.shape[0]
+    _need(qkv, "qkv", torch.bfloat16, (tokens, (nq + 2 * nkv) * d))
+    _need(out, "out", torch.bfloat16, (tokens, nq * d))
+    _need(k_cache, "k_cache", torch.bfloat16, (pages, nkv, page_size, d))
+    _need(v_cache, "v_cache", torch.bfloat16, (pages, nkv, d, page_size))
+    _need(block_table, "block_table", torch.int32)
+    if page_size % 4:
+        raise KernelError(f"the matrix-core attention kernels need a page size that is a multiple of 4, got {page_size}")
+    if ctx.max_position // page_size >= block_table.shape[1]:
+        raise KernelError(
+            f"position {ctx.max_position} needs page {ctx.max_position // page_size} of a block "
+            f"table with {block_table.shape[1]} columns"
         )
+    for w, name in ((q_norm_w, "q_norm weight"), (k_norm_w, "k_norm weight")):
+        if w is not None:
+            _need(w, name, torch.float32, (d,))
+    if cos is not None:
+        _need(cos, "cos table", torch.float32, (None, d // 2))
+        _need(sin, "sin table", torch.float32, tuple(cos.shape))
+        if ctx.max_position >= cos.shape[0]:
+            raise KernelError(
+                f"position {ctx.max_position} is beyond the rotation table of {cos.shape[0]} positions"
+            )
+    lib = attention_lib(d)
+    if not lib.rl_attn_decode_fusable():
+        raise KernelError(f"the fused decode kernel needs a head size that is a multiple of 64, got {d}")
+    plan = attention_plan(ctx, nq // nkv, d)
+    if plan.num_tiles or plan.num_decode != tokens:
+        raise KernelError("the fused decode kernel takes steps of single tokens only")
+    fused = (q_norm_w, k_norm_w, cos, sin, k_cache if write_cache else None,
+             v_cache if write_cache else None, eps)
+    _decode_launch(lib, plan, ctx, qkv, k_cache, v_cache, out, block_table, page_size, nq, nkv, d,
+                   window, scale, fused)

@@ -96,22 +96,29 @@ class GQAAttention(Mixer):
     def forward(self, x, ctx, cache):
         tokens = x.shape[0]
         qkv = self.qkv(x)
-        q = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         table = ctx.block_tables[cache.group_id]
         pos_enc = self.position
+        cos = pos_enc.cos if pos_enc is not None else None
+        sin = pos_enc.sin if pos_enc is not None else None
+        eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
+        out = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
+        rotary_half = cos.shape[1] if cos is not None else 0
+        if ops.decode_attention_fusable(ctx, qkv.dtype, self.nq // self.nkv, self.d, rotary_half):
+            # a step of single tokens: norm, rotation, cache write and attention in one kernel
+            ops.decode_attention_fused(
+                qkv, cache.k, cache.v, out, ctx, table, cache.page_size, self.nq, self.nkv, self.d,
+                self.window, self.scale, self.q_norm_w, self.k_norm_w, cos, sin, eps, cache.owns_pages,
+            )
+            return self.o(out)
+        q = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         ops.qknorm_rope_kvwrite(
             qkv, q,
             cache.k if cache.owns_pages else None,
             cache.v if cache.owns_pages else None,
-            self.q_norm_w, self.k_norm_w,
-            pos_enc.cos if pos_enc is not None else None,
-            pos_enc.sin if pos_enc is not None else None,
+            self.q_norm_w, self.k_norm_w, cos, sin,
             ctx.positions, ctx.token_slot, table, cache.page_size,
-            self.nq, self.nkv, self.d,
-            self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
-            ctx.max_position,
+            self.nq, self.nkv, self.d, eps, ctx.max_position,
         )
-        out = torch.empty_like(q)
         ops.paged_attention(
             q, cache.k, cache.v, out, ctx, table, cache.page_size,
             self.nq, self.nkv, self.d, self.window, self.scale,

@@ -96,7 +96,7 @@ def test_eviction_changes_nothing(tmp_path):
     assert tight.scheduler.cache.num_free_pages() == 23
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_bfloat16_generation_stays_near_the_plain_choice(tmp_path, which):
     from rapid_llm_amd import SamplingParams
 

@@ -310,3 +310,95 @@ def test_embed_and_argmax():
     ops.argmax(logits.to(DEV), out)
     assert out.cpu().tolist() == logits.argmax(-1).tolist()
     assert int(out[3]) == 777
+
+
+FUSED_CASES = [
+    # nq, nkv, d, page, window, cached lengths of the requests
+    (8, 2, 128, 16, 0, [0, 5, 699, 31, 256]),
+    (6, 3, 64, 4, 0, [17, 300, 1]),           # pages of four: values are read in two halves
+    (20, 1, 64, 8, 0, [90, 513]),             # 20 heads on one kv head: two chunks of heads
+    (4, 4, 192, 32, 57, [400, 20, 56, 57]),   # window
+    (32, 8, 128, 16, 0, [2047] * 3),
+]
+
+
+@pytest.mark.parametrize("case", FUSED_CASES, ids=lambda c: f"h{c[0]}kv{c[1]}d{c[2]}p{c[3]}w{c[4]}")
+@pytest.mark.parametrize("normed", [True, False], ids=["norm", "nonorm"])
+def test_decode_attention_fused(case, normed):
+    """Norm, rotation, cache write, split-key attention and merge of a decode step in one
+    kernel: the output and what lands in the cache against the plain formulas."""
+    ops = _ops()
+    nq, nkv, d, page, window, cached = case
+    theta, eps = 50000.0, 3e-6
+    gen = torch.Generator().manual_seed(d + nq)
+    rng = random.Random(nq * 31 + d)
+    n = len(cached)
+    total_pages = sum(-(-(a + 1) // page) for a in cached) + 1
+    order = list(range(1, total_pages))
+    rng.shuffle(order)
+    max_pages = max(-(-(a + 1) // page) for a in cached) + 1
+    table = torch.zeros((n + 2, max_pages), dtype=torch.int32)
+    kc = torch.full((total_pages, nkv, page, d), float("nan"))
+    vc = torch.full((total_pages, nkv, d, page), float("nan"))
+    slots = list(range(n + 2))
+    rng.shuffle(slots)
+    qw = 1 + 0.1 * torch.randn(d, generator=gen) if normed else None
+    kw = 1 + 0.1 * torch.randn(d, generator=gen) if normed else None
+    qkv = torch.randn(n, (nq + 2 * nkv) * d, generator=gen).bfloat16()
+    expect, new_k, new_v = [], [], []
+    for i, a in enumerate(cached):
+        k_old = torch.randn(a, nkv, d, generator=gen).bfloat16().float()
+        v_old = torch.randn(a, nkv, d, generator=gen).bfloat16().float()
+        slot = slots[i]
+        for p in range(-(-(a + 1) // page)):
+            pid = order.pop()
+            table[slot, p] = pid
+            lo, hi = p * page, min(a, (p + 1) * page)
+            if hi > lo:
+                kc[pid, :, : hi - lo, :] = k_old[lo:hi].transpose(0, 1)
+                vc[pid, :, :, : hi - lo] = v_old[lo:hi].permute(1, 2, 0)
+        row = qkv[i].float()
+        q = row[: nq * d].view(1, nq, d)
+        k = row[nq * d : (nq + nkv) * d].view(1, nkv, d)
+        v = row[(nq + nkv) * d :].view(1, nkv, d)
+        if normed:
+            q, k = plain_rmsnorm(q, qw, eps), plain_rmsnorm(k, kw, eps)
+        pc, ps = plain_rope_tables(torch.tensor([a]), d, theta)
+        q, k = plain_rope_apply(q, pc, ps), plain_rope_apply(k, pc, ps)
+        k, q = k.bfloat16().float(), q.bfloat16().float()  # what the cache and the product hold
+        keys, vals = torch.cat([k_old, k]), torch.cat([v_old, v])
+        expect.append(
+            plain_attention(q, keys, vals, d**-0.5, window or None, torch.tensor([a]), torch.arange(a + 1)).reshape(1, nq * d)
+        )
+        new_k.append(k[0])
+        new_v.append(v[0])
+    ctx = SimpleNamespace(
+        positions=torch.tensor(cached, dtype=torch.int32, device=DEV),
+        token_slot=torch.tensor(slots[:n], dtype=torch.int32, device=DEV),
+        token_ids=torch.zeros(n, dtype=torch.int32, device=DEV),
+        h_seq_starts=list(cached), h_seq_lens=[1] * n, max_position=max(cached), extra={},
+    )
+    assert ops.decode_attention_fusable(ctx, torch.bfloat16, nq // nkv, d, d // 2)
+    cos, sin = ops.rope_table(plain_inv_freq(d, theta).to(DEV), max(cached) + 1)
+    kcd, vcd = kc.bfloat16().to(DEV), vc.bfloat16().to(DEV)
+    out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    for _ in range(2):  # twice: the merge counters must be back at zero after a launch
+        ops.decode_attention_fused(
+            qkv.to(DEV), kcd, vcd, out, ctx, table.to(DEV), page, nq, nkv, d, window, d**-0.5,
+            qw.to(DEV) if normed else None, kw.to(DEV) if normed else None, cos, sin, eps, True,
+        )
+        got = out.float().cpu()
+        assert torch.isfinite(got).all()
+        torch.testing.assert_close(got, torch.cat(expect), rtol=2e-2, atol=2e-2)
+    kcc, vcc = kcd.float().cpu(), vcd.float().cpu()
+    for i, a in enumerate(cached):
+        pid, off = int(table[slots[i], a // page]), a % page
+        torch.testing.assert_close(kcc[pid, :, off, :], new_k[i], rtol=8e-3, atol=8e-3)
+        torch.testing.assert_close(vcc[pid, :, :, off], new_v[i], rtol=0, atol=0)
+    # nothing else in the cache was touched
+    before = kc.bfloat16().float()
+    same = torch.isnan(before) == torch.isnan(kcc)
+    for i, a in enumerate(cached):
+        same[int(table[slots[i], a // page]), :, a % page, :] = True
+    assert same.all()
+    assert int(ops._merge_counters(torch.device(DEV, torch.cuda.current_device())).abs().sum()) == 0

@@ -39,7 +39,7 @@ def _context(runner, entries):
     return runner._context(dev, offs, meta)
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_parts_alone(tmp_path, which, dtype):
     from rapid_llm_amd import StepEntry

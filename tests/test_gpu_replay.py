@@ -22,6 +22,7 @@ LENGTHS = {
     "A": [13, 17, 25, 41, 70, 100],          # prompts 1/5/13/29 + 12 decoded, and two longer
     "B": [22, 37, 51, 84, 110, 170],         # prompts 2/17/31/64/90/150 + 20 decoded
     "C": [9, 33, 48, 77, 130, 201],
+    "D": [12, 40, 66, 150, 333, 600],
 }
 
 
@@ -69,7 +70,7 @@ def _check(got, want, dtype, label):
             raise AssertionError(f"{label}: request {rid}, first wrong position {first}: {exc}") from None
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_every_cut_matches_plain(tmp_path, which, dtype):
     cfg, page, seed = TINY[which]

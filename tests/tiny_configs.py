@@ -36,7 +36,20 @@ TINY_C = dict(
 )
 PAGE_C = 8
 
-TINY = {"A": (TINY_A, PAGE_A, 11), "B": (TINY_B, PAGE_B, 22), "C": (TINY_C, PAGE_C, 33)}
+# D: head 64 (the size from which a decode step's norm, rotation, cache write and attention
+# run as one kernel), a window on the last layer, group 3, page 8
+TINY_D = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=112, num_attention_heads=6, num_key_value_heads=2,
+    head_dim=64, intermediate_size=200, vocab_size=389, rope_theta=250000.0,
+    rms_norm_eps=2e-6, tie_word_embeddings=True, max_position_embeddings=640,
+    hidden_act="silu", attention_bias=False,
+    sliding_window=150, layer_types=["full_attention", "sliding_attention"],
+)
+PAGE_D = 8
+
+TINY = {"A": (TINY_A, PAGE_A, 11), "B": (TINY_B, PAGE_B, 22), "C": (TINY_C, PAGE_C, 33),
+        "D": (TINY_D, PAGE_D, 44)}
 
 
 def make_model_dir(tmp_path: Path, which: str, dtype: str = "float32") -> Path:
