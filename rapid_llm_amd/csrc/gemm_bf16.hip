@@ -47,39 +47,74 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
 // one matrix instruction.  SWIGLU: tiles 2j / 2j+1 are gate rows / up rows; N is then the
 // width I of the result.
 //
+// The A operand wants lane (n, g) to hold W[n][k0 + 32g ..]: read straight from memory that
+// is sixteen rows per quarter wave, 16 bytes each.  Instead a quarter wave reads 256
+// contiguous bytes of one row (instruction j covers rows 4j .. 4j+3 of the tile) and the tile
+// is turned into the operand layout through a wave-private piece of LDS; no barrier is
+// needed, the wave reads what it wrote itself.
+//
 // Measured on MI355X (graph replays, weights rotated through 800 MB so that nothing stays in
-// cache): a plain 16-byte-per-lane read kernel reaches 6.2-6.5 TB/s on 1.2 GB and 5 TB/s on
-// 32 MB (launch and ramp are about 2 us); this kernel reaches 6.2 TB/s on the vocabulary
-// matrix and 3.7-4.7 TB/s on the 33-100 MB matrices of a layer at one row.  Deeper unrolling,
-// non-temporal loads, more waves and staggered K offsets did not help; fewer instructions in
-// the loop did, hence the unpredicated main loop with clamped row pointers.
+// cache), 8 rows, microseconds for the four products of a Qwen3-8B layer (50 / 34 / 101 / 201
+// MB): strided reads 16.2 / 10.5 / 22.8 / 46.9; this kernel 14.7 / 9.4 / 20.5 / 41.0; weights
+// stored pre-tiled so that every instruction reads 1 KB contiguous 14.3 / 9.2 / 19.9 / 41.2
+// (no better, and the library product of the prefill could not read them); a plain read of
+// the same bytes 10 / 6.5 / 16 / 34.  Deeper unrolling, non-temporal loads, more waves, K
+// split over workgroups and staggered K offsets did not help.
+#define WT_PITCH 272  // bytes between the 16 rows of the LDS tile: 256 + 16, conflict-free reads
+
 template <int NT, typename OutT, bool SWIGLU>
 __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, OutT* __restrict__ out, int M,
     int N, int K, int ldx, int ldw, int ldo) {
     __shared__ float red[GW][NT * 256];
+    __shared__ __attribute__((aligned(16))) unsigned char wtile[GW][16 * WT_PITCH];
 
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
     const int r16 = lane & 15;
     const int g = lane >> 4;
 
-    // weight row of this lane in each tile; rows beyond the matrix read the last row and
-    // their results are dropped in the epilogue
+    // first weight row of each tile; rows beyond the matrix read the last row and their
+    // results are dropped in the epilogue
+    int tile_row[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        if (SWIGLU)
+            tile_row[nt] = (blockIdx.x * (NT / 2) + nt / 2) * 16 + ((nt & 1) ? N : 0);
+        else
+            tile_row[nt] = (blockIdx.x * NT + nt) * 16;
+    }
+    const int row_limit = SWIGLU ? 2 * N - 1 : N - 1;
+    const int seg_limit = N - 1;  // within the gate (or up) half
+    // coalesced reads: instruction j of tile nt reads row 4j + g of the tile at bytes 16 r16
+    const bf16_t* wld[NT][4];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int row = tile_row[nt] + 4 * j + g;
+            if (SWIGLU) {
+                const int base = (nt & 1) ? N : 0;
+                row = base + min(row - base, seg_limit);
+            }
+            row = min(row, row_limit);
+            wld[nt][j] = W + (size_t)row * ldw + 8 * r16;
+        }
+    // strided reads (the last, partial chunk only): row r16 of the tile at elements 32 g
     const bf16_t* wrow[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        int row;
+        int row = tile_row[nt] + r16;
         if (SWIGLU) {
-            const int n = min((blockIdx.x * (NT / 2) + nt / 2) * 16 + r16, N - 1);
-            row = (nt & 1) ? N + n : n;
-        } else {
-            row = min((blockIdx.x * NT + nt) * 16 + r16, N - 1);
+            const int base = (nt & 1) ? N : 0;
+            row = base + min(row - base, seg_limit);
         }
+        row = min(row, row_limit);
         wrow[nt] = W + (size_t)row * ldw + 32 * g;
     }
     const bool xok = r16 < M;
     const bf16_t* xrow = X + (size_t)(xok ? r16 : 0) * ldx + 32 * g;
+    unsigned char* mytile = wtile[wave];
 
     f32x4 acc[NT];
 #pragma unroll
@@ -88,18 +123,29 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     // whole chunks of 128: no predicates.  The bound is the same for every lane of a wave.
     const int kfull = K & ~(KSTEP - 1);
     for (int kw = wave * KSTEP; kw < kfull; kw += GW * KSTEP) {
-        bf16x8 a[NT][4], x[4];
+        uint4 raw[NT][4];
+        bf16x8 x[4];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) a[nt][j] = ld16(wrow[nt] + kw + 8 * j);
+            for (int j = 0; j < 4; ++j) raw[nt][j] = *reinterpret_cast<const uint4*>(wld[nt][j] + kw);
 #pragma unroll
         for (int j = 0; j < 4; ++j) x[j] = xok ? ld16(xrow + kw + 8 * j) : z8();
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int nt = 0; nt < NT; ++nt) {
+            // the tiles of a wave go through the same piece of LDS one after the other
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nt][j], x[j], acc[nt], 0, 0, 0);
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<uint4*>(mytile + (4 * j + g) * WT_PITCH + 16 * r16) = raw[nt][j];
+            bf16x8 a[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                a[j] = __builtin_bit_cast(
+                    bf16x8, *reinterpret_cast<const uint4*>(mytile + r16 * WT_PITCH + 64 * g + 16 * j));
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], x[j], acc[nt], 0, 0, 0);
+        }
     }
     // the last, partial chunk (K is a multiple of 8: a piece is whole or absent)
     if (kfull < K && wave == (kfull / KSTEP) % GW) {

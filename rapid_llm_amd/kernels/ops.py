@@ -497,20 +497,6 @@ def attention_plan(ctx, group: int, d: int) -> AttentionPlan:
     return plan
 
 
-_MERGE_COUNTERS: dict[torch.device, torch.Tensor] = {}
-_NUM_MERGE_COUNTERS = 1 << 16
-
-
-def _merge_counters(device: torch.device) -> torch.Tensor:
-    """Zeroed ints the decode kernel's in-kernel merge counts finished splits with.  Every
-    launch leaves them zero again, so one buffer per device serves all layers of a stream."""
-    buf = _MERGE_COUNTERS.get(device)
-    if buf is None:
-        buf = torch.zeros(_NUM_MERGE_COUNTERS, dtype=torch.int32, device=device)
-        _MERGE_COUNTERS[device] = buf
-    return buf
-
-
 def _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_size, nq, nkv, d,
                    window, scale, fused) -> None:
     """Split-key decode attention of the step's single tokens.  ``fused`` is ``None`` (``q``
@@ -527,19 +513,17 @@ def _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_s
     chunk = max(_MIN_SPLIT_KEYS, -(-(-(-span // want)) // 128) * 128)
     chunk = min(chunk, max(32, ((_MAX_SPLIT_PAGES - 1) * page_size - 31) // 32 * 32))
     nsplit = -(-span // chunk)
-    part_o = part_ml = counters = None
+    part_o = part_ml = None
     if nsplit > 1:
         part_o = torch.empty((plan.num_decode, nq, nsplit, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((plan.num_decode, nq, nsplit, 2), dtype=torch.float32, device=q.device)
-        if pairs <= _NUM_MERGE_COUNTERS:
-            counters = _merge_counters(q.device)
     qn = kn = cos = sin = kw = vw = None
     eps = 0.0
     if fused is not None:
         qn, kn, cos, sin, kw, vw, eps = fused
     _ok(
         lib.rl_attn_decode(
-            _p(q), _p(k_cache), _p(v_cache), _p(out), _p(part_o), _p(part_ml), _p(counters),
+            _p(q), _p(k_cache), _p(v_cache), _p(out), _p(part_o), _p(part_ml),
             _p(plan.seq_token), _p(ctx.positions), _p(ctx.token_slot), _p(block_table),
             block_table.stride(0), page_size, plan.num_decode, nq, nkv, window,
             ctypes.c_float(scale), chunk, nsplit, int(fused is not None), _p(qn), _p(kn), _p(cos),
@@ -579,7 +563,7 @@ def decode_attention_fused(
     write_cache: bool,
 ) -> None:
     """Per-head norm, rotation, cache write and split-key attention of a step of single
-    tokens in one kernel (the merge of the splits included).  Same result as
+    tokens in one kernel (plus the merge of the splits).  Same result as
     ``qknorm_rope_kvwrite`` followed by ``paged_attention`` up to rounding."""
     tokens = qkv.shape[0]
     pages = k_cache.shape[0]
