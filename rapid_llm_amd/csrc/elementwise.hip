@@ -323,7 +323,8 @@ __global__ void qknorm_rope_kvwrite_kernel(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int d, int rotary_half, float eps, int write_cache) {
+    int page_size, int nq, int nkv, int d, int rotary_half, float eps, int write_cache,
+    int write_values) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -343,8 +344,8 @@ __global__ void qknorm_rope_kvwrite_kernel(
     for (int head = blockIdx.y * nwaves + wave; head < total_heads; head += nwaves * gridDim.y) {
         const T* x = row + (size_t)head * d;
         if (head >= nq + nkv) {
-            // value head: copy into the transposed page
-            if (!write_cache) continue;
+            // value head: copy into the transposed page (unless the tile kernel below does it)
+            if (!write_cache || !write_values) continue;
             const int h = head - nq - nkv;
             T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
             for (int i = lane; i < d; i += RL_WAVE) dst[(size_t)i * page_size] = x[i];
@@ -401,6 +402,189 @@ __global__ void qknorm_rope_kvwrite_kernel(
     }
 }
 
+// The same with four consecutive channels of each half per lane: LPH lanes (16 for heads up to
+// 128, else 32) take one head, a wave takes 64 / LPH heads, and every load and store moves 8
+// or 16 bytes.  Needs d % 8 == 0.
+template <typename T, int LPH>
+__global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, const int* __restrict__ positions,
+    const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
+    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values) {
+    constexpr int HPW = RL_WAVE / LPH;  // heads per wave
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int sub = lane / LPH;  // which of the wave's heads
+    const int li = lane % LPH;   // channels 4 li .. 4 li + 3 of each half
+    const int half = d / 2;
+    const int pos = positions[t];
+    const int total_heads = nq + (write_values ? 2 * nkv : nkv);
+    const T* row = qkv + (size_t)t * (nq + 2 * nkv) * d;
+    size_t page = 0;
+    int off = 0;
+    if (write_cache) {
+        page = (size_t)block_table[(size_t)token_slot[t] * table_stride + pos / page_size];
+        off = pos % page_size;
+    }
+    const int head = (blockIdx.y * (blockDim.x / RL_WAVE) + wave) * HPW + sub;
+    if (head >= total_heads) return;  // whole groups of LPH lanes leave together
+    const T* x = row + (size_t)head * d;
+    const bool active = 4 * li < half;
+    if (head >= nq + nkv) {
+        if (!write_cache) return;
+        const int h = head - nq - nkv;
+        T* dst = v_cache + ((page * nkv + h) * d) * page_size + off;
+        for (int i = li; i < d; i += LPH) dst[(size_t)i * page_size] = x[i];
+        return;
+    }
+    const bool is_q = head < nq;
+    if (!is_q && !write_cache) return;
+    const float* w = is_q ? q_norm_w : k_norm_w;
+    float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+    float ss = 0.f;
+    if (active) {
+        const Vec4<T> va = *reinterpret_cast<const Vec4<T>*>(x + 4 * li);
+        const Vec4<T> vb = *reinterpret_cast<const Vec4<T>*>(x + half + 4 * li);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            a[k] = to_float(va.v[k]);
+            b[k] = to_float(vb.v[k]);
+            ss += a[k] * a[k] + b[k] * b[k];
+        }
+    }
+    if (w) {
+        // sum over the LPH lanes of the head (a power of two, aligned in the wave)
+#pragma unroll
+        for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, RL_WAVE);
+        const float rrms = rsqrtf(ss / (float)d + eps);
+        if (active) {
+            const float4 wa = *reinterpret_cast<const float4*>(w + 4 * li);
+            const float4 wb = *reinterpret_cast<const float4*>(w + half + 4 * li);
+            a[0] *= rrms * wa.x; a[1] *= rrms * wa.y; a[2] *= rrms * wa.z; a[3] *= rrms * wa.w;
+            b[0] *= rrms * wb.x; b[1] *= rrms * wb.y; b[2] *= rrms * wb.z; b[3] *= rrms * wb.w;
+        }
+    }
+    if (!active) return;
+    if (cos_tab) {
+        const float4 c4 = *reinterpret_cast<const float4*>(cos_tab + (size_t)pos * half + 4 * li);
+        const float4 s4 = *reinterpret_cast<const float4*>(sin_tab + (size_t)pos * half + 4 * li);
+        const float cs[4] = {c4.x, c4.y, c4.z, c4.w}, sn[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float ra = a[k] * cs[k] - b[k] * sn[k];
+            b[k] = b[k] * cs[k] + a[k] * sn[k];
+            a[k] = ra;
+        }
+    }
+    T* dst = is_q ? q_out + ((size_t)t * nq + head) * d
+                  : k_cache + ((page * nkv + (head - nq)) * page_size + off) * d;
+    Vec4<T> oa, ob;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        oa.v[k] = from_float<T>(a[k]);
+        ob.v[k] = from_float<T>(b[k]);
+    }
+    *reinterpret_cast<Vec4<T>*>(dst + 4 * li) = oa;
+    *reinterpret_cast<Vec4<T>*>(dst + half + 4 * li) = ob;
+}
+
+template <typename T>
+static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const float* q_norm_w,
+                          const float* k_norm_w, const float* cos_tab, const float* sin_tab,
+                          const int* positions, const int* token_slot, const int* block_table,
+                          int table_stride, int page_size, int tokens, int nq, int nkv, int d,
+                          int rotary_half, float eps, int write_cache, int write_values,
+                          hipStream_t stream) {
+    const int total_heads = nq + (write_values ? 2 * nkv : nkv);
+    if (d % 8 == 0) {
+        const int lph = d <= 128 ? 16 : 32;
+        const int heads_per_block = 4 * (RL_WAVE / lph);
+        const int groups = (total_heads + heads_per_block - 1) / heads_per_block;
+        dim3 grid(tokens, groups), block(256);
+        if (lph == 16)
+            hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 16>), grid, block, 0, stream, qkv,
+                               q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
+                               positions, token_slot, block_table, table_stride, page_size, nq, nkv,
+                               d, eps, write_cache, write_values);
+        else
+            hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 32>), grid, block, 0, stream, qkv,
+                               q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
+                               positions, token_slot, block_table, table_stride, page_size, nq, nkv,
+                               d, eps, write_cache, write_values);
+        return;
+    }
+    const int head_groups = (total_heads + 3) / 4;
+    dim3 grid(tokens, head_groups > 65535 ? 65535 : head_groups), block(256);
+    hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, grid, block, 0, stream, qkv, q_out, k_cache,
+                       v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
+                       block_table, table_stride, page_size, nq, nkv, d, rotary_half, eps,
+                       write_cache, write_values);
+}
+
+// Values of 16 consecutive tokens of the batch and one kv head, written by one workgroup.
+// The cache stores values transposed, V[page][head][channel][slot]: the sixteen slots of a
+// channel are one 32-byte row (at a page of 16), and consecutive tokens of a request fill
+// consecutive slots of it.  Written token by token those rows are completed by sixteen
+// different workgroups, 2 bytes at a time; here a thread writes the four slots of four
+// consecutive tokens at once where they line up, and the four threads of a row sit in
+// adjacent lanes.
+#define VT_TOKENS 16
+
+template <typename T>
+__global__ __launch_bounds__(256) void v_tile_write_kernel(
+    const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
+    const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
+    int page_size, int tokens, int nq, int nkv, int d) {
+    __shared__ T vt[VT_TOKENS][256 + 8];
+    __shared__ int s_page[VT_TOKENS];
+    __shared__ int s_off[VT_TOKENS];
+    const int t0 = blockIdx.x * VT_TOKENS;
+    const int h = blockIdx.y;
+    const int row_width = (nq + 2 * nkv) * d;
+    if (threadIdx.x < VT_TOKENS) {
+        const int t = t0 + threadIdx.x;
+        int page = -1, off = 0;
+        if (t < tokens) {
+            const int pos = positions[t];
+            page = block_table[(size_t)token_slot[t] * table_stride + pos / page_size];
+            off = pos % page_size;
+        }
+        s_page[threadIdx.x] = page;
+        s_off[threadIdx.x] = off;
+    }
+    for (int idx = threadIdx.x; idx < VT_TOKENS * d; idx += 256) {
+        const int i = idx / d, c = idx - i * d;
+        if (t0 + i < tokens)
+            vt[i][c] = qkv[(size_t)(t0 + i) * row_width + (size_t)(nq + nkv + h) * d + c];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 4 * d; idx += 256) {
+        const int quarter = idx & 3, c = idx >> 2;
+        const int i0 = 4 * quarter;
+        const int page = s_page[i0], off = s_off[i0];
+        bool lined_up = page >= 0 && (off & 3) == 0 && (page_size & 3) == 0;
+#pragma unroll
+        for (int k = 1; k < 4; ++k)
+            lined_up = lined_up && s_page[i0 + k] == page && s_off[i0 + k] == off + k;
+        if (lined_up) {
+            Vec4<T> v;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v.v[k] = vt[i0 + k][c];
+            *reinterpret_cast<Vec4<T>*>(v_cache + (((size_t)page * nkv + h) * d + c) * page_size + off) = v;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int pg = s_page[i0 + k];
+                if (pg >= 0)
+                    v_cache[(((size_t)pg * nkv + h) * d + c) * page_size + s_off[i0 + k]] = vt[i0 + k][c];
+            }
+        }
+    }
+}
+
 extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cache, void* v_cache,
                                       const float* q_norm_w, const float* k_norm_w,
                                       const float* cos_tab, const float* sin_tab,
@@ -413,22 +597,32 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
     if (d % 2 || d > 256) return RL_ERR_ARG;
     // only a rotation over the whole head is implemented (pairs i, i + d/2)
     if (cos_tab && rotary_half != d / 2) return RL_ERR_ARG;
-    const int total_heads = nq + 2 * nkv;
-    const int head_groups = (total_heads + 3) / 4;
-    dim3 grid(tokens, head_groups > 65535 ? 65535 : head_groups), block(256);
-    if (act_type == RL_F32)
-        hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<float>, grid, block, 0, stream,
-                           (const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
-                           q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
-                           block_table, table_stride, page_size, nq, nkv, d, rotary_half, eps,
-                           write_cache);
-    else if (act_type == RL_BF16)
-        hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<bf16_t>, grid, block, 0, stream,
-                           (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
-                           (bf16_t*)v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions,
-                           token_slot, block_table, table_stride, page_size, nq, nkv, d,
-                           rotary_half, eps, write_cache);
-    else
+    // with enough tokens the values go through the tile kernel, and the per-head kernel
+    // covers the query and key heads only
+    const int tile_values = write_cache && tokens >= 8 && nkv <= 65535;
+    if ((long)nq + 2 * nkv > 65535 * 4) return RL_ERR_ARG;
+    dim3 block(256);
+    dim3 vgrid((tokens + VT_TOKENS - 1) / VT_TOKENS, nkv);
+    if (act_type == RL_F32) {
+        launch_qknorm<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
+                             q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
+                             block_table, table_stride, page_size, tokens, nq, nkv, d, rotary_half,
+                             eps, write_cache, !tile_values, stream);
+        if (tile_values)
+            hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, block, 0, stream,
+                               (const float*)qkv, (float*)v_cache, positions, token_slot,
+                               block_table, table_stride, page_size, tokens, nq, nkv, d);
+    } else if (act_type == RL_BF16) {
+        launch_qknorm<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
+                              (bf16_t*)v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions,
+                              token_slot, block_table, table_stride, page_size, tokens, nq, nkv, d,
+                              rotary_half, eps, write_cache, !tile_values, stream);
+        if (tile_values)
+            hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, block, 0, stream,
+                               (const bf16_t*)qkv, (bf16_t*)v_cache, positions, token_slot,
+                               block_table, table_stride, page_size, tokens, nq, nkv, d);
+    } else {
         return RL_ERR_ARG;
+    }
     return rl_launch_status();
 }

@@ -209,12 +209,17 @@ def test_rope_table_matches_plain():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("shape", [(5, 5, 48, 8), (6, 2, 128, 16), (3, 1, 16, 4), (4, 4, 256, 4)])
-def test_qknorm_rope_kvwrite(dtype, shape):
+@pytest.mark.parametrize("many", [False, True], ids=["few", "many"])
+def test_qknorm_rope_kvwrite(dtype, shape, many):
     ops = _ops()
     nq, nkv, d, page = shape
     theta, eps = 77777.0, 2e-5
-    positions = [0, 1, 2, 9, 300, 301, 4000]
-    slots = [2, 2, 2, 0, 1, 1, 3]
+    if many:  # enough tokens for the value tile kernel: runs that line up with pages and runs that do not
+        positions = list(range(3, 40)) + list(range(96, 117)) + [7] + list(range(4000, 3990, -1))
+        slots = [2] * 37 + [0] * 21 + [1] + [3] * 10
+    else:
+        positions = [0, 1, 2, 9, 300, 301, 4000]
+        slots = [2, 2, 2, 0, 1, 1, 3]
     t = len(positions)
     qkv = torch.randn(t, (nq + 2 * nkv) * d).to(dtype)
     qw = 1 + 0.1 * torch.randn(d)
@@ -222,7 +227,7 @@ def test_qknorm_rope_kvwrite(dtype, shape):
     max_pages = 4001 // page + 1
     table = torch.zeros((4, max_pages), dtype=torch.int32)
     pid = 1
-    for p, s in zip(positions, slots):
+    for p, s in sorted(zip(positions, slots), key=lambda ps: (ps[0] * 7 + ps[1]) % 13):  # pages in no order
         if table[s, p // page] == 0:
             table[s, p // page] = pid
             pid += 1
