@@ -582,7 +582,9 @@ extern "C" int rl_attn_decode_fusable() { return D % 64 == 0 ? 1 : 0; }
 // accumulators are rescaled only when some row's maximum moved.
 //
 // tile_info[4 * tile + {0,1,2,3}] = {first token of the request's portion in the flat batch,
-//   tokens of the request already in the cache, tokens in this portion, first row of the tile}
+//   tokens of the request already in the cache, tokens in this portion, first row of the tile};
+// work_order (optional): workgroup b takes (tile, kv head) = (work_order[b] / nkv, % nkv), so
+// that the host decides which workgroups start together.
 // Two waves per SIMD at most: the accumulators then live in ordinary vector registers, which
 // the rescale and the epilogue read directly (at the default budget of 128 the compiler parks
 // them in accumulation registers and moves them back and forth around every rescale).
@@ -590,15 +592,16 @@ __global__ __launch_bounds__(PF_WAVES* RL_WAVE) __attribute__((amdgpu_waves_per_
 attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out,
-    const int* __restrict__ tile_info, const int* __restrict__ token_slot,
-    const int* __restrict__ block_table, int table_stride, int page_size, int nq, int nkv,
-    int window, float scale_log2) {
+    const int* __restrict__ tile_info, const int* __restrict__ work_order,
+    const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
+    int page_size, int nq, int nkv, int window, float scale_log2) {
     __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_KEYS * K_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Vs[D * V_LD];
 
     const int G = nq / nkv;
-    const int tile = blockIdx.x;
-    const int hk = blockIdx.y;
+    const int item = work_order ? work_order[blockIdx.x] : blockIdx.x;
+    const int tile = item / nkv;
+    const int hk = item % nkv;
     const int tok0 = tile_info[4 * tile + 0];
     const int start = tile_info[4 * tile + 1];
     const int qlen = tile_info[4 * tile + 2];
@@ -838,16 +841,18 @@ attn_prefill_kernel(
 extern "C" int rl_attn_prefill_rows() { return PF_ROWS; }
 
 extern "C" int rl_attn_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
-                               const int* tile_info, int num_tiles, const int* token_slot,
+                               const int* tile_info, const int* work_order, int num_tiles,
+                               const int* token_slot,
                                const int* block_table, int table_stride, int page_size, int nq,
                                int nkv, int window, float scale, hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535) return RL_ERR_ARG;
     const float scale_log2 = scale * 1.4426950408889634f;
-    dim3 grid(num_tiles, nkv), block(PF_WAVES * RL_WAVE);
+    if ((long)num_tiles * nkv > 0x7fffffffL) return RL_ERR_ARG;
+    dim3 grid(num_tiles * nkv), block(PF_WAVES * RL_WAVE);
     hipLaunchKernelGGL(attn_prefill_kernel, grid, block, 0, stream, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_info,
-                       token_slot, block_table, table_stride, page_size, nq, nkv, window,
+                       work_order, token_slot, block_table, table_stride, page_size, nq, nkv, window,
                        scale_log2);
     return rl_launch_status();
 }

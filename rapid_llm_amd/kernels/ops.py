@@ -388,7 +388,7 @@ class AttentionPlan:
     (query heads per kv head): which requests are single tokens (decode kernel) and how the
     portions of the others are cut into row tiles (prefill kernel)."""
 
-    __slots__ = ("num_decode", "seq_token", "max_decode_ctx", "num_tiles", "tile_info")
+    __slots__ = ("num_decode", "seq_token", "max_decode_ctx", "num_tiles", "tile_info", "tile_keys", "orders")
 
     def __init__(self, ctx, group: int, tile_rows: int) -> None:
         fixed = ctx.extra.get("decode_only_tokens")
@@ -399,6 +399,8 @@ class AttentionPlan:
             self.max_decode_ctx = max(ctx.h_seq_starts) + 1
             self.num_tiles = 0
             self.tile_info = None
+            self.tile_keys = []
+            self.orders = {}
             return
         dec_tokens: list[int] = []
         tile_list: list[tuple[int, int, int, int]] = []
@@ -412,10 +414,10 @@ class AttentionPlan:
                 for row0 in range(0, n * group, tile_rows):
                     tile_list.append((at, start, n, row0))
             at += n
-        # tiles with the most keys first: workgroups are handed out in this order, and the
-        # short ones then fill the gaps the long ones leave
-        tile_list.sort(key=lambda t: -(t[1] + min(t[2], (t[3] + tile_rows) // group)))
         tiles = [v for t in tile_list for v in t]
+        # keys each tile reads: what its workgroups cost
+        self.tile_keys = [t[1] + min(t[2], (t[3] + tile_rows) // group) for t in tile_list]
+        self.orders = {}
         self.num_decode = len(dec_tokens)
         self.num_tiles = len(tiles) // 4
         device = ctx.token_ids.device
@@ -423,11 +425,28 @@ class AttentionPlan:
         self.seq_token = packed[: self.num_decode]
         self.tile_info = packed[self.num_decode :]
 
+    def work_order(self, nkv: int, device) -> torch.Tensor:
+        """Order in which the (tile, kv head) pairs of the prefill kernel are handed out.
+        The first round, one workgroup on every compute unit, takes the longest; the second
+        round, which joins them on the same units, the shortest in ascending order, so that a
+        unit's two workgroups add up alike; the rest follow longest first and fill the gaps."""
+        order = self.orders.get(nkv)
+        if order is None:
+            items = sorted(range(self.num_tiles * nkv), key=lambda i: (-self.tile_keys[i // nkv], i))
+            first = items[:_FIRST_ROUND]
+            rest = items[_FIRST_ROUND:]
+            second = rest[::-1][:_FIRST_ROUND]
+            middle = rest[: max(0, len(rest) - _FIRST_ROUND)]
+            order = torch.tensor(first + second + middle, dtype=torch.int32).to(device)
+            self.orders[nkv] = order
+        return order
+
 
 # Workgroups a decode launch should reach before it stops splitting the keys, and the fewest
 # keys a split is worth (measured at 2,048 keys, 8 kv heads: 1 request 256 keys a split,
 # 8 requests 512, 64 requests no split; finer splits only add merge work).
 _TARGET_BLOCKS = 256
+_FIRST_ROUND = 256  # workgroups that start first, one on each compute unit
 _MIN_SPLIT_KEYS = 256
 _MAX_SPLIT_PAGES = 1024  # page ids of one split are staged in LDS
 
@@ -476,7 +495,8 @@ def paged_attention(
     if plan.num_tiles:
         _ok(
             lib.rl_attn_prefill(
-                _p(q), _p(k_cache), _p(v_cache), _p(out), _p(plan.tile_info), plan.num_tiles,
+                _p(q), _p(k_cache), _p(v_cache), _p(out), _p(plan.tile_info),
+                _p(plan.work_order(nkv, q.device)), plan.num_tiles,
                 _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv,
                 window, ctypes.c_float(scale), _stream(),
             ),
