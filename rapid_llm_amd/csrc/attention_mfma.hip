@@ -9,12 +9,13 @@
 //
 // with v_mfma_f32_16x16x32_bf16: a wave owns 16 "rows" (queries) as the N dimension.  The
 // result of the first product leaves lane (row r, group g = lane / 16) with the scores of
-// keys 4g..4g+3 of each 16-key block; two such blocks are exactly the B operand of the
-// second product once its contraction slots are labelled (g, j): j < 4 -> key 4g + j of
-// the first block, j >= 4 -> key 4g + j - 4 of the second.  The A operand then needs, for
-// channel d, the values of those same keys: two 8-byte reads of four consecutive positions,
-// which is why the cache stores values transposed (V[page][head][d][slot]).  Softmax state
-// (running maximum and sum) is one scalar per lane, since a lane only ever sees one row.
+// four tile rows 4g..4g+3 of each 16-key block.  Which key a tile row holds is free, and it is
+// chosen so that the two blocks of a 32-key step leave the lane with the eight *consecutive*
+// keys 8g..8g+7: tile row i of block kb holds key 8 (i / 4) + 4 kb + i % 4.  Those eight
+// scores are then exactly the lane's contraction slots of the second product, whose A
+// operand needs, for channel d, the values of the same eight keys: one 16-byte read, which is
+// why the cache stores values transposed (V[page][head][d][slot]).  Softmax state (running
+// maximum and sum) is one scalar per lane, since a lane only ever sees one row.
 //
 // Rows are (token, query head of the kv group) pairs, so grouped-query attention reads each
 // key once for all heads of its group.  Softmax runs in the exp2 domain in float32
@@ -22,12 +23,14 @@
 // bfloat16 for the second product (:162), sums use the unrounded values.
 //
 //   rl_attn_prefill: portions of prompts.  Workgroup = 4 waves x 32 rows; K and V^T tiles of
-//                    64 keys are staged through LDS and shared by the waves.
+//                    64 keys go through LDS, the next tile travelling from memory while this
+//                    one is multiplied; one softmax step per 64 keys.
 //   rl_attn_decode:  single tokens.  Workgroup = (request, kv head, split of the keys); its
 //                    4 waves stride over 32-key steps reading K and V^T straight from
-//                    global memory (nothing is reused), combine through LDS, and a merge
-//                    kernel folds the splits (rapid_llm/kernels/ops/attention/flashdecoding.py:
-//                    115-263 stage 1, :334-407 stage 2).
+//                    global memory one step ahead (nothing is reused), combine through LDS,
+//                    and a merge kernel folds the splits (rapid_llm/kernels/ops/attention/
+//                    flashdecoding.py:115-263 stage 1, :334-407 stage 2).  In its fused form
+//                    it also norms and rotates q and k and writes the token's k and v.
 #include "common.h"
 
 #ifndef RL_HEAD_DIM
@@ -83,8 +86,8 @@ __device__ inline float row_sum4(float v) {
 
 // --------------------------------------------------------------------------- //
 // One 32-key step of the online softmax for one block of 16 rows.
-//   s0, s1: raw scores (q . k) of the two 16-key blocks, this lane's keys 4g..4g+3
-//   ok0, ok1: bit i set when key i of the block is visible to this lane's row
+//   s0, s1: raw scores (q . k) of the two 16-key blocks: this lane's keys 8g..8g+3, 8g+4..8g+7
+//   ok0, ok1: bit i set when key i of those four is visible to this lane's row
 // Updates (m, l), scales the accumulators, returns P^T as the B operand.
 // --------------------------------------------------------------------------- //
 __device__ inline bf16x8 softmax_step(f32x4 s0, f32x4 s1, unsigned ok0, unsigned ok1,
