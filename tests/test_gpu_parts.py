@@ -130,21 +130,81 @@ class ToyConfig:
     decay: float
     twice: bool = False
     share: bool = False
+    experts: int = 0  # > 0: layer 0's feed-forward routes every token to one of so many experts
+    period: float = 0.0  # > 0: the toy mixer adds a phase of the position to its input
 
     @classmethod
     def from_dict(cls, data, overrides=None):
         return cls(data["hidden"], data["vocab"], data["heads"], data["head_dim"], data["inter"],
-                   data["decay"], data.get("twice", False), data.get("share", False))
+                   data["decay"], data.get("twice", False), data.get("share", False),
+                   data.get("experts", 0), data.get("period", 0.0))
 
     def to_dict(self):
         return dict(architectures=["ToyForCausalLM"], hidden=self.hidden, vocab=self.vocab, heads=self.heads,
                     head_dim=self.head_dim, inter=self.inter, decay=self.decay, twice=self.twice,
-                    share=self.share, torch_dtype="float32")
+                    share=self.share, experts=self.experts, period=self.period, torch_dtype="float32")
+
+
+def _phase(positions, period, size):
+    """The toy position encoding: a sinusoid of the position, scaled differently per channel."""
+    scale = torch.linspace(0.5, 1.5, size, device=positions.device)
+    return torch.sin(positions.float()[:, None] * (2 * math.pi / period)) * scale
 
 
 def _toy_parts():
-    from rapid_llm_amd.parts import MIXERS, CacheNeed, Mixer, ParamSpec, Source
+    from rapid_llm_amd.parts import (
+        FEED_FORWARDS, MIXERS, POSITION_ENCODINGS, CacheNeed, FeedForward, Mixer, ParamSpec,
+        PositionEncoding, Source,
+    )
     from rapid_llm_amd.parts.linear import Linear
+
+    class PhaseTable(PositionEncoding):
+        """Another position encoding: an additive table by absolute position."""
+
+        kind = "toy_phase"
+
+        def __init__(self, size, period):
+            self.size, self.period, self.table = size, period, None
+
+        def bind(self, params, runtime):
+            pos = torch.arange(runtime.max_seq_len, device=runtime.device)
+            self.table = _phase(pos, self.period, self.size)
+
+    class RoutedFF(FeedForward):
+        """A feed-forward with routing: the router's logits in float32, the best expert takes
+        the token, its output is weighted with the router's probability."""
+
+        def __init__(self, hidden_size, inter, experts, checkpoint_prefix, name="ff"):
+            self.h, self.i, self.e, self.prefix, self.name = hidden_size, inter, experts, checkpoint_prefix, name
+
+        def param_specs(self):
+            p, n = self.prefix, self.name
+            return [
+                ParamSpec(n + ".router", (self.e, self.h), "matrix", (Source(p + "router", self.e),)),
+                ParamSpec(n + ".w1", (self.e * self.i, self.h), "matrix",
+                          tuple(Source(f"{p}e{k}.w1", self.i) for k in range(self.e))),
+                ParamSpec(n + ".w2", (self.e * self.h, self.i), "matrix",
+                          tuple(Source(f"{p}e{k}.w2", self.h) for k in range(self.e))),
+            ]
+
+        def bind(self, params, runtime):
+            self.router = params[self.name + ".router"]
+            self.w1 = params[self.name + ".w1"].view(self.e, self.i, self.h)
+            self.w2 = params[self.name + ".w2"].view(self.e, self.h, self.i)
+
+        def forward(self, x, ctx):
+            probs = torch.softmax(x.float() @ self.router.float().T, dim=-1)
+            weight, choice = probs.max(dim=-1)
+            out = torch.zeros_like(x)
+            for k in range(self.e):
+                rows = torch.nonzero(choice == k).flatten()
+                if rows.numel():
+                    y = torch.relu(x[rows] @ self.w1[k].T) @ self.w2[k].T
+                    out[rows] = y * weight[rows, None].to(x.dtype)
+            return out
+
+    POSITION_ENCODINGS.register("toy_phase", PhaseTable, replace=True)
+    FEED_FORWARDS.register("toy_routed", RoutedFF, replace=True)
 
     class DecayingSum(Mixer):
         """``s_t = decay * s_{t-1} + x_t`` per request, output ``W s_t``: no pages, one vector of
@@ -152,6 +212,7 @@ def _toy_parts():
 
         def __init__(self, hidden_size, decay, checkpoint_prefix, position=None, name="mixer"):
             self.h, self.decay, self.prefix, self.name = hidden_size, decay, checkpoint_prefix, name
+            self.position = position
             self.proj = Linear(hidden_size, hidden_size)
 
         def param_specs(self):
@@ -169,7 +230,10 @@ def _toy_parts():
             for slot, n in zip(ctx.h_seq_slots, ctx.h_seq_lens):
                 s = cache.state[slot]
                 for t in range(at, at + n):
-                    s = self.decay * s + x[t].float()
+                    xt = x[t].float()
+                    if self.position is not None and getattr(self.position, "table", None) is not None:
+                        xt = xt + self.position.table[ctx.positions[t]]
+                    s = self.decay * s + xt
                     out[t] = s
                 cache.state[slot] = s
                 at += n
@@ -194,9 +258,15 @@ def _toy_spec(cfg: ToyConfig):
         return PartSpec("gqa_attention", {"hidden_size": cfg.hidden, "num_heads": cfg.heads, "num_kv_heads": 1,
                                           "head_dim": cfg.head_dim, "checkpoint_prefix": f"l{i}.attn."})
 
+    ff0 = ff(0)
+    if cfg.experts:
+        ff0 = PartSpec("toy_routed", {"hidden_size": cfg.hidden, "inter": cfg.inter, "experts": cfg.experts,
+                                      "checkpoint_prefix": "l0.moe."})
+    pos0 = PartSpec("toy_phase", {"size": cfg.hidden, "period": cfg.period}) if cfg.period else PartSpec("none")
     layers = [
         LayerSpec(PartSpec("toy_decaying_sum", {"hidden_size": cfg.hidden, "decay": cfg.decay,
-                                                "checkpoint_prefix": "l0.mix."}), ff(0), norm("l0.n1"), norm("l0.n2")),
+                                                "checkpoint_prefix": "l0.mix."}), ff0, norm("l0.n1"), norm("l0.n2"),
+                  position=pos0),
         LayerSpec(attn(1), ff(1), norm("l1.n1"), norm("l1.n2"), position=rope),
     ]
     if cfg.share:
@@ -213,12 +283,22 @@ def _toy_plain(w, cfg: ToyConfig, toks):
 
     def ffn(i, h):
         x = plain_rmsnorm(h, w[f"l{i}.n2"], 1e-5)
+        if i == 0 and cfg.experts:
+            probs = torch.softmax(x @ w["l0.moe.router"].T, dim=-1)
+            weight, choice = probs.max(dim=-1)
+            y = torch.stack([
+                torch.relu(x[j] @ w[f"l0.moe.e{int(choice[j])}.w1"].T) @ w[f"l0.moe.e{int(choice[j])}.w2"].T * weight[j]
+                for j in range(t)
+            ])
+            return h + y
         return h + plain_swiglu_mlp(x, w[f"l{i}.ff.gate_proj.weight"], w[f"l{i}.ff.up_proj.weight"],
                                     w[f"l{i}.ff.down_proj.weight"])
 
     def toy(h):
         x = plain_rmsnorm(h, w["l0.n1"], 1e-5)
         s, rows = torch.zeros(cfg.hidden), []
+        if cfg.period:
+            x = x + _phase(pos, cfg.period, cfg.hidden)
         for j in range(t):
             s = cfg.decay * s + x[j]
             rows.append(s)
@@ -251,19 +331,20 @@ def _toy_plain(w, cfg: ToyConfig, toks):
     return plain_rmsnorm(h, w["final"], 1e-5) @ w["head"].T
 
 
-@pytest.mark.parametrize("variant", ["plain", "twice", "share"])
+@pytest.mark.parametrize("variant", ["plain", "twice", "share", "routed"])
 def test_toy_architecture_registers_builds_and_steps(tmp_path, variant):
     from safetensors.torch import load_file
 
     from rapid_llm_amd import StepEntry, write_random_model
     from rapid_llm_amd.config import register_architecture, unregister_architecture
-    from rapid_llm_amd.parts import MIXERS
+    from rapid_llm_amd.parts import FEED_FORWARDS, MIXERS, POSITION_ENCODINGS
 
     _toy_parts()
     register_architecture("ToyForCausalLM", ToyConfig, _toy_spec, replace=True)
     try:
         cfg = ToyConfig(hidden=48, vocab=97, heads=3, head_dim=16, inter=80, decay=0.8,
-                        twice=variant == "twice", share=variant == "share")
+                        twice=variant == "twice", share=variant == "share",
+                        experts=3 if variant == "routed" else 0, period=9.0 if variant == "routed" else 0.0)
         folder = write_random_model(cfg.to_dict(), 3, tmp_path / "toy", dtype="float32")
         weights = load_file(str(folder / "model.safetensors"))
         if variant == "share":  # the sharing layer's own k/v projections exist but are never used
@@ -271,6 +352,10 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant):
         runner = _runner(folder, "float32", 8)
         needs = runner.model.cache_needs()
         assert needs[0].kind == "state" and needs[1].kind == "kv"
+        if variant == "routed":
+            assert type(runner.model.blocks[0].feed_forward).__name__ == "RoutedFF"
+            assert type(runner.model.blocks[1].feed_forward).__name__ == "SwiGLU"
+            assert runner.model.blocks[0].mixer.position.table.shape == (128, cfg.hidden)
         if variant == "share":
             assert needs[2].share_with == 1 and not runner.device_cache.layers[2].owns_pages
             assert runner.device_cache.layers[2].k is runner.device_cache.layers[1].k
@@ -310,6 +395,8 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant):
     finally:
         unregister_architecture("ToyForCausalLM")
         MIXERS.unregister("toy_decaying_sum")
+        FEED_FORWARDS.unregister("toy_routed")
+        POSITION_ENCODINGS.unregister("toy_phase")
 
 
 def test_unknown_part_kinds_are_named():
