@@ -161,44 +161,6 @@ extern "C" int rl_add_rmsnorm(float* residual, const void* delta, const float* w
 }
 
 // --------------------------------------------------------------------------- //
-// The norm of rows whose residual add already happened (in the epilogue of the product that
-// made the addend, which also left partial sums of squares, one per workgroup and row):
-// out[r] = residual[row] * rsqrt(sum of the partials / hidden + eps) * weight.
-// --------------------------------------------------------------------------- //
-template <typename T>
-__global__ void apply_norm_kernel(const float* __restrict__ residual, const float* __restrict__ ssq,
-                                  int ssq_blocks, int ssq_stride, const float* __restrict__ weight,
-                                  T* __restrict__ out, const int* __restrict__ rows, int hidden,
-                                  float eps) {
-    __shared__ float scratch[16];
-    const int r = blockIdx.x;
-    const int row = rows ? rows[r] : r;
-    float part = 0.f;
-    for (int p = threadIdx.x; p < ssq_blocks; p += blockDim.x) part += ssq[(size_t)p * ssq_stride + row];
-    const float rrms = rsqrtf(block_sum(part, scratch) / (float)hidden + eps);
-    const float* res = residual + (size_t)row * hidden;
-    T* o = out + (size_t)r * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_float<T>(res[i] * rrms * weight[i]);
-}
-
-extern "C" int rl_apply_norm(const float* residual, const float* ssq, int ssq_blocks, int ssq_stride,
-                             const float* weight, void* out, const int* rows, int out_rows,
-                             int hidden, float eps, int act_type, hipStream_t stream) {
-    if (out_rows <= 0) return RL_OK;
-    if (ssq_blocks < 1) return RL_ERR_ARG;
-    dim3 grid(out_rows), block(256);
-    if (act_type == RL_F32)
-        hipLaunchKernelGGL(apply_norm_kernel<float>, grid, block, 0, stream, residual, ssq,
-                           ssq_blocks, ssq_stride, weight, (float*)out, rows, hidden, eps);
-    else if (act_type == RL_BF16)
-        hipLaunchKernelGGL(apply_norm_kernel<bf16_t>, grid, block, 0, stream, residual, ssq,
-                           ssq_blocks, ssq_stride, weight, (bf16_t*)out, rows, hidden, eps);
-    else
-        return RL_ERR_ARG;
-    return rl_launch_status();
-}
-
-// --------------------------------------------------------------------------- //
 // SwiGLU on the packed [gate | up] row: out[:, j] = silu(x[:, j]) * x[:, I + j]
 // rapid_llm/kernels/ops/activation/swiglu.py:91-121
 // --------------------------------------------------------------------------- //

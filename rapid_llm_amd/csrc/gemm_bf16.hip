@@ -62,42 +62,13 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
 // split over workgroups and staggered K offsets did not help.
 #define WT_PITCH 272  // bytes between the 16 rows of the LDS tile: 256 + 16, conflict-free reads
 
-// Two fusions remove the norm kernels from a decode step:
-//   RESID: the epilogue adds the product into the float32 residual stream in place and
-//          leaves, per workgroup and row, the sum of squares of the residual values it wrote
-//          (rapid_llm/kernels/ops/layernorm/skip_rmsnorm.py:51-85 forms the same sum before the
-//          norm).
-//   XNORM: X is that residual stream, normalised on the fly: the workgroup adds up the
-//          producers' partial sums in their order, takes rsqrt(mean + eps), and turns
-//          residual * rrms * weight into the bfloat16 operand (:41-47).
-struct SkinnyArgs {
-    const bf16_t* X;  // plain operand [M, K]
-    int ldx;
-    const float* R;  // XNORM: residual rows
-    int ldr;
-    const int* xrows;  // XNORM: residual row of each of the M rows (null: row m)
-    const float* ssq_in;  // XNORM: [ssq_blocks][ssq_stride] partial sums of squares
-    int ssq_blocks;
-    int ssq_stride;
-    const float* norm_w;  // XNORM: [K]
-    float eps;
-    const bf16_t* W;
-    int ldw;
-    void* out;  // [M, N] of OutT; RESID: the float32 residual, updated in place
-    int ldo;
-    float* ssq_out;  // RESID: [gridDim.x][M]
-    int M, N, K;
-};
-
-template <int NT, typename OutT, bool SWIGLU, bool XNORM, bool RESID>
-__global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(const SkinnyArgs a) {
+template <int NT, typename OutT, bool SWIGLU>
+__global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, OutT* __restrict__ out, int M,
+    int N, int K, int ldx, int ldw, int ldo) {
     __shared__ float red[GW][NT * 256];
     __shared__ __attribute__((aligned(16))) unsigned char wtile[GW][16 * WT_PITCH];
-    __shared__ float s_part[XNORM ? 32 : 1][16];
-    __shared__ float s_rrms[16];
-    extern __shared__ float s_nw[];  // XNORM: the norm's weights
 
-    const int M = a.M, N = a.N, K = a.K;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
     const int r16 = lane & 15;
@@ -127,7 +98,7 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(const SkinnyAr
                 row = base + min(row - base, seg_limit);
             }
             row = min(row, row_limit);
-            wld[nt][j] = a.W + (size_t)row * a.ldw + 8 * r16;
+            wld[nt][j] = W + (size_t)row * ldw + 8 * r16;
         }
     // strided reads (the last, partial chunk only): row r16 of the tile at elements 32 g
     const bf16_t* wrow[NT];
@@ -139,55 +110,10 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(const SkinnyAr
             row = base + min(row - base, seg_limit);
         }
         row = min(row, row_limit);
-        wrow[nt] = a.W + (size_t)row * a.ldw + 32 * g;
+        wrow[nt] = W + (size_t)row * ldw + 32 * g;
     }
     const bool xok = r16 < M;
-    const bf16_t* xrow = nullptr;
-    const float* rrow = nullptr;
-    float rrms = 0.f;
-    if (XNORM) {
-        // the producers' partial sums of squares, added in their order; the norm's weights
-        const int m = threadIdx.x & 15, c = threadIdx.x >> 4;  // 512 threads: 32 strides of 16 rows
-        float part = 0.f;
-        if (m < M) {
-            const int rm = a.xrows ? a.xrows[m] : m;
-            for (int p = c; p < a.ssq_blocks; p += 32) part += a.ssq_in[(size_t)p * a.ssq_stride + rm];
-        }
-        s_part[c][m] = part;
-        for (int i = threadIdx.x; i < K; i += GW * RL_WAVE) s_nw[i] = a.norm_w[i];
-        __syncthreads();
-        if (threadIdx.x < 16) {
-            float total = 0.f;
-            for (int cc = 0; cc < 32; ++cc) total += s_part[cc][threadIdx.x];
-            s_rrms[threadIdx.x] = rsqrtf(total / (float)K + a.eps);
-        }
-        __syncthreads();
-        rrms = s_rrms[r16];
-        const int rm = xok ? (a.xrows ? a.xrows[r16] : r16) : 0;
-        rrow = a.R + (size_t)rm * a.ldr + 32 * g;
-    } else {
-        xrow = a.X + (size_t)(xok ? r16 : 0) * a.ldx + 32 * g;
-    }
-    // eight consecutive elements of this lane's row of X at k (relative to its 32 g)
-    auto x_piece = [&](int k) -> bf16x8 {
-        if (!xok) return z8();
-        if (XNORM) {
-            const float4 lo = *reinterpret_cast<const float4*>(rrow + k);
-            const float4 hi = *reinterpret_cast<const float4*>(rrow + k + 4);
-            const float* nw = s_nw + 32 * g + k;
-            bf16x8 v;
-            v[0] = (__bf16)(lo.x * rrms * nw[0]);
-            v[1] = (__bf16)(lo.y * rrms * nw[1]);
-            v[2] = (__bf16)(lo.z * rrms * nw[2]);
-            v[3] = (__bf16)(lo.w * rrms * nw[3]);
-            v[4] = (__bf16)(hi.x * rrms * nw[4]);
-            v[5] = (__bf16)(hi.y * rrms * nw[5]);
-            v[6] = (__bf16)(hi.z * rrms * nw[6]);
-            v[7] = (__bf16)(hi.w * rrms * nw[7]);
-            return v;
-        }
-        return ld16(xrow + k);
-    };
+    const bf16_t* xrow = X + (size_t)(xok ? r16 : 0) * ldx + 32 * g;
     unsigned char* mytile = wtile[wave];
 
     f32x4 acc[NT];
@@ -204,21 +130,21 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(const SkinnyAr
 #pragma unroll
             for (int j = 0; j < 4; ++j) raw[nt][j] = *reinterpret_cast<const uint4*>(wld[nt][j] + kw);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) x[j] = x_piece(kw + 8 * j);
+        for (int j = 0; j < 4; ++j) x[j] = xok ? ld16(xrow + kw + 8 * j) : z8();
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             // the tiles of a wave go through the same piece of LDS one after the other
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 *reinterpret_cast<uint4*>(mytile + (4 * j + g) * WT_PITCH + 16 * r16) = raw[nt][j];
-            bf16x8 av[4];
+            bf16x8 a[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                av[j] = __builtin_bit_cast(
+                a[j] = __builtin_bit_cast(
                     bf16x8, *reinterpret_cast<const uint4*>(mytile + r16 * WT_PITCH + 64 * g + 16 * j));
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[j], x[j], acc[nt], 0, 0, 0);
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], x[j], acc[nt], 0, 0, 0);
         }
     }
     // the last, partial chunk (K is a multiple of 8: a piece is whole or absent)
@@ -226,11 +152,11 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(const SkinnyAr
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const bool ok = kfull + 32 * g + 8 * j < K;
-            const bf16x8 xv = ok ? x_piece(kfull + 8 * j) : z8();
+            const bf16x8 xv = (ok && xok) ? ld16(xrow + kfull + 8 * j) : z8();
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const bf16x8 wv = ok ? ld16(wrow[nt] + kfull + 8 * j) : z8();
-                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, xv, acc[nt], 0, 0, 0);
+                const bf16x8 av = ok ? ld16(wrow[nt] + kfull + 8 * j) : z8();
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, xv, acc[nt], 0, 0, 0);
             }
         }
     }
@@ -244,124 +170,59 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(const SkinnyAr
 
     // thread -> (tile pair / tile, lane of the tile); sums the waves in order
     constexpr int OUT_TILES = SWIGLU ? NT / 2 : NT;
-    __shared__ float s_sq[RESID ? OUT_TILES * 64 : 1];
     for (int e = threadIdx.x; e < OUT_TILES * 64; e += GW * RL_WAVE) {
         const int ln = e & 63;
         const int ot = e >> 6;
         const int m = ln & 15;
         const int nbase = (blockIdx.x * OUT_TILES + ot) * 16 + 4 * (ln >> 4);
-        float sq = 0.f;
-        if (m < M) {
+        if (m >= M) continue;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int n = nbase + i;
-                if (n >= N) continue;
-                float v;
-                if (SWIGLU) {
-                    float gate = 0.f, up = 0.f;
+        for (int i = 0; i < 4; ++i) {
+            const int n = nbase + i;
+            if (n >= N) continue;
+            float v;
+            if (SWIGLU) {
+                float gate = 0.f, up = 0.f;
 #pragma unroll
-                    for (int w = 0; w < GW; ++w) {
-                        gate += red[w][((2 * ot) * 4 + i) * 64 + ln];
-                        up += red[w][((2 * ot + 1) * 4 + i) * 64 + ln];
-                    }
-                    // the activation reads its operands rounded to bfloat16, as the unfused
-                    // path does where the product's result is stored before the activation
-                    gate = bf16_to_float(float_to_bf16(gate));
-                    up = bf16_to_float(float_to_bf16(up));
-                    v = gate / (1.f + expf(-gate)) * up;
-                } else {
-                    v = 0.f;
-#pragma unroll
-                    for (int w = 0; w < GW; ++w) v += red[w][(ot * 4 + i) * 64 + ln];
+                for (int w = 0; w < GW; ++w) {
+                    gate += red[w][((2 * ot) * 4 + i) * 64 + ln];
+                    up += red[w][((2 * ot + 1) * 4 + i) * 64 + ln];
                 }
-                if (RESID) {
-                    float* r = (float*)a.out + (size_t)m * a.ldo + n;
-                    // rounded as the unfused path rounds the product before the add
-                    const float sum = *r + bf16_to_float(float_to_bf16(v));
-                    *r = sum;
-                    sq += sum * sum;
-                } else {
-                    store_out<OutT>((OutT*)a.out + (size_t)m * a.ldo + n, v);
-                }
+                // the activation reads its operands rounded to bfloat16, as the unfused
+                // path does where the product's result is stored before the activation
+                gate = bf16_to_float(float_to_bf16(gate));
+                up = bf16_to_float(float_to_bf16(up));
+                v = gate / (1.f + expf(-gate)) * up;
+            } else {
+                v = 0.f;
+#pragma unroll
+                for (int w = 0; w < GW; ++w) v += red[w][(ot * 4 + i) * 64 + ln];
             }
-        }
-        if (RESID) s_sq[e] = sq;
-    }
-    if (RESID) {
-        __syncthreads();
-        if (threadIdx.x < M) {
-            float total = 0.f;
-            for (int ot = 0; ot < OUT_TILES; ++ot)
-                for (int q = 0; q < 4; ++q) total += s_sq[ot * 64 + q * 16 + threadIdx.x];
-            a.ssq_out[(size_t)blockIdx.x * M + threadIdx.x] = total;
+            store_out<OutT>(out + (size_t)m * ldo + n, v);
         }
     }
 }
 
-template <int NT, typename OutT, bool SWIGLU, bool XNORM, bool RESID>
-static int launch(const SkinnyArgs& a, hipStream_t stream) {
+template <int NT, typename OutT, bool SWIGLU>
+static int launch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
+                  int ldw, int ldo, hipStream_t stream) {
     constexpr int rows_per_block = (SWIGLU ? NT / 2 : NT) * 16;
-    dim3 grid((a.N + rows_per_block - 1) / rows_per_block), block(GW * RL_WAVE);
-    const size_t dyn = XNORM ? (size_t)a.K * sizeof(float) : 0;
-    hipLaunchKernelGGL((gemm_skinny_kernel<NT, OutT, SWIGLU, XNORM, RESID>), grid, block, dyn, stream,
-                       a);
+    dim3 grid((N + rows_per_block - 1) / rows_per_block), block(GW * RL_WAVE);
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, OutT, SWIGLU>), grid, block, 0, stream, X, W, out,
+                       M, N, K, ldx, ldw, ldo);
     return rl_launch_status();
 }
 
-extern "C" int rl_gemm_skinny_blocks(int N, int nt) { return (N + nt * 16 - 1) / (nt * 16); }
-
-// The general entry point.  x_mode 0: X bfloat16 [M, K]; 1: residual rows normalised on the
-// fly (XNORM).  e_mode 0: out of out_type; 1: SwiGLU of the packed [gate | up] rows, N = I,
-// bfloat16 out; 2: add into the float32 residual `out` and write partial sums of squares
-// (RESID).  nt: weight-row tiles per workgroup: 1 or 2 (e_mode 1: 2 or 4, pairs).
-extern "C" int rl_gemm_skinny_ex(const void* X, int ldx, const float* R, int ldr, const int* xrows,
-                                 const float* ssq_in, int ssq_blocks, int ssq_stride,
-                                 const float* norm_w, float eps, const void* W, int ldw, void* out,
-                                 int ldo, float* ssq_out, int M, int N, int K, int x_mode,
-                                 int e_mode, int out_type, int nt, hipStream_t stream) {
-    if (M <= 0 || N <= 0) return RL_OK;
-    if (M > 16 || K < 8 || K % 8 || ldw % 8 || ldw < K || ldo < N) return RL_ERR_ARG;
-    if (x_mode == 0 && (!X || ldx % 8 || ldx < K)) return RL_ERR_ARG;
-    if (x_mode == 1 && (!R || !ssq_in || !norm_w || ldr % 4 || ldr < K || ssq_blocks < 1 ||
-                        (size_t)K * sizeof(float) > 48 * 1024))
-        return RL_ERR_ARG;
-    if (e_mode == 2 && !ssq_out) return RL_ERR_ARG;
-    SkinnyArgs a;
-    a.X = (const bf16_t*)X;
-    a.ldx = ldx;
-    a.R = R;
-    a.ldr = ldr;
-    a.xrows = xrows;
-    a.ssq_in = ssq_in;
-    a.ssq_blocks = ssq_blocks;
-    a.ssq_stride = ssq_stride;
-    a.norm_w = norm_w;
-    a.eps = eps;
-    a.W = (const bf16_t*)W;
-    a.ldw = ldw;
-    a.out = out;
-    a.ldo = ldo;
-    a.ssq_out = ssq_out;
-    a.M = M;
-    a.N = N;
-    a.K = K;
-#define RL_CASE(XM, EM, OT, NTV, OutT, SW, XN, RS)                                             \
-    if (x_mode == XM && e_mode == EM && (OT < 0 || out_type == OT) && nt == NTV)               \
-        return launch<NTV, OutT, SW, XN, RS>(a, stream);
-    RL_CASE(0, 0, RL_BF16, 1, bf16_t, false, false, false)
-    RL_CASE(0, 0, RL_BF16, 2, bf16_t, false, false, false)
-    RL_CASE(0, 0, RL_F32, 1, float, false, false, false)
-    RL_CASE(0, 0, RL_F32, 2, float, false, false, false)
-    RL_CASE(1, 0, RL_BF16, 1, bf16_t, false, true, false)
-    RL_CASE(1, 0, RL_BF16, 2, bf16_t, false, true, false)
-    RL_CASE(1, 0, RL_F32, 1, float, false, true, false)
-    RL_CASE(1, 0, RL_F32, 2, float, false, true, false)
-    RL_CASE(0, 1, -1, 2, bf16_t, true, false, false)
-    RL_CASE(0, 1, -1, 4, bf16_t, true, false, false)
-    RL_CASE(1, 1, -1, 2, bf16_t, true, true, false)
-    RL_CASE(1, 1, -1, 4, bf16_t, true, true, false)
-    RL_CASE(0, 2, -1, 1, float, false, false, true)
-    RL_CASE(0, 2, -1, 2, float, false, false, true)
+template <typename OutT, bool SWIGLU>
+static int dispatch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
+                    int ldw, int ldo, int nt, hipStream_t stream) {
+#define RL_CASE(NTV)                                                                           \
+    if (nt == NTV) return launch<NTV, OutT, SWIGLU>(X, W, out, M, N, K, ldx, ldw, ldo, stream);
+    if (SWIGLU) {
+        RL_CASE(2) RL_CASE(4)
+    } else {
+        RL_CASE(1) RL_CASE(2)
+    }
 #undef RL_CASE
     return RL_ERR_ARG;
 }
@@ -370,13 +231,24 @@ extern "C" int rl_gemm_skinny_ex(const void* X, int ldx, const float* R, int ldr
 extern "C" int rl_gemm_skinny(const void* X, const void* W, void* out, int M, int N, int K,
                               int ldx, int ldw, int ldo, int out_type, int nt,
                               hipStream_t stream) {
-    return rl_gemm_skinny_ex(X, ldx, nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0.f, W, ldw, out,
-                             ldo, nullptr, M, N, K, 0, 0, out_type, nt, stream);
+    if (M <= 0 || N <= 0) return RL_OK;
+    if (M > 16 || K < 8 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < N)
+        return RL_ERR_ARG;
+    if (out_type == RL_F32)
+        return dispatch<float, false>((const bf16_t*)X, (const bf16_t*)W, (float*)out, M, N, K,
+                                      ldx, ldw, ldo, nt, stream);
+    if (out_type == RL_BF16)
+        return dispatch<bf16_t, false>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, N, K,
+                                       ldx, ldw, ldo, nt, stream);
+    return RL_ERR_ARG;
 }
 
 // out[M, I] = silu(X Wg^T) * (X Wu^T) with W = [Wg | Wu] stacked by rows, [2I, K].
 extern "C" int rl_gemm_skinny_swiglu(const void* X, const void* W, void* out, int M, int I, int K,
                                      int ldx, int ldw, int ldo, int nt, hipStream_t stream) {
-    return rl_gemm_skinny_ex(X, ldx, nullptr, 0, nullptr, nullptr, 0, 0, nullptr, 0.f, W, ldw, out,
-                             ldo, nullptr, M, I, K, 0, 1, RL_BF16, nt, stream);
+    if (M <= 0 || I <= 0) return RL_OK;
+    if (M > 16 || K < 8 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < I)
+        return RL_ERR_ARG;
+    return dispatch<bf16_t, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx,
+                                  ldw, ldo, nt, stream);
 }

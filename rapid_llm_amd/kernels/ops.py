@@ -8,7 +8,6 @@ GPU or without the compiled library these raise.
 from __future__ import annotations
 
 import ctypes
-from dataclasses import dataclass
 from typing import Optional
 
 import torch
@@ -340,146 +339,48 @@ def _skinny_tiles(rows: int, out_features: int) -> int:
     return 2 if rows > 4 and -(-out_features // 32) >= _MIN_BLOCKS else 1
 
 
-@dataclass
-class ResidualUpdate:
-    """What a product returns when it added its result into the residual stream itself
-    (``gemm_bf16_add``): the residual, and per workgroup and row the sum of squares of the
-    values it wrote there, ``ssq [workgroups, rows]``."""
-
-    residual: torch.Tensor
-    ssq: torch.Tensor
-
-
-@dataclass
-class NormedRows:
-    """Rows of the residual stream to be normalised, not yet computed: a product that takes
-    them (``gemm_bf16``, ``gemm_bf16_swiglu``) normalises while it loads; anything else calls
-    :meth:`materialize`."""
-
-    update: ResidualUpdate
-    weight: torch.Tensor
-    eps: float
-    rows: Optional[torch.Tensor]  # int32 residual rows to produce (None: all)
-    dtype: torch.dtype
-
-    @property
-    def shape(self) -> tuple[int, int]:
-        n = self.update.residual.shape[0] if self.rows is None else self.rows.numel()
-        return (n, self.update.residual.shape[1])
-
-    @property
-    def device(self) -> torch.device:
-        return self.update.residual.device
-
-    def materialize(self) -> torch.Tensor:
-        res, ssq = self.update.residual, self.update.ssq
-        out = torch.empty(self.shape, dtype=self.dtype, device=res.device)
-        _ok(
-            core().rl_apply_norm(
-                _p(res), _p(ssq), ssq.shape[0], ssq.stride(0), _p(self.weight), _p(out), _p(self.rows),
-                out.shape[0], res.shape[1], ctypes.c_float(self.eps), _tag(self.dtype), _stream(),
-            ),
-            "rl_apply_norm",
-        )
-        return out
-
-
-_XNORM_MAX_K = 48 * 1024 // 4  # the fused norm keeps the norm's weights in LDS
-
-
-def _skinny_ex(x, w, out, m, n, k, *, e_mode: int, nt: int, ssq_out=None) -> None:
-    """One launch of the skinny product; ``x`` a bfloat16 matrix or :class:`NormedRows`."""
-    lazy = isinstance(x, NormedRows)
-    if lazy:
-        res, ssq = x.update.residual, x.update.ssq
-        args = (None, 0, _p(res), res.stride(0), _p(x.rows), _p(ssq), ssq.shape[0], ssq.stride(0),
-                _p(x.weight), ctypes.c_float(x.eps))
-    else:
-        args = (_p(x), k, None, 0, None, None, 0, 0, None, ctypes.c_float(0.0))
-    _ok(
-        core().rl_gemm_skinny_ex(
-            *args, _p(w), k, _p(out), out.stride(0), _p(ssq_out), m, n, k, int(lazy), e_mode,
-            _tag(out.dtype), nt, _stream(),
-        ),
-        "rl_gemm_skinny_ex",
-    )
-
-
-def _skinny_input(x, w: torch.Tensor):
-    """``x`` as the skinny product can take it, or ``None`` if this shape goes elsewhere."""
-    m, k = x.shape
-    if m > SKINNY_MAX_ROWS or k % 8 or w.dtype != torch.bfloat16:
-        return None
-    if isinstance(x, NormedRows):
-        if k > _XNORM_MAX_K or x.dtype != torch.bfloat16:
-            return x.materialize()
-        return x
-    return x if x.dtype == torch.bfloat16 else None
-
-
-def gemm_bf16(x, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     """``x[M,K] @ w[N,K]^T`` with bfloat16 operands and float32 accumulation.
 
     Up to 16 rows (decode) run the hand-written bandwidth-bound kernel, which can write
-    float32 directly and can take its rows as :class:`NormedRows`.  More rows go to the
-    library product, as the reference's dense products do (``F.linear``); its bfloat16 result
-    is returned as is and widened by the caller."""
+    float32 directly.  More rows go to the library product, as the reference's dense products do
+    (``F.linear``); its bfloat16 result is returned as is and widened by the caller."""
+    _need(x, "x", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
     m, k = x.shape
     n = w.shape[0]
     if k != w.shape[1]:
         raise KernelError(f"gemm_bf16 shapes do not agree: x {tuple(x.shape)}, w {tuple(w.shape)}")
-    xs = _skinny_input(x, w)
-    if xs is not None:
+    if m <= SKINNY_MAX_ROWS and k % 8 == 0:
         if out_dtype not in (torch.bfloat16, torch.float32):
             raise KernelError(f"gemm_bf16 writes bfloat16 or float32, not {out_dtype}")
-        if not isinstance(xs, NormedRows):
-            _need(xs, "x", torch.bfloat16)
-        out = torch.empty((m, n), dtype=out_dtype, device=w.device)
-        _skinny_ex(xs, w, out, m, n, k, e_mode=0, nt=_skinny_tiles(m, n))
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        nt = _skinny_tiles(m, n)
+        _ok(
+            core().rl_gemm_skinny(_p(x), _p(w), _p(out), m, n, k, k, k, n, _tag(out_dtype), nt, _stream()),
+            "rl_gemm_skinny",
+        )
         return out
-    if isinstance(x, NormedRows):
-        x = x.materialize()
-    _need(x, "x", torch.bfloat16)
     return torch.matmul(x, w.t())
 
 
-def gemm_bf16_swiglu(x, w_gate_up: torch.Tensor) -> torch.Tensor | None:
+def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor | None:
     """``silu(x Wg^T) * (x Wu^T)`` for the packed ``[gate | up]`` matrix in one kernel, for
     few rows; ``None`` when the shape is not one the fused kernel takes."""
     m, k = x.shape
     two_i = w_gate_up.shape[0]
-    if two_i % 2 or w_gate_up.dtype != torch.bfloat16:
-        return None
-    xs = _skinny_input(x, w_gate_up)
-    if xs is None:
-        return None
-    _need(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, k))
-    inter = two_i // 2
-    out = torch.empty((m, inter), dtype=torch.bfloat16, device=w_gate_up.device)
-    nt = _skinny_tiles(m, inter) * 2  # pairs of (gate, up) tiles
-    _skinny_ex(xs, w_gate_up, out, m, inter, k, e_mode=1, nt=nt)
-    return out
-
-
-def gemm_bf16_add(x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor) -> ResidualUpdate | None:
-    """``residual += x @ w^T`` inside the product's epilogue (the product rounded to bfloat16
-    first, as when it is stored), for few rows; ``None`` when the shape is not one it takes."""
-    m, k = x.shape
-    n = w.shape[0]
-    if (
-        m > SKINNY_MAX_ROWS or k % 8 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16
-        or residual.dtype != torch.float32 or tuple(residual.shape) != (m, n)
-    ):
+    if m > SKINNY_MAX_ROWS or k % 8 or two_i % 2 or x.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16:
         return None
     _need(x, "x", torch.bfloat16)
-    _need(w, "w", torch.bfloat16, (n, k))
-    _need(residual, "residual", torch.float32, (m, n))
-    nt = _skinny_tiles(m, n)
-    blocks = core().rl_gemm_skinny_blocks(n, nt)
-    ssq = torch.empty((blocks, m), dtype=torch.float32, device=x.device)
-    _skinny_ex(x, w, residual, m, n, k, e_mode=2, nt=nt, ssq_out=ssq)
-    return ResidualUpdate(residual, ssq)
+    _need(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, k))
+    inter = two_i // 2
+    out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
+    nt = _skinny_tiles(m, inter) * 2  # pairs of (gate, up) tiles
+    _ok(
+        core().rl_gemm_skinny_swiglu(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, _stream()),
+        "rl_gemm_skinny_swiglu",
+    )
+    return out
 
 
 class AttentionPlan:

@@ -19,7 +19,6 @@ from ..parts.base import (
     CacheNeed,
     ParamSpec,
 )
-from ..parts.block import run_norm
 from ..parts.embedding import OutputProjection, TokenEmbedding
 from .spec import ModelSpec
 
@@ -124,7 +123,7 @@ class CausalLM:
             delta = self.blocks[li].forward(residual, delta, ctx, caches[place])
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=residual.device)
-        h = run_norm(self.final_norm, residual, delta, ctx, rows=ctx.logit_rows)
+        h = self.final_norm.forward(residual, delta, ctx, rows=ctx.logit_rows)
         return self.output.forward(h)
 
 

@@ -24,8 +24,6 @@ from .linear import Linear
 
 
 class GQAAttention(Mixer):
-    fuses_residual = True
-
     def __init__(
         self,
         hidden_size: int,
@@ -95,7 +93,7 @@ class GQAAttention(Mixer):
         return CacheNeed("kv", window=self.window, num_kv_heads=self.nkv, head_dim=self.d)
 
     # ---- step ------------------------------------------------------------------
-    def forward(self, x, ctx, cache, residual=None):
+    def forward(self, x, ctx, cache):
         tokens = x.shape[0]
         qkv = self.qkv(x)
         table = ctx.block_tables[cache.group_id]
@@ -103,7 +101,7 @@ class GQAAttention(Mixer):
         cos = pos_enc.cos if pos_enc is not None else None
         sin = pos_enc.sin if pos_enc is not None else None
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        out = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
+        out = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         rotary_half = cos.shape[1] if cos is not None else 0
         if ops.decode_attention_fusable(ctx, qkv.dtype, self.nq // self.nkv, self.d, rotary_half):
             # a step of single tokens: norm, rotation, cache write and attention in one kernel
@@ -111,8 +109,8 @@ class GQAAttention(Mixer):
                 qkv, cache.k, cache.v, out, ctx, table, cache.page_size, self.nq, self.nkv, self.d,
                 self.window, self.scale, self.q_norm_w, self.k_norm_w, cos, sin, eps, cache.owns_pages,
             )
-            return self.o(out, add_to=residual)
-        q = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
+            return self.o(out)
+        q = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         ops.qknorm_rope_kvwrite(
             qkv, q,
             cache.k if cache.owns_pages else None,
@@ -125,7 +123,7 @@ class GQAAttention(Mixer):
             q, cache.k, cache.v, out, ctx, table, cache.page_size,
             self.nq, self.nkv, self.d, self.window, self.scale,
         )
-        return self.o(out, add_to=residual)
+        return self.o(out)
 
 
 MIXERS.register("gqa_attention", GQAAttention)

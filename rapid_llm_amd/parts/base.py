@@ -108,14 +108,6 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    #: A part that sets this takes two liberties the block then offers it.  Its input may be
-    #: :class:`~rapid_llm_amd.kernels.ops.NormedRows`, a norm not yet computed, which a
-    #: product can compute while it loads; and it receives ``residual=``, the float32 stream,
-    #: into which its last product may add its result itself, returning a
-    #: :class:`~rapid_llm_amd.kernels.ops.ResidualUpdate` instead of a matrix.  Both save a
-    #: kernel in steps of few tokens; a part that leaves the flag alone never sees either.
-    fuses_residual = False
-
     def cache_need(self) -> CacheNeed:
         return CacheNeed("none")
 
@@ -127,18 +119,11 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    fuses_residual = False  # see Mixer.fuses_residual
-
     def forward(self, x: "torch.Tensor", ctx: "StepContext") -> "torch.Tensor":
         raise NotImplementedError
 
 
 class Norm(Part):
-    #: A norm that sets this accepts a :class:`~rapid_llm_amd.kernels.ops.ResidualUpdate` as
-    #: ``delta`` (the add has happened already) and may then answer with
-    #: :class:`~rapid_llm_amd.kernels.ops.NormedRows`.  Other norms get ``delta=None`` then.
-    accepts_update = False
-
     def forward(
         self,
         residual: "torch.Tensor",

@@ -30,18 +30,11 @@ class Linear:
             )
         self.weight = weight
 
-    def __call__(self, x, out_dtype: torch.dtype | None = None, add_to: torch.Tensor | None = None):
-        """``x`` is a matrix or :class:`~rapid_llm_amd.kernels.ops.NormedRows`.  With
-        ``add_to`` (the float32 residual stream) the product may add its result there itself
-        and return a :class:`~rapid_llm_amd.kernels.ops.ResidualUpdate`; it returns the plain
-        result when the shape is not one that kernel takes."""
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
         w = self.weight
-        lazy = isinstance(x, ops.NormedRows)
         rows = x.shape[0]
+        out_dtype = out_dtype or x.dtype
         if w.dtype == torch.float32:
-            if lazy:
-                x = x.materialize()
-            out_dtype = out_dtype or x.dtype
             if x.dtype != torch.float32:
                 wide = torch.empty(x.shape, dtype=torch.float32, device=x.device)
                 ops.cast(x, wide)
@@ -49,11 +42,6 @@ class Linear:
             y = torch.empty((rows, self.out_features), dtype=torch.float32, device=x.device)
             ops.gemm_f32(x, w, y)
         else:
-            out_dtype = out_dtype or x.dtype
-            if add_to is not None and not lazy:
-                update = ops.gemm_bf16_add(x, w, add_to)
-                if update is not None:
-                    return update
             y = ops.gemm_bf16(x, w, out_dtype)
         if y.dtype != out_dtype:
             narrow = torch.empty(y.shape, dtype=out_dtype, device=y.device)

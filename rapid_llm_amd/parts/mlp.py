@@ -15,8 +15,6 @@ from .linear import Linear
 
 
 class SwiGLU(FeedForward):
-    fuses_residual = True
-
     def __init__(
         self,
         hidden_size: int,
@@ -47,16 +45,16 @@ class SwiGLU(FeedForward):
         self.gate_up.bind(params[self.name + ".gate_up"])
         self.down.bind(params[self.name + ".down"])
 
-    def forward(self, x, ctx, residual=None):
+    def forward(self, x, ctx):
         w = self.gate_up.weight
-        if w.dtype == torch.bfloat16:
+        if w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
             act = ops.gemm_bf16_swiglu(x, w)  # few rows: product and activation in one kernel
             if act is not None:
-                return self.down(act, add_to=residual)
+                return self.down(act)
         gu = self.gate_up(x)
-        act = torch.empty((gu.shape[0], self.intermediate_size), dtype=gu.dtype, device=gu.device)
+        act = torch.empty((x.shape[0], self.intermediate_size), dtype=gu.dtype, device=x.device)
         ops.swiglu(gu, act)
-        return self.down(act, add_to=residual)
+        return self.down(act)
 
 
 FEED_FORWARDS.register("swiglu", SwiGLU)

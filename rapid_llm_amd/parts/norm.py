@@ -15,8 +15,6 @@ from .base import NORMS, Norm, ParamSpec, Source
 
 
 class RMSNorm(Norm):
-    accepts_update = True
-
     def __init__(self, size: int, eps: float, checkpoint_name: str, name: str = "norm") -> None:
         self.size = size
         self.eps = float(eps)
@@ -40,12 +38,6 @@ class RMSNorm(Norm):
         self.dtype = runtime.dtype
 
     def forward(self, residual, delta, ctx, rows=None):
-        if isinstance(delta, ops.ResidualUpdate):
-            # the product that made the addend added it and left the sums of squares: the
-            # norm is computed by whoever consumes it
-            if delta.residual is not residual:
-                raise ValueError("the update belongs to another residual stream")
-            return ops.NormedRows(delta, self.weight, self.eps, rows, self.dtype)
         n = residual.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=self.dtype, device=residual.device)
         ops.add_rmsnorm(residual, delta, self.weight, out, self.eps, rows)

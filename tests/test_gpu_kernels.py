@@ -406,46 +406,3 @@ def test_decode_attention_fused(case, normed):
     for i, a in enumerate(cached):
         same[int(table[slots[i], a // page]), :, a % page, :] = True
     assert same.all()
-
-
-@pytest.mark.parametrize("shape", [(1, 96, 64), (8, 4096, 4096), (16, 200, 1000), (5, 112, 200), (3, 4096, 12288)])
-def test_product_adds_into_the_residual_and_next_product_norms(shape):
-    """The two fusions of a decode step: a product that adds its result into the float32
-    residual and leaves partial sums of squares, and products that read the residual
-    normalised on the fly (all rows, chosen rows, with SwiGLU), against the plain formulas."""
-    ops = _ops()
-    m, n, k = shape
-    gen = torch.Generator().manual_seed(n + k)
-    x = torch.randn(m, k, generator=gen).bfloat16()
-    w = (torch.randn(n, k, generator=gen) / math.sqrt(k)).bfloat16()
-    res = torch.randn(m, n, generator=gen)
-    res_dev = res.to(DEV)
-    update = ops.gemm_bf16_add(x.to(DEV), w.to(DEV), res_dev)
-    assert update is not None and update.residual is res_dev
-    want_res = res + (x.float() @ w.float().T).bfloat16().float()
-    torch.testing.assert_close(res_dev.cpu(), want_res, rtol=0, atol=2e-2)  # bfloat16 rounding of the addend
-    got_res = res_dev.cpu()
-    torch.testing.assert_close(update.ssq.sum(0).cpu(), got_res.square().sum(-1), rtol=1e-5, atol=1e-5)
-    # shapes the kernel refuses come back as None, with the residual untouched
-    assert ops.gemm_bf16_add(torch.zeros(17, k, dtype=torch.bfloat16, device=DEV), w.to(DEV),
-                             torch.zeros(17, n, device=DEV)) is None
-
-    norm_w = (1 + 0.1 * torch.randn(n, generator=gen)).to(DEV)
-    eps = 2e-5
-    normed = plain_rmsnorm(got_res, norm_w.cpu(), eps)
-    n2 = 176
-    w2 = (torch.randn(2 * n2, n, generator=gen) / math.sqrt(n)).bfloat16()
-    for rows in (None, torch.tensor([m - 1, 0], dtype=torch.int32)):
-        lazy = ops.NormedRows(update, norm_w, eps, None if rows is None else rows.to(DEV), torch.bfloat16)
-        want_x = (normed if rows is None else normed[rows.long()]).bfloat16().float()
-        torch.testing.assert_close(lazy.materialize().float().cpu(), want_x, rtol=8e-3, atol=8e-3)
-        assert lazy.shape == tuple(want_x.shape)
-        for out_dtype in (torch.bfloat16, torch.float32):
-            got = ops.gemm_bf16(lazy, w2.to(DEV), out_dtype)
-            assert got.dtype == out_dtype
-            torch.testing.assert_close(got.float().cpu(), want_x @ w2.float().T, rtol=2e-2, atol=2e-2)
-        if n % 8 == 0:
-            gu = (want_x @ w2.float().T).bfloat16().float()
-            want_act = torch.nn.functional.silu(gu[:, :n2]) * gu[:, n2:]
-            got = ops.gemm_bf16_swiglu(lazy, w2.to(DEV))
-            torch.testing.assert_close(got.float().cpu(), want_act, rtol=3e-2, atol=3e-2)
