@@ -129,7 +129,10 @@ __device__ inline bf16x8 softmax_step(f32x4 s0, f32x4 s1, unsigned ok0, unsigned
 // =========================================================================== //
 // decode
 // =========================================================================== //
-#define DEC_WAVES 4
+#ifndef RL_DEC_WAVES
+#define RL_DEC_WAVES 4
+#endif
+#define DEC_WAVES RL_DEC_WAVES
 #define DEC_MAX_PAGES 1024  // pages one split may span (their ids are staged in LDS)
 
 // Keys of one 32-key step as the two matrix products see them.  Tile row i of key block kb
@@ -211,9 +214,9 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
     const int* __restrict__ positions, const int* __restrict__ token_slot,
     const int* __restrict__ block_table, int table_stride, int page_size, int nq, int nkv,
     int window, float scale_log2, int split_chunk, int nsplit, DecodeExtra ex) {
-    __shared__ float lds_o[2][D * 16];
-    __shared__ float lds_m[2][16];
-    __shared__ float lds_l[2][16];
+    __shared__ float lds_o[DEC_WAVES / 2][D * 16];
+    __shared__ float lds_m[DEC_WAVES / 2][16];
+    __shared__ float lds_l[DEC_WAVES / 2][16];
     __shared__ int lds_pages[DEC_MAX_PAGES + 2];
 
     const int G = nq / nkv;
@@ -404,7 +407,7 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
             cur = nxt;
         }
 
-        // ---- combine the waves: (2,3) -> (0,1), then 1 -> 0, in the accumulators' own layout --
+        // ---- combine the waves pairwise, in the accumulators' own layout --------------------
         l = row_sum4(l);
         auto put = [&](int slot) {
             if (g == 0) {
@@ -431,14 +434,15 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
             l = l * f1 + l_o * f2;
             m = mm;
         };
-        if (wave >= 2) put(wave - 2);
-        __syncthreads();
-        if (wave < 2) take(wave);
-        __syncthreads();
-        if (wave == 1) put(0);
-        __syncthreads();
+        // waves [s, 2s) hand their state to waves [0, s), for s = DEC_WAVES / 2, .., 1
+#pragma unroll
+        for (int s = DEC_WAVES / 2; s >= 1; s >>= 1) {
+            if (wave >= s && wave < 2 * s) put(wave - s);
+            __syncthreads();
+            if (wave < s) take(wave);
+            if (s > 1) __syncthreads();
+        }
         if (wave != 0) return;
-        take(0);
     } else if (wave != 0) {
         return;
     }
