@@ -32,7 +32,7 @@ class LayerCache:
     k: torch.Tensor | None  # [pages, kv_heads, page_size, head_dim]
     v: torch.Tensor | None  # [pages, kv_heads, head_dim, page_size]
     owns_pages: bool  # False: reads another layer's pages and must not write them
-    state: torch.Tensor | None  # [max_seqs, *state_shape], zeroed when a slot is taken
+    state: torch.Tensor | None  # [max_seqs + 1, *state_shape], zeroed when a slot is taken
 
 
 def plan_groups(needs: list[CacheNeed]) -> tuple[list[GroupSpec], list[int | None]]:
@@ -103,14 +103,19 @@ class DeviceCache:
             state = None
             if need.state_shape is not None:
                 sdt = getattr(torch, need.state_dtype) if need.state_dtype else dtype
-                state = torch.zeros((manager.max_seqs, *need.state_shape), dtype=sdt, device=device)
+                state = torch.zeros((manager.max_seqs + 1, *need.state_shape), dtype=sdt, device=device)
             self.layers.append(LayerCache(i, gid, P, k, v, owns, state))
         for i, need in enumerate(needs):
             if need.kind == "kv" and need.share_with is not None:
                 src = self.layers[need.share_with]
                 self.layers[i].k, self.layers[i].v = src.k, src.v
+        # One row more than there are slots: the filler slot, whose row maps every position to
+        # the null page for good.  Rows that only pad a batch to a captured size name it (the
+        # reference keeps its last table row for the same purpose,
+        # rapid_llm/executor/slot_batch.py:97-100).
+        self.filler_slot = manager.max_seqs
         self.tables: dict[int, torch.Tensor] = {
-            gid: torch.zeros(tab.shape, dtype=torch.int32, device=device)
+            gid: torch.zeros((tab.shape[0] + 1, tab.shape[1]), dtype=torch.int32, device=device)
             for gid, tab in manager.tables.items()
         }
 

@@ -9,6 +9,8 @@ Options that the reference's command line has keep their spelling and meaning
 
 * ``batch``   run a file of prompts through the continuous-batching engine;
 * ``chat``    a read-eval-print loop with streamed output (``/clear``, ``exit``);
+* ``bench``   offline generation speed of a model folder with synthetic prompts of exact token
+  lengths: TTFT, TPOT, TPS and TGS as the reference defines them (docs/benchmark_models.md:141-149);
 * ``init``    write a model folder with random weights from a config.json and a seed;
 * ``replay``  feed given token ids step by step and write logits (the same as ``bin/trace_run``).
 """
@@ -157,6 +159,53 @@ def cmd_chat(args) -> int:
     return 0
 
 
+def cmd_bench(args) -> int:
+    """All prompts submitted at once, run to completion, timed between device
+    synchronisations: TTFT = time to the first token of the batch, TPOT = (latency - TTFT) /
+    (output_len - 1), TPS = 1000 / TPOT per request, TGS = all output tokens / latency.
+    Prompts are uniform random token ids of exactly ``--input-len`` tokens, as the
+    reference's RandomDataset makes them (rapid_llm/benchmark/datasets/random.py:70-110)."""
+    import random
+    import statistics
+
+    import torch
+
+    from .sampling.params import SamplingParams
+
+    engine = _engine(args, args.batch_size)
+    vocab = engine.runner.vocab_size
+    rng = random.Random(args.seed)
+    params = SamplingParams(temperature=0.0, max_gen_len=args.gen_len, ignore_eos=True)
+    rows = []
+    for it in range(args.warmup + args.iterations):
+        prompts = [[rng.randrange(vocab) for _ in range(args.input_len)] for _ in range(args.batch_size)]
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        requests = [engine.add_request(p, params) for p in prompts]
+        ttft = None
+        while engine.has_unfinished_requests():
+            engine.step()
+            if ttft is None and all(r.output_token_ids for r in requests):
+                torch.cuda.synchronize()
+                ttft = time.perf_counter() - start
+        torch.cuda.synchronize()
+        latency = time.perf_counter() - start
+        if it >= args.warmup:
+            rows.append((ttft, latency, sum(len(r.output_token_ids) for r in requests)))
+    ttft = statistics.median(r[0] for r in rows)
+    latency = statistics.median(r[1] for r in rows)
+    tokens = rows[0][2]
+    tpot = (latency - ttft) / max(1, args.gen_len - 1)
+    print(json.dumps({
+        "batch_size": args.batch_size, "input_len": args.input_len, "gen_len": args.gen_len,
+        "ttft_s": round(ttft, 4), "tpot_ms": round(tpot * 1e3, 3),
+        "tps": round(1.0 / tpot, 1) if tpot > 0 else None, "tgs": round(tokens / latency, 1),
+        "prefill_tok_s": round(args.batch_size * args.input_len / ttft, 1),
+        "preemptions": engine.num_preemptions,
+    }))
+    return 0
+
+
 def cmd_init(args) -> int:
     from .weights.random_init import write_random_model
 
@@ -190,6 +239,15 @@ def main(argv=None) -> int:
     chat = subs.add_parser("chat", help="Interactive loop with streamed output")
     _common(chat, graph_default=False)
     chat.set_defaults(fn=cmd_chat)
+
+    bench = subs.add_parser("bench", help="Offline generation speed with synthetic prompts")
+    _common(bench, graph_default=True)
+    bench.add_argument("--batch-size", type=int, default=8)
+    bench.add_argument("--input-len", type=int, default=128)
+    bench.add_argument("--gen-len", type=int, default=128)
+    bench.add_argument("--iterations", type=int, default=3)
+    bench.add_argument("--warmup", type=int, default=1)
+    bench.set_defaults(fn=cmd_bench)
 
     init = subs.add_parser("init", help="Write a model folder with random weights")
     init.add_argument("--config", required=True, help="a config.json")

@@ -33,6 +33,8 @@ from ..weights.loader import load_model_dir
 from ..weights.random_init import random_params
 
 _TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+# batch sizes decode graphs are captured for; other sizes are padded up with filler rows
+GRAPH_BATCHES = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 
 
 class OutOfPages(CacheError):
@@ -284,20 +286,47 @@ class ModelRunner:
         )
 
     # ------------------------------------------------------------------ decode graphs
-    def _graph_step(self, entries, host, offs, meta) -> torch.Tensor:
-        """A step of single tokens, all wanted: replayed from a HIP graph captured once per
-        batch size.  The graph holds only this package's kernels; its inputs are one static
-        int32 buffer, refreshed by a copy on the same stream before each replay.  Launch
-        decisions that depend on the context length are made for the bucket's longest context,
-        so one capture serves every step of that bucket."""
+    def _padded_decode(self, meta: dict, token_ids: list[int], rows: int):
+        """The packed upload of a step of single tokens, padded to ``rows`` rows with filler
+        rows: token 0 at position 0 of the filler slot, whose block-table row is the null page."""
+        n = meta["num_seqs"]
+        pad = rows - n
+        filler = self.device_cache.filler_slot
+        ids = np.asarray(token_ids + [0] * pad, dtype=np.int32)
+        starts = np.asarray(meta["h_seq_starts"] + [0] * pad, dtype=np.int32)
+        slots = np.asarray(meta["h_seq_slots"] + [filler] * pad, dtype=np.int32)
+        ones = np.ones(rows, dtype=np.int32)
+        arange = np.arange(rows + 1, dtype=np.int32)
+        # ids | positions | token_slot | slots | starts | lens | cu | rows  (as _prepare lays it out)
+        host = np.concatenate([ids, starts, slots, slots, starts, ones, arange, arange[:rows]])
+        sizes = [rows, rows, rows, rows, rows, rows, rows + 1, rows]
+        offs = np.concatenate(([0], np.cumsum(sizes)))
+        padded = dict(
+            meta, num_tokens=rows, num_seqs=rows, num_logit_rows=rows,
+            h_seq_slots=meta["h_seq_slots"] + [filler] * pad,
+            h_seq_starts=meta["h_seq_starts"] + [0] * pad,
+            h_seq_lens=[1] * rows,
+        )
+        return host, offs, padded
+
+    def _graph_step(self, entries, meta) -> torch.Tensor:
+        """A step of single tokens, all wanted: replayed from a HIP graph.  Graphs exist for a
+        ladder of batch sizes and for context buckets (the next power of two); a batch is
+        padded with filler rows to the next size of the ladder, so that a few captures serve
+        every batch a scheduler produces.  The graph holds only this package's kernels (and
+        the library's products above 16 rows); its inputs are one static int32 buffer,
+        refreshed by a copy on the same stream before each replay.  Launch decisions that
+        depend on the context length are made for the bucket's longest context."""
         batch = len(entries)
-        # one graph per batch size and context bucket (the next power of two): the split of
-        # the keys over workgroups is fixed at capture and should fit the contexts it serves
+        rows = next(b for b in GRAPH_BATCHES if b >= batch)
+        host, offs, meta = self._padded_decode(meta, [int(e.tokens[0]) for e in entries], rows)
+        # the split of the keys over workgroups is fixed at capture and should fit the contexts
+        # it serves
         bound = 512
         while bound <= meta["max_position"]:
             bound *= 2
         bound = min(bound, self.engine.max_seq_len)
-        key = (batch, bound)
+        key = (rows, bound)
         entry = self._graphs.get(key)
         if entry is None:
             static = torch.zeros(len(host), dtype=torch.int32, device=self.device)
@@ -305,7 +334,7 @@ class ModelRunner:
             pinned.numpy()[:] = host
             static.copy_(pinned, non_blocking=True)
             ctx = self._context(static, offs, dict(meta, max_position=bound - 1))
-            ctx.extra["decode_only_tokens"] = torch.arange(batch, dtype=torch.int32, device=self.device)
+            ctx.extra["decode_only_tokens"] = torch.arange(rows, dtype=torch.int32, device=self.device)
             ctx.extra["context_bound"] = bound
             # one eager run on a side stream first: kernels get loaded, the allocator warm
             current = torch.cuda.current_stream()
@@ -328,7 +357,7 @@ class ModelRunner:
         pinned.numpy()[:] = host
         static.copy_(pinned, non_blocking=True)
         graph.replay()
-        return logits
+        return logits[:batch]
 
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry], use_graph: bool | None = None) -> torch.Tensor:
@@ -342,10 +371,10 @@ class ModelRunner:
         host, offs, meta = self._prepare(entries)
         if (
             (self.engine.use_graph if use_graph is None else use_graph)
-            and len(entries) <= ops.GRAPH_MAX_ROWS
+            and len(entries) <= GRAPH_BATCHES[-1]
             and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
         ):
-            logits = self._graph_step(entries, host, offs, meta)
+            logits = self._graph_step(entries, meta)
         else:
             dev = torch.from_numpy(host).to(self.device, non_blocking=False)
             logits = self.model.forward(self._context(dev, offs, meta), self.device_cache.layers)

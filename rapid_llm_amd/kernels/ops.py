@@ -328,7 +328,6 @@ def sample_uniform(seed: int, counter: int) -> float:
 
 
 SKINNY_MAX_ROWS = 16  # rows up to which the hand-written bandwidth-bound product is used
-GRAPH_MAX_ROWS = 64  # decode batches up to this size are replayed from HIP graphs
 _MIN_BLOCKS = 512  # workgroups a skinny product should keep when it widens its tiles
 
 

@@ -154,6 +154,18 @@ def test_command_line_batch(tmp_path, capsys):
     assert str(_plain_generate(pcfg, pw, [1, 2, 3, 4], 6)) in text
 
 
+def test_command_line_bench(tmp_path, capsys):
+    import json
+
+    from rapid_llm_amd.cli import main
+
+    model_dir = make_model_dir(tmp_path, "D", "bfloat16")
+    code = main(["bench", "--model-dir", str(model_dir), "--max-seq-len", "128", "--batch-size", "5",
+                 "--input-len", "40", "--gen-len", "12", "--iterations", "2", "--warmup", "1"])
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert code == 0 and line["batch_size"] == 5 and line["tgs"] > 0 and line["ttft_s"] > 0 and line["tpot_ms"] > 0
+
+
 def test_smoke_entry():
     import __graft_entry__
 

@@ -101,4 +101,27 @@ def test_graph_of_a_batch_beyond_the_skinny_product(tmp_path, batch):
             eager.finish("x")
         for k, rid in enumerate(nxt):
             nxt[rid] = int(a[k].argmax())
-    assert any(key[0] == batch for key in graph._graphs)
+    assert any(key[0] >= batch for key in graph._graphs)  # padded up to a size of the ladder
+
+
+def test_ragged_batches_share_a_few_graphs(tmp_path):
+    """Requests that end at different times walk the batch size down one by one: the steps are
+    padded with filler rows to a ladder of sizes, so few graphs are captured, and the tokens
+    are those of an engine without graphs."""
+    from rapid_llm_amd import LLM, SamplingParams
+
+    cfg, page, seed = TINY["D"]
+    model_dir = make_model_dir(tmp_path, "D", "bfloat16")
+    prompts = [random_tokens(3 + i, cfg["vocab_size"], seed + i) for i in range(11)]
+    params = [SamplingParams(temperature=0.0, max_gen_len=4 + 3 * i) for i in range(11)]
+    outs = {}
+    for graph in (False, True):
+        llm = LLM(str(model_dir), dtype="bfloat16", max_seq_len=128, page_size=page, num_pages=200,
+                  max_num_seqs=16, use_cuda_graph=graph)
+        outs[graph] = [o.token_ids for o in llm.generate(prompts, params)]
+        if graph:
+            sizes = sorted({key[0] for key in llm.scheduler.runner._graphs})
+            assert sizes and set(sizes) <= {1, 2, 4, 8, 12, 16}, sizes
+    same = sum(a == b for a, b in zip(outs[False], outs[True]))
+    assert same >= 9, (outs[False], outs[True])  # bfloat16: a near-tie may fall the other way
+    assert [len(o) for o in outs[True]] == [4 + 3 * i for i in range(11)]
