@@ -86,6 +86,7 @@ class _Request:
     request_id: str
     slot: int
     reserved: int = 0  # positions [0, reserved) are addressable in every group
+    capacity: int = 0  # positions the mapped pages reach to (reserved rounded up to whole pages)
     trimmed: list[int] = field(default_factory=list)  # per group: pages below this index were returned
 
 
@@ -146,7 +147,7 @@ class CacheManager:
         if not self._free_slots:
             return None
         slot = self._free_slots.pop()
-        self._requests[request_id] = _Request(request_id, slot, 0, [0] * len(self.groups))
+        self._requests[request_id] = _Request(request_id, slot, trimmed=[0] * len(self.groups))
         self.fresh_slots.add(slot)
         return slot
 
@@ -182,6 +183,11 @@ class CacheManager:
                 f"request {request_id!r} asks for {upto} positions; the cache is laid out for "
                 f"sequences of at most {self.max_seq_len}"
             )
+        if upto <= req.capacity:
+            # the pages that were mapped last reach that far (a decoded token needs a new page
+            # only every page_size-th step); pages a window has passed stay returned
+            req.reserved = max(req.reserved, upto)
+            return True
         if start is None:
             start = req.reserved
         need = self.pages_needed(request_id, upto, start)
@@ -201,6 +207,7 @@ class CacheManager:
                 row[i] = page
             self.dirty_slots.add(req.slot)
         req.reserved = max(req.reserved, upto)
+        req.capacity = max(req.capacity, last * self.page_size)
         return True
 
     def trim(self, request_id: str, next_position: int) -> int:

@@ -192,7 +192,9 @@ class ModelRunner:
         self.computed.pop(request_id, None)
 
     # ------------------------------------------------------------------ the step
-    def _prepare(self, entries: Sequence[StepEntry]):
+    def _prepare(self, entries: Sequence[StepEntry]) -> dict:
+        """Check the entries, take the slots and pages they need (all or none), bring the device
+        tables up to date; returns what the step knows about its batch on the host."""
         cache = self.cache
         seen = set()
         for e in entries:
@@ -225,13 +227,32 @@ class ModelRunner:
                 raise CacheError("pages counted as free could not be taken")
 
         vocab = self.vocab_size
-        n_seq = len(entries)
         lens = [len(e.tokens) for e in entries]
-        total = sum(lens)
         starts = [self.computed.get(e.request_id, 0) for e in entries]
         slots = [cache.slot_of(e.request_id) for e in entries]
-        n_rows = sum(len(e.want) for e in entries)
-        # one packed int32 upload: ids | positions | token_slot | slots | starts | lens | cu | rows
+        for e in entries:
+            lo, hi = min(e.tokens), max(e.tokens)
+            if lo < 0 or hi >= vocab:
+                raise ValueError(
+                    f"request {e.request_id!r} has a token id outside [0, {vocab}): min {lo}, max {hi}"
+                )
+        self.device_cache.refresh()
+        return dict(
+            num_tokens=sum(lens),
+            num_seqs=len(entries),
+            num_logit_rows=sum(len(e.want) for e in entries),
+            h_seq_slots=slots,
+            h_seq_starts=starts,
+            h_seq_lens=lens,
+            max_position=max(s + n for s, n in zip(starts, lens)) - 1,
+            max_seq_tokens=max(lens),
+        )
+
+    @staticmethod
+    def _pack(entries: Sequence[StepEntry], meta: dict):
+        """One packed int32 upload: ids | positions | token_slot | slots | starts | lens | cu | rows."""
+        n_seq, total, n_rows = meta["num_seqs"], meta["num_tokens"], meta["num_logit_rows"]
+        lens, starts, slots = meta["h_seq_lens"], meta["h_seq_starts"], meta["h_seq_slots"]
         sizes = [total, total, total, n_seq, n_seq, n_seq, n_seq + 1, n_rows]
         offs = np.concatenate(([0], np.cumsum(sizes)))
         host = np.empty(int(offs[-1]), dtype=np.int32)
@@ -239,13 +260,7 @@ class ModelRunner:
         row = 0
         for i, e in enumerate(entries):
             n = lens[i]
-            toks = np.asarray(e.tokens, dtype=np.int64)
-            if toks.min() < 0 or toks.max() >= vocab:
-                raise ValueError(
-                    f"request {e.request_id!r} has a token id outside [0, {vocab}): "
-                    f"min {toks.min()}, max {toks.max()}"
-                )
-            host[offs[0] + cu : offs[0] + cu + n] = toks
+            host[offs[0] + cu : offs[0] + cu + n] = e.tokens
             host[offs[1] + cu : offs[1] + cu + n] = np.arange(starts[i], starts[i] + n)
             host[offs[2] + cu : offs[2] + cu + n] = slots[i]
             for w in e.want:
@@ -257,17 +272,7 @@ class ModelRunner:
         host[offs[3] : offs[4]] = slots
         host[offs[4] : offs[5]] = starts
         host[offs[5] : offs[6]] = lens
-        self.device_cache.refresh()
-        return host, offs, dict(
-            num_tokens=total,
-            num_seqs=n_seq,
-            num_logit_rows=n_rows,
-            h_seq_slots=slots,
-            h_seq_starts=starts,
-            h_seq_lens=lens,
-            max_position=max(s + n for s, n in zip(starts, lens)) - 1,
-            max_seq_tokens=max(lens),
-        )
+        return host, offs
 
     def _context(self, dev: torch.Tensor, offs, meta: dict) -> StepContext:
         part = [dev[offs[i] : offs[i + 1]] for i in range(len(offs) - 1)]
@@ -297,7 +302,7 @@ class ModelRunner:
         slots = np.asarray(meta["h_seq_slots"] + [filler] * pad, dtype=np.int32)
         ones = np.ones(rows, dtype=np.int32)
         arange = np.arange(rows + 1, dtype=np.int32)
-        # ids | positions | token_slot | slots | starts | lens | cu | rows  (as _prepare lays it out)
+        # ids | positions | token_slot | slots | starts | lens | cu | rows  (as _pack lays it out)
         host = np.concatenate([ids, starts, slots, slots, starts, ones, arange, arange[:rows]])
         sizes = [rows, rows, rows, rows, rows, rows, rows + 1, rows]
         offs = np.concatenate(([0], np.cumsum(sizes)))
@@ -368,7 +373,7 @@ class ModelRunner:
         ``use_graph`` overrides the engine's setting for this one step."""
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
-        host, offs, meta = self._prepare(entries)
+        meta = self._prepare(entries)
         if (
             (self.engine.use_graph if use_graph is None else use_graph)
             and len(entries) <= GRAPH_BATCHES[-1]
@@ -376,6 +381,7 @@ class ModelRunner:
         ):
             logits = self._graph_step(entries, meta)
         else:
+            host, offs = self._pack(entries, meta)
             dev = torch.from_numpy(host).to(self.device, non_blocking=False)
             logits = self.model.forward(self._context(dev, offs, meta), self.device_cache.layers)
         for e in entries:

@@ -34,7 +34,8 @@ def _runner(model_dir, dtype, page, **kw):
 
 
 def _context(runner, entries):
-    host, offs, meta = runner._prepare(entries)
+    meta = runner._prepare(entries)
+    host, offs = runner._pack(entries, meta)
     dev = torch.from_numpy(host).to(runner.device)
     return runner._context(dev, offs, meta)
 
