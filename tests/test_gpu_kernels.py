@@ -95,6 +95,8 @@ ATTN_CASES = [
     (4, 4, 256, 32, 0, [(90, 1), (0, 75)]),
     (6, 2, 64, 4, 19, [(0, 90), (45, 1), (200, 1), (30, 31)]),  # window
     (10, 5, 112, 12, 40, [(333, 1), (77, 50)]),
+    (8, 2, 128, 16, 0, [(20000, 1), (16000, 150), (9000, 1)]),  # long contexts: many splits, a long prefix
+    (4, 1, 64, 8, 3000, [(12000, 1), (5000, 40)]),               # a window deep in a long context
 ]
 
 
