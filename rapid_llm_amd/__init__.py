@@ -10,6 +10,7 @@ _LAZY = {
     "LLM": ("rapid_llm_amd.engine.llm", "LLM"),
     "Scheduler": ("rapid_llm_amd.engine.scheduler", "Scheduler"),
     "SamplingParams": ("rapid_llm_amd.sampling.params", "SamplingParams"),
+    "PositionLogprobs": ("rapid_llm_amd.sampling.logprobs", "PositionLogprobs"),
     "RequestOutput": ("rapid_llm_amd.engine.outputs", "RequestOutput"),
     "CompletionOutput": ("rapid_llm_amd.engine.outputs", "CompletionOutput"),
     "EngineConfig": ("rapid_llm_amd.config.engine_config", "EngineConfig"),

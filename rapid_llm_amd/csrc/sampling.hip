@@ -2,10 +2,18 @@
 // among equal maxima, as torch.argmax does on one device).
 #include "common.h"
 
-__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+// row_index (optional, in every kernel of this file): the row of `logits` that output row b
+// reads; without it output row b reads row b.
+__device__ inline const float* logits_row(const float* logits, const int* row_index, int b,
+                                          int vocab) {
+    return logits + (size_t)(row_index ? row_index[b] : b) * vocab;
+}
+
+__global__ void argmax_kernel(const float* __restrict__ logits, const int* __restrict__ row_index,
+                              int* __restrict__ out, int vocab) {
     __shared__ float best_v[1024 / RL_WAVE];
     __shared__ int best_i[1024 / RL_WAVE];
-    const float* row = logits + (size_t)blockIdx.x * vocab;
+    const float* row = logits_row(logits, row_index, blockIdx.x, vocab);
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
@@ -48,12 +56,13 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict_
 #define ARGMAX_SLICE 4096
 
 __global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restrict__ logits,
+                                                           const int* __restrict__ row_index,
                                                            float* __restrict__ part_v,
                                                            int* __restrict__ part_i, int vocab,
                                                            int slices) {
     __shared__ float best_v[4];
     __shared__ int best_i[4];
-    const float* row = logits + (size_t)blockIdx.y * vocab;
+    const float* row = logits_row(logits, row_index, blockIdx.y, vocab);
     const int lo = blockIdx.x * ARGMAX_SLICE;
     const int hi = min(vocab, lo + ARGMAX_SLICE);
     float bv = -INFINITY;
@@ -120,20 +129,21 @@ extern "C" int rl_argmax_slices(int vocab) { return (vocab + ARGMAX_SLICE - 1) /
 
 // part_v / part_i: [rows, rl_argmax_slices(vocab)] scratch of the caller; without it (null)
 // the one-stage kernel runs.
-extern "C" int rl_argmax(const float* logits, int* out, float* part_v, int* part_i, int rows,
-                         int vocab, hipStream_t stream) {
+extern "C" int rl_argmax(const float* logits, const int* row_index, int* out, float* part_v,
+                         int* part_i, int rows, int vocab, hipStream_t stream) {
     if (rows <= 0) return RL_OK;
     if (vocab < 1) return RL_ERR_ARG;
     const int slices = (vocab + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
     if (part_v && part_i && slices > 1 && rows <= 65535) {
         hipLaunchKernelGGL(argmax_slices_kernel, dim3(slices, rows), dim3(256), 0, stream, logits,
-                           part_v, part_i, vocab, slices);
+                           row_index, part_v, part_i, vocab, slices);
         if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
         hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(RL_WAVE), 0, stream, part_v,
                            part_i, out, slices);
         return rl_launch_status();
     }
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, stream, logits, out, vocab);
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, stream, logits, row_index,
+                       out, vocab);
     return rl_launch_status();
 }
 
@@ -193,9 +203,9 @@ __device__ inline float wave_inclusive_scan(float v) {
 }
 
 __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
-    const float* __restrict__ logits, const int* __restrict__ row_params,
-    const int* __restrict__ history, int* __restrict__ out, float* __restrict__ out_logprob,
-    int vocab, int bitmap_words) {
+    const float* __restrict__ logits, const int* __restrict__ row_index,
+    const int* __restrict__ row_params, const int* __restrict__ history, int* __restrict__ out,
+    float* __restrict__ out_logprob, int vocab, int bitmap_words) {
     extern __shared__ uint32_t seen[];  // one bit per token id, when the row has a penalty
     __shared__ unsigned long long cand[SMP_POOL];
     __shared__ float cum[SMP_POOL];
@@ -216,7 +226,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const bool penalise = bitmap_words > 0 && penalty != 1.0f && rp[7] > rp[6];
     const bool greedy = !(temperature > 0.f);
     const float inv_t = greedy ? 1.f : 1.f / temperature;
-    const float* row = logits + (size_t)blockIdx.x * vocab;
+    const float* row = logits_row(logits, row_index, blockIdx.x, vocab);
 
     if (penalise) {
         for (int i = tid; i < bitmap_words; i += SMP_THREADS) seen[i] = 0u;
@@ -467,9 +477,9 @@ extern "C" int rl_sample_pool() { return SMP_POOL; }
 
 // history may be null when no row has a penalty.  out_logprob (optional): log-probability
 // of the chosen token under the penalised, temperature-scaled distribution.
-extern "C" int rl_sample(const float* logits, const int* row_params, const int* history, int* out,
-                         float* out_logprob, int rows, int vocab, int any_penalty,
-                         hipStream_t stream) {
+extern "C" int rl_sample(const float* logits, const int* row_index, const int* row_params,
+                         const int* history, int* out, float* out_logprob, int rows, int vocab,
+                         int any_penalty, hipStream_t stream) {
     if (rows <= 0) return RL_OK;
     if (vocab < 1) return RL_ERR_ARG;
     int words = 0;
@@ -479,6 +489,147 @@ extern "C" int rl_sample(const float* logits, const int* row_params, const int* 
         if (!history) return RL_ERR_ARG;
     }
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), (size_t)words * 4, stream,
-                       logits, row_params, history, out, out_logprob, vocab, words);
+                       logits, row_index, row_params, history, out, out_logprob, vocab, words);
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
+// Log-probability records (rapid_llm/engine/sampler.py:343-369): for every row the
+// log-probability of a given token (the one chosen, or the prompt's own next token) and the
+// k most likely tokens with theirs, in descending order, equal values by ascending id.
+//
+// The distribution is the one the row is sampled from: log_softmax of the penalised logits
+// over the temperature, a greedy row counting as temperature 1 (:708-712).  Without
+// row_params it is log_softmax of the raw logits, as prompt positions are scored (:425-447).
+//
+// One workgroup per row; the k tokens are found one after the other, each as the largest
+// (value, lowest id) that comes after the previous one in that order: k + 2 passes over a
+// row that stays in cache, no memory beyond the outputs, and a fixed result.
+// --------------------------------------------------------------------------- //
+__global__ __launch_bounds__(SMP_THREADS) void logprobs_kernel(
+    const float* __restrict__ logits, const int* __restrict__ row_index,
+    const int* __restrict__ row_params, const int* __restrict__ history,
+    const int* __restrict__ targets, float* __restrict__ out_target, int* __restrict__ out_top_ids,
+    float* __restrict__ out_top_lp, int vocab, int k, int bitmap_words) {
+    extern __shared__ uint32_t seen[];
+    __shared__ float wave_tot[SMP_WAVES];
+    __shared__ float best_v[SMP_WAVES];
+    __shared__ int best_i[SMP_WAVES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (RL_WAVE - 1), wave = tid / RL_WAVE;
+    const int* rp = row_params ? row_params + 8 * blockIdx.x : nullptr;
+    const float temperature = rp ? __int_as_float(rp[0]) : 1.f;
+    const float penalty = rp ? __int_as_float(rp[2]) : 1.f;
+    const bool penalise = rp && bitmap_words > 0 && penalty != 1.0f && rp[7] > rp[6];
+    const float inv_t = temperature > 0.f ? 1.f / temperature : 1.f;
+    const float* row = logits_row(logits, row_index, blockIdx.x, vocab);
+
+    if (penalise) {
+        for (int i = tid; i < bitmap_words; i += SMP_THREADS) seen[i] = 0u;
+        __syncthreads();
+        for (int i = rp[6] + tid; i < rp[7]; i += SMP_THREADS) {
+            const int tok = history[i];
+            if (tok >= 0 && tok < vocab) atomicOr(&seen[tok >> 5], 1u << (tok & 31));
+        }
+        __syncthreads();
+    }
+    auto zval = [&](int i) -> float {
+        float x = row[i];
+        if (penalise && ((seen[i >> 5] >> (i & 31)) & 1u)) x = x < 0.f ? x * penalty : x / penalty;
+        return x * inv_t;
+    };
+    // the largest (value, lowest id) after (pv, pi) in descending order; first: no bound
+    auto next_best = [&](bool first, float pv, int pi, float& rv, int& ri) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int i = tid; i < vocab; i += SMP_THREADS) {
+            const float v = zval(i);
+            const bool after = first || v < pv || (v == pv && i > pi);
+            if (after && (v > bv || (v == bv && i < bi))) {
+                bv = v;
+                bi = i;
+            }
+        }
+#pragma unroll
+        for (int off = RL_WAVE / 2; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, RL_WAVE);
+            const int oi = __shfl_xor(bi, off, RL_WAVE);
+            if (ov > bv || (ov == bv && oi < bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        __syncthreads();  // the previous round's readers are done
+        if (lane == 0) {
+            best_v[wave] = bv;
+            best_i[wave] = bi;
+        }
+        __syncthreads();
+        bv = best_v[0];
+        bi = best_i[0];
+        for (int w = 1; w < SMP_WAVES; ++w)
+            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+                bv = best_v[w];
+                bi = best_i[w];
+            }
+        rv = bv;
+        ri = bi;
+    };
+
+    float top_v;
+    int top_i;
+    next_best(true, 0.f, 0, top_v, top_i);
+    const float zmax = top_v;
+
+    // sum of exp in a fixed order: wave w owns a contiguous segment
+    const int seg = ((vocab + SMP_WAVES - 1) / SMP_WAVES + RL_WAVE - 1) / RL_WAVE * RL_WAVE;
+    const int seg_lo = min(vocab, wave * seg), seg_hi = min(vocab, seg_lo + seg);
+    float wsum = 0.f;
+    for (int base = seg_lo; base < seg_hi; base += RL_WAVE) {
+        const int i = base + lane;
+        wsum += (i < seg_hi) ? expf(zval(i) - zmax) : 0.f;
+    }
+    wsum = wave_sum(wsum);
+    if (lane == 0) wave_tot[wave] = wsum;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < SMP_WAVES; ++w) total += wave_tot[w];
+    const float log_z = zmax + logf(total);
+
+    if (tid == 0) {
+        const int t = targets[blockIdx.x];
+        out_target[blockIdx.x] = (t >= 0 && t < vocab) ? zval(t) - log_z : NAN;
+    }
+    for (int j = 0; j < k; ++j) {
+        if (j > 0 && top_i != 0x7fffffff) next_best(false, top_v, top_i, top_v, top_i);
+        if (tid == 0) {
+            // fewer than k values that can be ordered (NaN cannot): the rest is marked empty
+            const bool none = top_i == 0x7fffffff;
+            out_top_ids[(size_t)blockIdx.x * k + j] = none ? -1 : top_i;
+            out_top_lp[(size_t)blockIdx.x * k + j] = none ? -INFINITY : top_v - log_z;
+        }
+    }
+}
+
+// targets [rows]: the token whose log-probability goes to out_target [rows] (NaN for an id
+// outside the vocabulary).  out_top_ids / out_top_lp [rows, k]; k may be 0.  row_params and
+// history as for rl_sample, or null for the raw distribution.
+extern "C" int rl_logprobs(const float* logits, const int* row_index, const int* row_params,
+                           const int* history, const int* targets, float* out_target,
+                           int* out_top_ids, float* out_top_lp, int rows, int vocab, int k,
+                           int any_penalty, hipStream_t stream) {
+    if (rows <= 0) return RL_OK;
+    if (vocab < 1 || k < 0 || k > vocab || !targets || !out_target) return RL_ERR_ARG;
+    if (k > 0 && (!out_top_ids || !out_top_lp)) return RL_ERR_ARG;
+    int words = 0;
+    if (any_penalty) {
+        words = (vocab + 31) / 32;
+        if ((size_t)words * 4 > 40 * 1024) return RL_ERR_ARG;
+        if (!history || !row_params) return RL_ERR_ARG;
+    }
+    hipLaunchKernelGGL(logprobs_kernel, dim3(rows), dim3(SMP_THREADS), (size_t)words * 4, stream,
+                       logits, row_index, row_params, history, targets, out_target, out_top_ids,
+                       out_top_lp, vocab, k, words);
     return rl_launch_status();
 }

@@ -14,11 +14,14 @@ from __future__ import annotations
 from pathlib import Path
 from typing import Any, Iterator, Mapping, Sequence
 
+import torch
+
 from ..config.engine_config import EngineConfig
 from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler, to_records
 from .outputs import CompletionOutput, RequestOutput
 from .request import Request
-from .scheduler import Scheduler
+from .scheduler import SamplingPlan, Scheduler, StepOutput
 
 
 class GpuExecutor:
@@ -29,11 +32,43 @@ class GpuExecutor:
         self.sampler = sampler
         self.cache = runner.cache
 
-    def execute(self, entries, rows, want_logprobs: bool = False):
+    def execute(self, entries, sampling: SamplingPlan) -> StepOutput:
         logits = self.runner.step(entries)
-        ids, logprobs = self.sampler.sample(logits, rows, want_logprobs)
+        in_order = sampling.logits_rows == list(range(logits.shape[0]))
+        ids, _ = self.sampler.sample(
+            logits, sampling.rows, row_index=None if in_order else sampling.logits_rows
+        )
+        chosen = prompt = None
+        asked = [b for b, k in enumerate(sampling.logprob_ks) if k is not None]
+        if asked:
+            pick = torch.tensor(asked, dtype=torch.int64).to(ids.device)
+            chosen = self.sampler.logprobs(
+                logits,
+                ids[pick],
+                max(sampling.logprob_ks[b] for b in asked),
+                rows=[sampling.rows[b] for b in asked],
+                row_index=[sampling.logits_rows[b] for b in asked],
+            )
+        if sampling.prompt_rows:
+            prompt = self.sampler.logprobs(
+                logits, sampling.prompt_targets, max(sampling.prompt_ks), row_index=sampling.prompt_rows
+            )
         # the step's one host synchronisation (rapid_llm/engine/scheduler.py:1000-1005)
-        return ids.tolist(), (logprobs.tolist() if logprobs is not None else None)
+        out = StepOutput(ids.tolist())
+        if chosen is not None:
+            records = to_records(
+                [out.token_ids[b] for b in asked],
+                [sampling.logprob_ks[b] for b in asked],
+                *(t.tolist() for t in chosen),
+            )
+            out.logprobs = [None] * len(out.token_ids)
+            for b, record in zip(asked, records):
+                out.logprobs[b] = record
+        if prompt is not None:
+            out.prompt_logprobs = to_records(
+                sampling.prompt_targets, sampling.prompt_ks, *(t.tolist() for t in prompt)
+            )
+        return out
 
     def finish(self, request_id: str) -> None:
         self.runner.finish(request_id)
@@ -58,7 +93,6 @@ def build_engine(
     hf_overrides: Mapping[str, Any] | None = None,
     gpu_memory_utilization: float = 0.9,
 ) -> Scheduler:
-    from ..sampling.sampler import Sampler
     from .step import ModelRunner
     from .tokenizer import load_stop_token_ids, load_tokenizer
 
@@ -154,6 +188,7 @@ class LLM:
             ],
             prompt_token_ids=list(request.prompt_token_ids),
             request_id=request.request_id,
+            prompt_logprobs=list(request.prompt_logprobs) if request.prompt_logprobs is not None else None,
         )
 
     def generate(

@@ -5,6 +5,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+from ..sampling.logprobs import PositionLogprobs
+
 
 @dataclass
 class CompletionOutput:
@@ -12,7 +14,7 @@ class CompletionOutput:
     text: str
     finish_reason: str | None
     token_ids: list[int] = field(default_factory=list)
-    logprobs: list[float] | None = None  # the chosen tokens' log-probabilities, if asked
+    logprobs: list[PositionLogprobs] | None = None  # parallel to token_ids, if asked
 
 
 @dataclass
@@ -21,6 +23,8 @@ class RequestOutput:
     outputs: list[CompletionOutput]
     prompt_token_ids: list[int] = field(default_factory=list)
     request_id: str = ""
+    # per prompt position, if asked; position 0 has no predictor and is None
+    prompt_logprobs: list[PositionLogprobs | None] | None = None
 
     @property
     def text(self) -> str:

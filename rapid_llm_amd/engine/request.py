@@ -14,6 +14,7 @@ import time
 from dataclasses import dataclass, field
 from enum import Enum
 
+from ..sampling.logprobs import PositionLogprobs
 from ..sampling.params import SamplingParams
 
 
@@ -37,7 +38,8 @@ class Request:
     admission_number: int = -1  # order of the latest admission: larger is younger
     status: RequestStatus = RequestStatus.WAITING
     output_token_ids: list[int] = field(default_factory=list)
-    output_logprobs: list[float] | None = None
+    output_logprobs: list[PositionLogprobs] | None = None  # parallel to output_token_ids, if asked
+    prompt_logprobs: list[PositionLogprobs | None] | None = None  # per prompt position; [0] is None
     text: str = ""
     delta: str = ""
     finish_reason: str | None = None  # "eos" | "length" | "repeat" | "abort"

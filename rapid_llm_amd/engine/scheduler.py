@@ -37,6 +37,7 @@ from dataclasses import dataclass, field
 from typing import Any, Iterable, Sequence
 
 from ..config.engine_config import EngineConfig
+from ..sampling.logprobs import PositionLogprobs
 from ..sampling.params import SamplingParams
 from ..sampling.rng import derive_seed
 from .request import Request, RequestStatus
@@ -65,6 +66,27 @@ class StepPlan:
         return sum(w.count for w in self.work)
 
 
+@dataclass
+class SamplingPlan:
+    """What is to be read off the logits of one step.  The step returns one row of logits
+    per wanted place, in the order of the entries and of their ``want``."""
+
+    rows: list = field(default_factory=list)  # RowSampling, one per token to choose
+    logits_rows: list[int] = field(default_factory=list)  # the row of logits each reads
+    logprob_ks: list[int | None] = field(default_factory=list)  # per chosen token: alternatives to report
+    # prompt positions to score: row of logits, the token that follows there, alternatives
+    prompt_rows: list[int] = field(default_factory=list)
+    prompt_targets: list[int] = field(default_factory=list)
+    prompt_ks: list[int] = field(default_factory=list)
+
+
+@dataclass
+class StepOutput:
+    token_ids: list[int]  # parallel to SamplingPlan.rows
+    logprobs: list[PositionLogprobs | None] | None = None  # parallel to rows, if any asked
+    prompt_logprobs: list[PositionLogprobs] | None = None  # parallel to prompt_rows
+
+
 def detect_repetition(token_ids: Sequence[int], window: int = 32, min_reps: int = 3) -> bool:
     """Whether the output ends in a block of ``window`` tokens that occurred at least
     ``min_reps`` times before.  The reference applies the same test to the last 128
@@ -86,9 +108,9 @@ def detect_repetition(token_ids: Sequence[int], window: int = 32, min_reps: int 
 class Scheduler:
     """``executor`` owns the model side.  It has ``cache`` (the
     :class:`~rapid_llm_amd.cache.manager.CacheManager` whose slots and pages the plan takes),
-    ``execute(entries, rows, want_logprobs) -> (token ids, logprobs or None)`` running one
-    step and choosing a token for every entry that wants one, and ``finish(request_id)``
-    giving back what a request holds."""
+    ``execute(entries, sampling: SamplingPlan) -> StepOutput`` running one step, choosing
+    a token for every row of the plan and scoring what it asks to be scored, and
+    ``finish(request_id)`` giving back what a request holds."""
 
     def __init__(
         self,
@@ -338,16 +360,30 @@ class Scheduler:
         advanced: list[Request] = list(plan.finished)
         if not plan.work:
             return advanced
-        entries, rows, sampled = [], [], []
-        want_logprobs = False
+        entries, sampled = [], []
+        sampling = SamplingPlan()
+        scored: list[tuple[Request, int]] = []  # (request, prompt position the record is for)
+        num_rows = 0
         for w in plan.work:
             r = w.request
-            entries.append(
-                StepEntry(r.request_id, r.tokens(w.start, w.start + w.count), [w.count - 1] if w.samples else [])
-            )
+            p = r.params
+            want: list[int] = []
+            if p.prompt_logprobs is not None:
+                # the logits at position q score the prompt's token q + 1
+                # (rapid_llm/engine/scheduler.py:143-148); what an earlier run of these
+                # positions has scored (before an eviction) is not scored again
+                if r.prompt_logprobs is None:
+                    r.prompt_logprobs = [None] * r.prompt_len
+                for j in range(w.count):
+                    q = w.start + j + 1
+                    if q < r.prompt_len and r.prompt_logprobs[q] is None:
+                        sampling.prompt_rows.append(num_rows + len(want))
+                        sampling.prompt_targets.append(r.prompt_token_ids[q])
+                        sampling.prompt_ks.append(p.prompt_logprobs)
+                        scored.append((r, q))
+                        want.append(j)
             if w.samples:
-                p = r.params
-                rows.append(
+                sampling.rows.append(
                     RowSampling(
                         temperature=p.temperature,
                         top_p=p.top_p,
@@ -357,12 +393,19 @@ class Scheduler:
                         generated=r.output_token_ids if p.repetition_penalty != 1.0 else (),
                     )
                 )
+                sampling.logits_rows.append(num_rows + len(want))
+                sampling.logprob_ks.append(p.logprobs)
                 sampled.append(r)
-                want_logprobs |= r.output_logprobs is not None
-        tokens, logprobs = self.executor.execute(entries, rows, want_logprobs)
+                want.append(w.count - 1)
+            entries.append(StepEntry(r.request_id, r.tokens(w.start, w.start + w.count), want))
+            num_rows += len(want)
+        result = self.executor.execute(entries, sampling)
+        tokens, logprobs = result.token_ids, result.logprobs
         for w in plan.work:
             w.request.num_computed_tokens = w.start + w.count
             self.cache.trim(w.request.request_id, w.request.num_computed_tokens)
+        for (request, q), record in zip(scored, result.prompt_logprobs or ()):
+            request.prompt_logprobs[q] = record
 
         now = time.monotonic()
         check_repeat = self._step_count % REPEAT_POLL_INTERVAL == 0
@@ -378,7 +421,7 @@ class Scheduler:
                 continue
             request.output_token_ids.append(token)
             if request.output_logprobs is not None and logprobs is not None:
-                request.output_logprobs.append(float(logprobs[i]))
+                request.output_logprobs.append(logprobs[i])
             detok = self._detok.get(request.request_id)
             if detok is not None:
                 piece = detok.append(token)

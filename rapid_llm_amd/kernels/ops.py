@@ -275,17 +275,45 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     )
 
 
-def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
-    rows, vocab = logits.shape
+def _row_index(row_index: Optional[torch.Tensor]) -> None:
+    if row_index is not None:
+        _need(row_index, "row_index", torch.int32)
+        if row_index.dim() != 1:
+            raise KernelError(f"row_index must have one dimension, got {tuple(row_index.shape)}")
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, row_index: Optional[torch.Tensor] = None) -> None:
+    """``out[b]`` = arg-max of row ``row_index[b]`` of ``logits`` (row ``b`` without an index)."""
+    vocab = logits.shape[1]
+    rows = out.shape[0]
     _need(logits, "logits", torch.float32)
     _need(out, "out", torch.int32, (rows,))
+    _row_index(row_index)
+    if row_index is not None and row_index.shape[0] != rows:
+        raise KernelError(f"{row_index.shape[0]} row indices for {rows} outputs")
+    if row_index is None and logits.shape[0] != rows:
+        raise KernelError(f"{logits.shape[0]} rows of logits for {rows} outputs")
     lib = core()
     slices = lib.rl_argmax_slices(vocab)
     part_v = part_i = None
     if slices > 1 and rows * 4 < slices * 16:  # few wide rows: two stages fill the chip
         part_v = torch.empty((rows, slices), dtype=torch.float32, device=logits.device)
         part_i = torch.empty((rows, slices), dtype=torch.int32, device=logits.device)
-    _ok(lib.rl_argmax(_p(logits), _p(out), _p(part_v), _p(part_i), rows, vocab, _stream()), "rl_argmax")
+    _ok(
+        lib.rl_argmax(_p(logits), _p(row_index), _p(out), _p(part_v), _p(part_i), rows, vocab, _stream()),
+        "rl_argmax",
+    )
+
+
+_PENALTY_MAX_VOCAB = 40 * 1024 * 8  # one bit per token id in 40 KB of LDS
+
+
+def _penalty_fits(vocab: int) -> None:
+    if vocab > _PENALTY_MAX_VOCAB:
+        raise KernelError(
+            f"the repetition penalty keeps one bit per token id in 40 KB of LDS: vocabulary "
+            f"{vocab} is beyond {_PENALTY_MAX_VOCAB}"
+        )
 
 
 def sample(
@@ -295,29 +323,77 @@ def sample(
     out: torch.Tensor,
     out_logprob: Optional[torch.Tensor],
     any_penalty: bool,
+    row_index: Optional[torch.Tensor] = None,
 ) -> None:
     """General token selection (penalty, temperature, nucleus, seeded draw), one row per
-    workgroup.  ``row_params [rows * 8]`` int32 as the kernel documents them."""
-    rows, vocab = logits.shape
+    workgroup.  ``row_params [rows * 8]`` int32 as the kernel documents them; output row
+    ``b`` reads row ``row_index[b]`` of ``logits`` (row ``b`` without an index)."""
+    vocab = logits.shape[1]
+    rows = out.shape[0]
     _need(logits, "logits", torch.float32)
     _need(row_params, "row_params", torch.int32, (rows * 8,))
     _need(out, "out", torch.int32, (rows,))
+    _row_index(row_index)
+    if (row_index.shape[0] if row_index is not None else logits.shape[0]) != rows:
+        raise KernelError(f"{rows} outputs do not match the rows to read")
     if out_logprob is not None:
         _need(out_logprob, "out_logprob", torch.float32, (rows,))
     if history is not None:
         _need(history, "history", torch.int32)
-    if any_penalty and vocab > 40 * 1024 * 8:
-        raise KernelError(
-            f"the repetition penalty keeps one bit per token id in 40 KB of LDS: vocabulary "
-            f"{vocab} is beyond {40 * 1024 * 8}"
-        )
+    if any_penalty:
+        _penalty_fits(vocab)
     _ok(
         core().rl_sample(
-            _p(logits), _p(row_params), _p(history), _p(out), _p(out_logprob), rows, vocab,
-            int(bool(any_penalty)), _stream(),
+            _p(logits), _p(row_index), _p(row_params), _p(history), _p(out), _p(out_logprob), rows,
+            vocab, int(bool(any_penalty)), _stream(),
         ),
         "rl_sample",
     )
+
+
+def logprobs(
+    logits: torch.Tensor,
+    targets: torch.Tensor,
+    k: int,
+    row_params: Optional[torch.Tensor] = None,
+    history: Optional[torch.Tensor] = None,
+    any_penalty: bool = False,
+    row_index: Optional[torch.Tensor] = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Log-probability of ``targets[b]`` and the ``k`` most likely tokens of every row:
+    ``(target [rows] float32, top ids [rows, k] int32, top log-probabilities [rows, k]
+    float32)``, descending, equal values by ascending id.  With ``row_params`` the
+    distribution is the one ``sample`` draws from (penalty, temperature; greedy rows count
+    as temperature 1); without, log_softmax of the raw logits."""
+    vocab = logits.shape[1]
+    rows = targets.shape[0]
+    _need(logits, "logits", torch.float32)
+    _need(targets, "targets", torch.int32, (rows,))
+    _row_index(row_index)
+    if (row_index.shape[0] if row_index is not None else logits.shape[0]) != rows:
+        raise KernelError(f"{rows} targets do not match the rows to read")
+    if not 0 <= k <= vocab:
+        raise KernelError(f"top-k width {k} is outside [0, vocabulary {vocab}]")
+    if row_params is not None:
+        _need(row_params, "row_params", torch.int32, (rows * 8,))
+    if history is not None:
+        _need(history, "history", torch.int32)
+    if any_penalty:
+        _penalty_fits(vocab)
+        if row_params is None or history is None:
+            raise KernelError("a penalty needs row_params and history")
+    target_lp = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    top_ids = torch.empty((rows, k), dtype=torch.int32, device=logits.device)
+    top_lp = torch.empty((rows, k), dtype=torch.float32, device=logits.device)
+    _ok(
+        core().rl_logprobs(
+            _p(logits), _p(row_index), _p(row_params), _p(history), _p(targets), _p(target_lp),
+            _p(top_ids if k else None), _p(top_lp if k else None), rows, vocab, k,
+            int(bool(any_penalty)), _stream(),
+        ),
+        "rl_logprobs",
+    )
+    return target_lp, top_ids, top_lp
 
 
 def sample_uniform(seed: int, counter: int) -> float:

@@ -1,7 +1,8 @@
+from .logprobs import PositionLogprobs
 from .params import SamplingParams
 from .rng import uniform_draw
 
-__all__ = ["SamplingParams", "Sampler", "RowSampling", "uniform_draw"]
+__all__ = ["SamplingParams", "PositionLogprobs", "Sampler", "RowSampling", "uniform_draw"]
 
 
 def __getattr__(name):

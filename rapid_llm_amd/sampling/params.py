@@ -20,8 +20,8 @@ class SamplingParams:
     max_gen_len: int | None = None  # None: fill the remaining context window
     repetition_penalty: float = 1.0  # over generated tokens; 1.0 disables it
     stop_on_repeat: bool = False  # engine-side breaker of repeating output
-    logprobs: int | None = None  # report the chosen token's log-probability (0) ...
-    prompt_logprobs: int | None = None
+    logprobs: int | None = None  # per generated token: its log-probability and the k most likely
+    prompt_logprobs: int | None = None  # the same for the prompt's own tokens (position 0 has none)
     seed: int | None = None  # None: derived from the engine's seed and the request's number
     ignore_eos: bool = False  # keep generating through stop tokens (benchmarks)
 
@@ -38,13 +38,6 @@ class SamplingParams:
             value = getattr(self, name)
             if value is not None and value < 0:
                 raise ValueError(f"{name} must be >= 0, got {value}")
-        if self.logprobs is not None and self.logprobs > 0:
-            raise ValueError(
-                "logprobs > 0 (alternatives beside the chosen token) is not implemented; "
-                "logprobs=0 reports the chosen token's log-probability"
-            )
-        if self.prompt_logprobs is not None:
-            raise ValueError("prompt_logprobs is not implemented in this engine")
         if self.seed is not None and not 0 <= self.seed < 1 << 64:
             raise ValueError(f"seed must fit 64 unsigned bits, got {self.seed}")
 

@@ -75,3 +75,19 @@ def plain_logprob(logits: torch.Tensor, token: int, temperature: float, penalty:
         logits = plain_repetition_penalty(logits, list(generated), penalty)
     t = temperature if temperature > 0 else 1.0  # rapid_llm/engine/sampler.py:508
     return float(torch.log_softmax(logits.double() / t, dim=-1)[token])
+
+
+def plain_top_logprobs(logits: torch.Tensor, k: int, temperature: float = 1.0, penalty: float = 1.0,
+                       generated: list[int] = ()) -> tuple[list[int], list[float]]:
+    """The ``k`` most likely tokens and their log-probabilities, descending, equal values by
+    ascending id: ``log_softmax`` of the final logits, then ``topk``
+    (rapid_llm/engine/sampler.py:362-369).  The raw logits with the defaults, as a prompt is
+    scored (:425-447)."""
+    logits = logits.to(torch.float32)
+    if penalty != 1.0 and len(generated):
+        logits = plain_repetition_penalty(logits, list(generated), penalty)
+    t = temperature if temperature > 0 else 1.0
+    z = logits / t
+    lp = torch.log_softmax(z.double(), dim=-1)
+    order = torch.sort(z, descending=True, stable=True).indices[:k]
+    return order.tolist(), lp[order].tolist()

@@ -69,7 +69,8 @@ def test_sampled_generation_tiny_b_chunked_and_mixed(tmp_path):
     for i, (prompt, out) in enumerate(zip(prompts, outs)):
         want = _plain_generate(pcfg, pw, prompt, 20, 0.8, 0.9, 77 + i)
         assert out.token_ids == want, i
-        assert len(out.outputs[0].logprobs) == 20 and all(lp <= 0 for lp in out.outputs[0].logprobs)
+        records = out.outputs[0].logprobs
+        assert [r.token_id for r in records] == want and all(r.logprob <= 0 and not r.top_token_ids for r in records)
     # the same requests, unchunked and one at a time, draw the same tokens
     solo = _llm(model_dir, "float32", page, max_seq_len=256, max_chunk_size=0, max_num_batched_tokens=256,
                 max_num_seqs=1)
@@ -94,6 +95,61 @@ def test_eviction_changes_nothing(tmp_path):
     assert [o.token_ids for o in outs] == [o.token_ids for o in ample]
     tight.scheduler.cache.check_invariants()
     assert tight.scheduler.cache.num_free_pages() == 23
+
+
+def test_logprob_records_of_prompt_and_output(tmp_path):
+    """Prompt positions are scored on the raw logits, generated tokens on the distribution
+    they were drawn from; portions of 5 tokens beside decoded tokens, and a pool so small
+    that requests are evicted and run again, change no record."""
+    from plain_sampler import plain_logprob, plain_top_logprobs
+    from rapid_llm_amd import SamplingParams
+
+    cfg, page, seed = TINY["A"]
+    model_dir = make_model_dir(tmp_path, "A", "float32")
+    pcfg, pw = plain_load(model_dir)
+    prompts = [random_tokens(n, cfg["vocab_size"], seed + 3 * n) for n in (1, 12, 7)]
+    params = [
+        SamplingParams(temperature=0.0, max_gen_len=9, logprobs=3, prompt_logprobs=2),
+        SamplingParams(temperature=0.9, top_p=0.9, max_gen_len=9, seed=5, logprobs=2, prompt_logprobs=4,
+                       repetition_penalty=1.2),
+        SamplingParams(temperature=0.7, top_p=1.0, max_gen_len=9, seed=6, logprobs=0),
+    ]
+    llm = _llm(model_dir, "float32", page, max_seq_len=128, max_chunk_size=5, max_num_batched_tokens=12)
+    outs = llm.generate(prompts, params)
+    tight = _llm(model_dir, "float32", page, max_seq_len=128, max_chunk_size=5, max_num_batched_tokens=12,
+                 num_pages=9)
+    evicted = tight.generate(prompts, params)
+    assert tight.scheduler.num_preemptions > 0
+
+    def near(a, b):
+        return abs(a - b) < 1e-4 * max(1.0, abs(b))
+
+    for prompt, p, out, again in zip(prompts, params, outs, evicted):
+        tokens = out.token_ids
+        assert again.token_ids == tokens
+        logits = plain_forward(pcfg, pw, prompt + tokens)
+        if p.prompt_logprobs is None:
+            assert out.prompt_logprobs is None
+        else:
+            assert len(out.prompt_logprobs) == len(prompt) and out.prompt_logprobs[0] is None
+            for q in range(1, len(prompt)):
+                rec = out.prompt_logprobs[q]
+                assert rec.token_id == prompt[q]
+                assert near(rec.logprob, plain_logprob(logits[q - 1], prompt[q], 1.0))
+                ids, lps = plain_top_logprobs(logits[q - 1], p.prompt_logprobs)
+                assert list(rec.top_token_ids) == ids and all(near(a, b) for a, b in zip(rec.top_logprobs, lps))
+        records = out.outputs[0].logprobs
+        assert [r.token_id for r in records] == tokens
+        for i, rec in enumerate(records):
+            row = logits[len(prompt) - 1 + i]
+            args = (p.temperature, p.repetition_penalty, tokens[:i])
+            assert near(rec.logprob, plain_logprob(row, tokens[i], *args))
+            ids, lps = plain_top_logprobs(row, p.logprobs, *args)
+            assert list(rec.top_token_ids) == ids and all(near(a, b) for a, b in zip(rec.top_logprobs, lps))
+        for mine, theirs in zip(records, again.outputs[0].logprobs):
+            assert mine.token_id == theirs.token_id and near(mine.logprob, theirs.logprob)
+        if p.prompt_logprobs is not None:
+            assert [r and r.token_id for r in again.prompt_logprobs] == [r and r.token_id for r in out.prompt_logprobs]
 
 
 @pytest.mark.parametrize("which", ["A", "B", "C", "D"])

@@ -133,3 +133,73 @@ def test_penalty_needs_a_vocabulary_the_bitmap_holds():
     sampler.sample(logits, [Row(temperature=1.0, top_p=0.9)])  # no penalty: fine
     with pytest.raises(KernelError, match="beyond"):
         sampler.sample(logits, [Row(temperature=1.0, repetition_penalty=1.1, generated=[1])])
+
+
+@pytest.mark.parametrize("vocab", [3, 64, 503, 4099, 151936])
+def test_logprob_records_match_the_plain_ones(vocab):
+    """The given token's log-probability and the k most likely, under the distribution the
+    row is sampled from (penalty, temperature, greedy as temperature 1) and under the raw
+    logits; rows read through an index, in another order than they lie."""
+    from plain_sampler import plain_top_logprobs
+
+    sampler, Row = _sampler()
+    gen = torch.Generator().manual_seed(7 * vocab)
+    kinds = [dict(temperature=0.0), dict(temperature=0.7), dict(temperature=1.6, repetition_penalty=1.4),
+             dict(temperature=0.0, repetition_penalty=0.7)]
+    n = 9
+    logit_rows = [torch.randn(vocab, generator=gen) * (1.0, 5.0, 0.3)[i % 3] for i in range(n)]
+    # equal values: the lower id comes first, among the best and further down
+    logit_rows[2][: min(vocab, 6)] = float(logit_rows[2].max()) + 1.0
+    logit_rows[4][vocab // 2 :] = -3.0
+    order = [5, 0, 8, 2, 4, 7, 1]
+    rows, targets = [], []
+    for b, r in enumerate(order):
+        generated = torch.randint(0, vocab, (11,), generator=gen).tolist() + [int(logit_rows[r].argmax())]
+        rows.append(Row(seed=b, counter=b, generated=generated, **kinds[b % len(kinds)]))
+        targets.append(int(torch.randint(0, vocab, (1,), generator=gen)))
+    logits = torch.stack(logit_rows).cuda()
+    k = min(vocab, 7)
+    for with_rows in (True, False):
+        target_lp, top_ids, top_lp = sampler.logprobs(
+            logits, targets, k, rows=rows if with_rows else None, row_index=order)
+        target_lp, top_ids, top_lp = target_lp.tolist(), top_ids.tolist(), top_lp.tolist()
+        for b, r in enumerate(order):
+            row = rows[b] if with_rows else Row(temperature=1.0)
+            args = (row.temperature, row.repetition_penalty, list(row.generated))
+            want = plain_logprob(logit_rows[r], targets[b], *args)
+            assert abs(target_lp[b] - want) < 2e-4 * max(1.0, abs(want)), (vocab, b)
+            ids, lps = plain_top_logprobs(logit_rows[r], k, *args)
+            assert top_ids[b] == ids, (vocab, with_rows, b)
+            assert max(abs(x - y) for x, y in zip(top_lp[b], lps)) < 2e-4 * max(1.0, abs(lps[-1])), (vocab, b)
+    # k = 0: the token's own log-probability only; without an index the rows in order
+    lp0, ids0, _ = sampler.logprobs(logits, [1] * n, 0)
+    assert ids0.shape == (n, 0)
+    for r in range(n):
+        want = plain_logprob(logit_rows[r], 1, 1.0)
+        assert abs(float(lp0[r]) - want) < 2e-4 * max(1.0, abs(want))
+
+
+def test_logprob_records_with_values_that_cannot_be_ordered():
+    """NaN is never listed: with fewer than k comparable values the rest is marked empty;
+    -inf is comparable and comes last, by ascending id."""
+    sampler, _ = _sampler()
+    logits = torch.tensor([[0.5, float("nan"), -float("inf"), 2.0, -float("inf")]]).cuda()
+    _, ids, _ = sampler.logprobs(logits, [3], 5)
+    assert ids.tolist() == [[3, 0, 2, 4, -1]]
+    logits = torch.tensor([[0.5, -float("inf"), 2.0, -float("inf")]]).cuda()
+    lp, ids, lps = sampler.logprobs(logits, [1], 4)
+    assert ids.tolist() == [[2, 0, 1, 3]] and lp.item() == -float("inf")
+    assert lps[0, 2:].tolist() == [-float("inf")] * 2 and abs(lps[0, :2].exp().sum().item() - 1.0) < 1e-6
+
+
+def test_sampling_through_a_row_index():
+    sampler, Row = _sampler()
+    gen = torch.Generator().manual_seed(5)
+    logits = torch.randn(12, 9001, generator=gen).cuda()
+    index = [11, 3, 3, 0, 7]
+    ids, _ = sampler.sample(logits, [Row() for _ in index], row_index=index)
+    assert ids.tolist() == logits.argmax(-1)[index].tolist()
+    rows = [Row(temperature=0.9, top_p=0.8, seed=3, counter=i) for i in range(len(index))]
+    picked, _ = sampler.sample(logits, rows, row_index=index)
+    direct, _ = sampler.sample(logits[index].contiguous(), rows)
+    assert picked.tolist() == direct.tolist()

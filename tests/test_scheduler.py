@@ -8,8 +8,8 @@ import pytest
 from rapid_llm_amd.cache import CacheManager, GroupSpec
 from rapid_llm_amd.config import EngineConfig
 from rapid_llm_amd.engine.request import RequestStatus
-from rapid_llm_amd.engine.scheduler import Scheduler, detect_repetition
-from rapid_llm_amd.sampling import SamplingParams
+from rapid_llm_amd.engine.scheduler import Scheduler, StepOutput, detect_repetition
+from rapid_llm_amd.sampling import PositionLogprobs, SamplingParams
 
 EOS = 99
 
@@ -22,12 +22,15 @@ class ScriptedExecutor:
         self.cache = CacheManager([GroupSpec(0, window, (0,))], num_pages, page, seqs, max_len)
         self.token = token or (lambda rid, i: 1000 + i)
         self.steps = []
+        self.wants = []  # (request, first position, tokens, wanted places) of every entry run
         self.computed = {}
         self.fed = {}
 
-    def execute(self, entries, rows, want_logprobs=False):
+    def execute(self, entries, sampling):
+        rows = sampling.rows
         shape, out = [], []
         k = 0
+        num_rows = 0
         for e in entries:
             assert self.cache.has(e.request_id), "an entry without a slot"
             start = self.computed.get(e.request_id, 0)
@@ -35,14 +38,28 @@ class ScriptedExecutor:
             self.computed[e.request_id] = start + len(e.tokens)
             self.fed.setdefault(e.request_id, []).extend(e.tokens)
             shape.append((e.request_id, len(e.tokens), bool(e.want)))
-            if e.want:
-                assert list(e.want) == [len(e.tokens) - 1]
+            self.wants.append((e.request_id, start, len(e.tokens), list(e.want)))
+            if e.want and k < len(rows) and sampling.logits_rows[k] == num_rows + len(e.want) - 1:
+                assert e.want[-1] == len(e.tokens) - 1
                 out.append(self.token(e.request_id, rows[k].counter))
                 k += 1
+            num_rows += len(e.want)
         assert k == len(rows)
         self.steps.append(shape)
         self.cache.check_invariants()
-        return out, ([-1.0] * len(out) if want_logprobs else None)
+        result = StepOutput(out)
+        if any(kk is not None for kk in sampling.logprob_ks):
+            result.logprobs = [
+                None if kk is None else PositionLogprobs(t, -1.0, tuple(range(kk)), (-2.0,) * kk)
+                for t, kk in zip(out, sampling.logprob_ks)
+            ]
+        if sampling.prompt_rows:
+            assert max(sampling.prompt_rows) < num_rows
+            result.prompt_logprobs = [
+                PositionLogprobs(t, -float(row), tuple(range(kk)), (-2.0,) * kk)
+                for row, t, kk in zip(sampling.prompt_rows, sampling.prompt_targets, sampling.prompt_ks)
+            ]
+        return result
 
     def finish(self, request_id):
         self.cache.release(request_id)
@@ -272,8 +289,61 @@ def test_logprobs_are_collected_when_asked():
     s, _ = _make()
     r = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=3, logprobs=0))
     q = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=3))
+    w = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=3, logprobs=2))
     s.run_to_completion()
-    assert r.output_logprobs == [-1.0, -1.0, -1.0] and q.output_logprobs is None
+    assert [x.logprob for x in r.output_logprobs] == [-1.0] * 3 and q.output_logprobs is None
+    assert [x.token_id for x in r.output_logprobs] == r.output_token_ids
+    assert all(x.top_token_ids == () for x in r.output_logprobs)
+    assert [x.token_id for x in w.output_logprobs] == w.output_token_ids
+    assert all(x.top_token_ids == (0, 1) and x.top_logprobs == (-2.0, -2.0) for x in w.output_logprobs)
+
+
+def test_a_stop_token_leaves_no_record():
+    s, _ = _make(token=lambda rid, i: EOS if i == 2 else 7)
+    r = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=8, logprobs=1))
+    s.run_to_completion()
+    assert r.finish_reason == "eos" and r.output_token_ids == [7, 7] and len(r.output_logprobs) == 2
+
+
+def test_prompt_logprobs_cover_every_position_once_across_portions():
+    """Position q is scored by the logits at q - 1, whichever portion holds them: the last
+    place of a portion scores the first token of the next one; position 0 has no predictor
+    (rapid_llm/engine/scheduler.py:143-148, rapid_llm/engine/llm_engine.py:274-291)."""
+    s, ex = _make(max_chunk_size=4, max_num_batched_tokens=6)
+    prompt = list(range(20, 31))  # 11 tokens: portions of 4, 4, 3
+    r = s.add_request(prompt, SamplingParams(temperature=0.0, max_gen_len=3, prompt_logprobs=2, logprobs=0))
+    other = s.add_request([5, 6, 7, 8, 9], SamplingParams(temperature=0.0, max_gen_len=3))
+    s.run_to_completion()
+    assert other.prompt_logprobs is None
+    assert len(r.prompt_logprobs) == 11 and r.prompt_logprobs[0] is None
+    assert [x.token_id for x in r.prompt_logprobs[1:]] == prompt[1:]
+    assert all(x.top_token_ids == (0, 1) for x in r.prompt_logprobs[1:])
+    mine = [(start, want) for rid, start, _, want in ex.wants if rid == r.request_id]
+    # every place of a portion but the prompt's last is scored; the last one chooses a token
+    assert mine[:3] == [(0, [0, 1, 2, 3]), (4, [0, 1, 2, 3]), (8, [0, 1, 2])]
+    assert all(want == [0] for _, want in mine[3:])
+    assert len(r.output_logprobs) == 3
+
+
+def test_prompt_logprobs_of_one_token_prompt_and_after_eviction():
+    s, _ = _make()
+    r = s.add_request([4], SamplingParams(temperature=0.0, max_gen_len=2, prompt_logprobs=0))
+    s.run_to_completion()
+    assert r.prompt_logprobs == [None]
+    # a pool of 6 pages of 4: two requests outgrow it, one is evicted and runs again; what
+    # was scored before the eviction is kept and not asked for again
+    s, ex = _make(num_pages=7, page=4, seqs=2, max_len=64)
+    params = SamplingParams(temperature=0.0, max_gen_len=12, prompt_logprobs=1)
+    a = s.add_request(list(range(10, 16)), params)
+    b = s.add_request(list(range(30, 36)), params)
+    s.run_to_completion()
+    assert s.num_preemptions > 0
+    for r in (a, b):
+        assert [x.token_id for x in r.prompt_logprobs[1:]] == r.prompt_token_ids[1:]
+    evicted = a if a.num_preemptions else b
+    again = [(n, want) for rid, start, n, want in ex.wants if rid == evicted.request_id and start == 0]
+    assert again[0] == (6, [0, 1, 2, 3, 4, 5]) and len(again) >= 2
+    assert all(want == [n - 1] for n, want in again[1:])
 
 
 def test_repetition_breaker():
@@ -292,7 +362,7 @@ def test_repetition_breaker():
 def test_sampling_params_validation():
     SamplingParams()
     for bad in (dict(temperature=-1), dict(top_p=0), dict(top_p=1.5), dict(max_gen_len=0),
-                dict(repetition_penalty=0), dict(logprobs=-1), dict(logprobs=5), dict(prompt_logprobs=1),
+                dict(repetition_penalty=0), dict(logprobs=-1), dict(prompt_logprobs=-1),
                 dict(seed=-3)):
         with pytest.raises(ValueError):
             SamplingParams(**bad)
