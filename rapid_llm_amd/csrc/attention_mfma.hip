@@ -358,7 +358,8 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
         }
         __syncthreads();
 
-        // the loads of the next step are issued before this step's arithmetic
+        // the loads of the next step are issued before this step's arithmetic (two steps ahead
+        // was measured: never faster, and slower wherever a compute unit holds several waves)
         DecodeFrags cur, nxt;
         int base = lo + 32 * wave;
         if (base < hi)
@@ -477,29 +478,41 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
     }
 }
 
-// merge of the splits: out = sum_s w_s o_s / sum_s w_s with w_s = l_s * 2^(m_s - max m)
+// merge of the splits: out = sum_s w_s o_s / sum_s w_s with w_s = l_s * 2^(m_s - max m).
+// One thread per channel; the loads of MERGE_STEP splits are issued together and folded into a
+// running (max, weight, output), in the order of the splits.
+#define MERGE_STEP 8
 __global__ void attn_merge_kernel(const float* __restrict__ part_o,
                                   const float* __restrict__ part_ml, bf16_t* __restrict__ out,
                                   const int* __restrict__ seq_token, int nq, int nsplit) {
     const int seq = blockIdx.x, head = blockIdx.y;
     const size_t slot0 = ((size_t)seq * nq + head) * nsplit;
-    float mm = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(slot0 + s) * 2]);
-    float wsum = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-        const float ms = part_ml[(slot0 + s) * 2];
-        if (ms != -INFINITY) wsum += part_ml[(slot0 + s) * 2 + 1] * exp2f(ms - mm);
-    }
     const int t = seq_token[seq];
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float o = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const float ms = part_ml[(slot0 + s) * 2];
-            if (ms == -INFINITY) continue;  // an empty split wrote no output
-            o += part_o[(slot0 + s) * D + d] * (part_ml[(slot0 + s) * 2 + 1] * exp2f(ms - mm));
+    const int d = threadIdx.x;
+    if (d >= D) return;
+    float mm = -INFINITY, wsum = 0.f, o = 0.f;
+    for (int s0 = 0; s0 < nsplit; s0 += MERGE_STEP) {
+        float ms[MERGE_STEP], ls[MERGE_STEP], os[MERGE_STEP];
+#pragma unroll
+        for (int j = 0; j < MERGE_STEP; ++j) {
+            const bool in = s0 + j < nsplit;
+            const size_t slot = slot0 + (in ? s0 + j : 0);
+            ms[j] = in ? part_ml[slot * 2] : -INFINITY;
+            ls[j] = part_ml[slot * 2 + 1];
+            os[j] = part_o[slot * D + d];
         }
-        out[((size_t)t * nq + head) * D + d] = float_to_bf16(o / wsum);
+#pragma unroll
+        for (int j = 0; j < MERGE_STEP; ++j) {
+            if (ms[j] == -INFINITY) continue;  // an empty split wrote no output
+            const float mn = fmaxf(mm, ms[j]);
+            const float keep = exp2f(mm - mn);  // 0 while nothing has been folded in
+            const float w = ls[j] * exp2f(ms[j] - mn);
+            o = o * keep + os[j] * w;
+            wsum = wsum * keep + w;
+            mm = mn;
+        }
     }
+    out[((size_t)t * nq + head) * D + d] = float_to_bf16(o / wsum);
 }
 
 extern "C" int rl_attn_head_dim() { return D; }

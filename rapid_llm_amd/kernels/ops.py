@@ -518,11 +518,12 @@ class AttentionPlan:
 
 
 # Workgroups a decode launch should reach before it stops splitting the keys, and the fewest
-# keys a split is worth (measured at 2,048 keys, 8 kv heads: 1 request 256 keys a split,
-# 8 requests 512, 64 requests no split; finer splits only add merge work).
+# keys a split is worth (measured at 2,048 keys, 8 kv heads: 1 request 128 keys a split,
+# 8 requests 512, 64 requests no split; at 512 keys 128 a split for 1 and 8 requests; finer
+# splits only add merge work).
 _TARGET_BLOCKS = 256
 _FIRST_ROUND = 256  # workgroups that start first, one on each compute unit
-_MIN_SPLIT_KEYS = 256
+_MIN_SPLIT_KEYS = 128
 _MAX_SPLIT_PAGES = 1024  # page ids of one split are staged in LDS
 
 
