@@ -84,8 +84,16 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const T* __
     float4* res = reinterpret_cast<float4*>(residual + (size_t)row * hidden);
     const Vec4<T>* dl = delta ? reinterpret_cast<const Vec4<T>*>(delta + (size_t)row * hidden) : nullptr;
     const int nvec = hidden >> 2;
-    float4 val[CHUNKS];
+    const float4* w4 = reinterpret_cast<const float4*>(weight);
+    float4 val[CHUNKS], wt[CHUNKS];
     float ss = 0.f;
+    // the weights are read before the sum, not after its barrier: one wait less in a kernel
+    // that is all latency when it has a handful of rows
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) wt[c] = w4[i];
+    }
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int i = threadIdx.x + c * blockDim.x;
@@ -106,12 +114,11 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const T* __
     ss = block_sum(ss, scratch);
     const float rrms = rsqrtf(ss / (float)hidden + eps);
     Vec4<T>* o = reinterpret_cast<Vec4<T>*>(out + (size_t)r * hidden);
-    const float4* w4 = reinterpret_cast<const float4*>(weight);
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int i = threadIdx.x + c * blockDim.x;
         if (i < nvec) {
-            const float4 w = w4[i];
+            const float4 w = wt[c];
             Vec4<T> y;
             y.v[0] = from_float<T>(val[c].x * rrms * w.x);
             y.v[1] = from_float<T>(val[c].y * rrms * w.y);
