@@ -95,6 +95,7 @@ def main() -> int:
     ap.add_argument("--point-steps", type=int, default=32)
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-pipeline", action="store_true", help="read every step's tokens before queueing the next")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
@@ -103,7 +104,10 @@ def main() -> int:
     import torch
 
     from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
-    from rapid_llm_amd.kernels import ops
+    from rapid_llm_amd.engine.feed import fed_token
+    from rapid_llm_amd.engine.llm import GpuExecutor
+    from rapid_llm_amd.engine.scheduler import SamplingPlan
+    from rapid_llm_amd.sampling.sampler import RowSampling, Sampler
 
     shape = load_shape()
     context, prompt_len = shape.pop("context"), shape.pop("prompt_len")
@@ -158,28 +162,46 @@ def main() -> int:
         print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
 
     # ---- decode ----------------------------------------------------------------
+    executor = GpuExecutor(runner, Sampler(runner.device))
+
+    def greedy(rows: int) -> SamplingPlan:
+        return SamplingPlan(
+            rows=[RowSampling() for _ in range(rows)], logits_rows=list(range(rows)), logprob_ks=[None] * rows
+        )
+
     def decode(batch: int, steps: int, warmup: int) -> tuple[float, float]:
-        """Mean seconds per decode step and the mean context length over the timed steps."""
+        """Mean seconds per decode step and the mean context length over the timed steps.
+        A step is what the engine's loop does for one token of every request: queue the
+        forward pass and the choice of the tokens, read the chosen tokens back.  Pipelined
+        (the engine's default), the next step is queued, fed from the device, before the
+        last one's tokens are read."""
         ids = [f"d{i}" for i in range(batch)]
-        last = torch.empty(batch, dtype=torch.int32, device=runner.device)
-        for k, rid in enumerate(ids):  # prompts, one request a step
-            logits = runner.step([StepEntry(rid, prompt(), [prompt_len - 1])])
-            ops.argmax(logits, last[k : k + 1])
-        tokens = last.tolist()
+        tokens = []
+        for rid in ids:  # prompts, one request a step
+            tokens += executor.execute([StepEntry(rid, prompt(), [prompt_len - 1])], greedy(1)).token_ids
+        plan = greedy(batch)
+        fed = [StepEntry(rid, [fed_token(i)], [0]) for i, rid in enumerate(ids)]
+        inflight = executor.launch([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)], plan)
 
         def one_step():
-            nonlocal tokens
-            logits = runner.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
-            ops.argmax(logits, last)
-            tokens = last.tolist()  # the step's one host synchronisation
+            nonlocal inflight
+            if args.no_pipeline:
+                tokens = inflight.result().token_ids  # the step's one host synchronisation
+                inflight = executor.launch([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)], plan)
+            else:
+                queued = executor.launch(fed, plan)
+                inflight.result()
+                inflight = queued
 
         for _ in range(warmup):
             one_step()
+        inflight.result()
         torch.cuda.synchronize()
-        ctx_start = runner.tokens_cached(ids[0])
+        ctx_start = runner.tokens_cached(ids[0]) - 1  # one step is in flight
         t = time.perf_counter()
         for _ in range(steps):
             one_step()
+        inflight.result()
         torch.cuda.synchronize()
         sec = (time.perf_counter() - t) / steps
         mean_ctx = ctx_start + (steps - 1) / 2.0 + 1
@@ -221,6 +243,7 @@ def main() -> int:
             "context": context,
             "page_size": engine.page_size,
             "graph": engine.use_graph,
+            "pipeline": not args.no_pipeline,
             "parallelism": "single GPU",
         },
         "prefill": prefill,

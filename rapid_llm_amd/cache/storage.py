@@ -18,6 +18,7 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
+from ..kernels.upload import upload, upload_ints
 from ..parts.base import CacheNeed
 from .manager import CacheManager, GroupSpec
 
@@ -121,18 +122,20 @@ class DeviceCache:
 
     def refresh(self) -> None:
         """Bring the device block tables and state slots up to date with the manager: rows
-        of slots whose pages changed are copied, state of newly taken slots is cleared."""
+        of slots whose pages changed are copied, state of newly taken slots is cleared.
+        Everything is queued on the current stream; the host does not wait."""
         m = self.manager
         if m.dirty_slots:
             slots = sorted(m.dirty_slots)
-            index = torch.tensor(slots, dtype=torch.int64, device=self.device)
+            index = upload_ints(slots, self.device, np.int64)
             for gid, host in m.tables.items():
-                rows = torch.from_numpy(np.ascontiguousarray(host[slots])).to(self.device)
-                self.tables[gid].index_copy_(0, index, rows)
+                self.tables[gid].index_copy_(0, index, upload(host[slots], self.device))
             m.dirty_slots.clear()
         if m.fresh_slots:
-            slots = sorted(m.fresh_slots)
+            index = None
             for layer in self.layers:
                 if layer.state is not None:
-                    layer.state[slots] = 0
+                    if index is None:
+                        index = upload_ints(sorted(m.fresh_slots), self.device, np.int64)
+                    layer.state.index_fill_(0, index, 0)
             m.fresh_slots.clear()

@@ -24,6 +24,9 @@ class EngineConfig:
     max_num_batched_tokens: int = 8192
     max_chunk_size: int = 512  # 0 turns chunked prefill off
     use_graph: bool = True  # replay decode-only steps from a captured HIP graph
+    # queue the next step before the last one's tokens are read (rapid_llm/engine/scheduler.py:
+    # 302-303); None: the environment variable RAPID_LLM_PIPELINE, on when it is not set
+    pipeline: bool | None = None
     seed: int = 0
 
     def __post_init__(self) -> None:

@@ -7,11 +7,16 @@
 // embedding: residual[t, :] = table[ids[t], :]   (float32 residual stream)
 // rapid_llm/modules/vocab_parallel.py:102-103
 // --------------------------------------------------------------------------- //
+// A negative id -(r + 1) stands for "the token chosen in row r of the previous step", which
+// the host may not have seen yet: it is read from `fed` (the sampling kernels' output)
+// (rapid_llm/engine/scheduler.py:241-249: the placeholder a device-side gather replaces).
 template <typename W>
-__global__ void embed_kernel(const int* __restrict__ ids, const W* __restrict__ table,
-                             float* __restrict__ out, int hidden, int vocab) {
+__global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ fed, int fed_rows,
+                             const W* __restrict__ table, float* __restrict__ out, int hidden,
+                             int vocab) {
     const int t = blockIdx.x;
     int id = ids[t];
+    if (id < 0 && fed && -id - 1 < fed_rows) id = fed[-id - 1];
     // ids are validated on the host; an id outside the table reads row 0 rather than faulting
     if (id < 0 || id >= vocab) id = 0;
     const W* row = table + (size_t)id * hidden;
@@ -19,15 +24,16 @@ __global__ void embed_kernel(const int* __restrict__ ids, const W* __restrict__ 
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]);
 }
 
-extern "C" int rl_embed(const int* ids, const void* table, int table_type, float* out,
-                        int tokens, int hidden, int vocab, hipStream_t stream) {
+extern "C" int rl_embed(const int* ids, const int* fed, int fed_rows, const void* table,
+                        int table_type, float* out, int tokens, int hidden, int vocab,
+                        hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     dim3 grid(tokens), block(256);
     if (table_type == RL_F32)
-        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids,
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, fed, fed_rows,
                            (const float*)table, out, hidden, vocab);
     else if (table_type == RL_BF16)
-        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids,
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, fed, fed_rows,
                            (const bf16_t*)table, out, hidden, vocab);
     else
         return RL_ERR_ARG;

@@ -14,14 +14,53 @@ from __future__ import annotations
 from pathlib import Path
 from typing import Any, Iterator, Mapping, Sequence
 
+import numpy as np
 import torch
 
 from ..config.engine_config import EngineConfig
 from ..sampling.params import SamplingParams
+from ..kernels.upload import upload_ints
 from ..sampling.sampler import Sampler, to_records
 from .outputs import CompletionOutput, RequestOutput
 from .request import Request
 from .scheduler import SamplingPlan, Scheduler, StepOutput
+
+
+class PendingStep:
+    """A step that has been queued on the device.  ``result()`` waits for it and returns its
+    :class:`StepOutput`; until then the host is free to plan and queue the next step."""
+
+    def __init__(self, sampling: SamplingPlan, host: dict[str, torch.Tensor], asked: list[int]) -> None:
+        self._sampling = sampling
+        self._host = host  # pinned copies of what the step chose and scored
+        self._asked = asked
+        self._event = torch.cuda.Event()
+        self._event.record()
+        self._output: StepOutput | None = None
+
+    def result(self) -> StepOutput:
+        if self._output is not None:
+            return self._output
+        # the step's one host synchronisation (rapid_llm/engine/scheduler.py:1000-1005)
+        self._event.synchronize()
+        sampling, host = self._sampling, self._host
+        out = StepOutput(host["ids"].tolist())
+        if self._asked:
+            records = to_records(
+                [out.token_ids[b] for b in self._asked],
+                [sampling.logprob_ks[b] for b in self._asked],
+                host["lp"].tolist(), host["top_ids"].tolist(), host["top_lp"].tolist(),
+            )
+            out.logprobs = [None] * len(out.token_ids)
+            for b, record in zip(self._asked, records):
+                out.logprobs[b] = record
+        if sampling.prompt_rows:
+            out.prompt_logprobs = to_records(
+                sampling.prompt_targets, sampling.prompt_ks,
+                host["p_lp"].tolist(), host["p_top_ids"].tolist(), host["p_top_lp"].tolist(),
+            )
+        self._output = out
+        return out
 
 
 class GpuExecutor:
@@ -32,43 +71,42 @@ class GpuExecutor:
         self.sampler = sampler
         self.cache = runner.cache
 
-    def execute(self, entries, sampling: SamplingPlan) -> StepOutput:
-        logits = self.runner.step(entries)
+    @staticmethod
+    def _to_host(t: torch.Tensor) -> torch.Tensor:
+        host = torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+        host.copy_(t, non_blocking=True)
+        return host
+
+    def launch(self, entries, sampling: SamplingPlan) -> PendingStep:
+        """Queue the step, the choice of its tokens (left in ``runner.sampled``, where the next
+        step's fed tokens are read) and the copies back to the host; does not wait."""
+        runner = self.runner
+        logits = runner.step(entries)
         in_order = sampling.logits_rows == list(range(logits.shape[0]))
         ids, _ = self.sampler.sample(
-            logits, sampling.rows, row_index=None if in_order else sampling.logits_rows
+            logits, sampling.rows, row_index=None if in_order else sampling.logits_rows, out=runner.sampled
         )
-        chosen = prompt = None
+        host = {"ids": self._to_host(ids)}
         asked = [b for b, k in enumerate(sampling.logprob_ks) if k is not None]
         if asked:
-            pick = torch.tensor(asked, dtype=torch.int64).to(ids.device)
-            chosen = self.sampler.logprobs(
+            chosen = ids if len(asked) == len(sampling.rows) else ids[upload_ints(asked, ids.device, np.int64)]
+            lp, top_ids, top_lp = self.sampler.logprobs(
                 logits,
-                ids[pick],
+                chosen,
                 max(sampling.logprob_ks[b] for b in asked),
                 rows=[sampling.rows[b] for b in asked],
                 row_index=[sampling.logits_rows[b] for b in asked],
             )
+            host.update(lp=self._to_host(lp), top_ids=self._to_host(top_ids), top_lp=self._to_host(top_lp))
         if sampling.prompt_rows:
-            prompt = self.sampler.logprobs(
+            lp, top_ids, top_lp = self.sampler.logprobs(
                 logits, sampling.prompt_targets, max(sampling.prompt_ks), row_index=sampling.prompt_rows
             )
-        # the step's one host synchronisation (rapid_llm/engine/scheduler.py:1000-1005)
-        out = StepOutput(ids.tolist())
-        if chosen is not None:
-            records = to_records(
-                [out.token_ids[b] for b in asked],
-                [sampling.logprob_ks[b] for b in asked],
-                *(t.tolist() for t in chosen),
-            )
-            out.logprobs = [None] * len(out.token_ids)
-            for b, record in zip(asked, records):
-                out.logprobs[b] = record
-        if prompt is not None:
-            out.prompt_logprobs = to_records(
-                sampling.prompt_targets, sampling.prompt_ks, *(t.tolist() for t in prompt)
-            )
-        return out
+            host.update(p_lp=self._to_host(lp), p_top_ids=self._to_host(top_ids), p_top_lp=self._to_host(top_lp))
+        return PendingStep(sampling, host, asked)
+
+    def execute(self, entries, sampling: SamplingPlan) -> StepOutput:
+        return self.launch(entries, sampling).result()
 
     def finish(self, request_id: str) -> None:
         self.runner.finish(request_id)
@@ -92,6 +130,7 @@ def build_engine(
     seed: int = 0,
     hf_overrides: Mapping[str, Any] | None = None,
     gpu_memory_utilization: float = 0.9,
+    pipeline: bool | None = None,
 ) -> Scheduler:
     from .step import ModelRunner
     from .tokenizer import load_stop_token_ids, load_tokenizer
@@ -107,6 +146,7 @@ def build_engine(
         max_num_batched_tokens=max_num_batched_tokens,
         max_chunk_size=max_chunk_size,
         use_graph=bool(use_cuda_graph),
+        pipeline=pipeline,
         seed=seed,
     )
     runner = ModelRunner(model, config, load_format=load_format, overrides=hf_overrides, device=device)
@@ -144,6 +184,7 @@ class LLM:
         num_pages: int | None = None,
         load_format: str = "auto",
         seed: int = 0,
+        pipeline: bool | None = None,
     ) -> None:
         if quantization is not None:
             raise ValueError("quantization is not supported by this engine (bfloat16 and float32 only)")
@@ -157,7 +198,7 @@ class LLM:
             max_gpu_num_blocks=max_gpu_num_blocks, device=device,
             use_cuda_graph=True if use_cuda_graph is None else use_cuda_graph, dtype=dtype,
             page_size=page_size, num_pages=num_pages, load_format=load_format, seed=seed,
-            hf_overrides=hf_overrides,
+            hf_overrides=hf_overrides, pipeline=pipeline,
         )
         self.tokenizer = self.scheduler.tokenizer
 

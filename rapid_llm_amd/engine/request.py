@@ -6,6 +6,11 @@ The tokens a request has to run are ``prompt_token_ids + output_token_ids``;
 them, the logits at that place choose the next token.  A prompt portion, a decoded token
 and the recomputation after an eviction are therefore the same thing: the next
 ``n`` uncomputed tokens.
+
+Under the launch/harvest pipeline a request may own one token that the device has chosen
+and the host has not read yet (``pending``, rapid_llm/engine/scheduler.py:214-262): it
+counts as part of the sequence, and where its id is needed the placeholder of the sampling
+row that chose it stands (``pending_row``).
 """
 
 from __future__ import annotations
@@ -16,6 +21,7 @@ from enum import Enum
 
 from ..sampling.logprobs import PositionLogprobs
 from ..sampling.params import SamplingParams
+from .feed import fed_token
 
 
 class RequestStatus(str, Enum):
@@ -46,6 +52,9 @@ class Request:
     first_token_time: float | None = None
     finish_time: float | None = None
     num_preemptions: int = 0
+    pending: int = 0  # tokens chosen on the device that the host has not read yet (0 or 1)
+    pending_row: int = -1  # the sampling row of the step in flight that chooses the pending token
+    discard: int = 0  # pending tokens that belong to nobody: the request stopped before them
 
     @property
     def prompt_len(self) -> int:
@@ -53,7 +62,7 @@ class Request:
 
     @property
     def seq_len(self) -> int:
-        return len(self.prompt_token_ids) + len(self.output_token_ids)
+        return len(self.prompt_token_ids) + len(self.output_token_ids) + self.pending
 
     @property
     def num_uncomputed(self) -> int:
@@ -65,21 +74,23 @@ class Request:
 
     @property
     def has_room(self) -> bool:
-        return len(self.output_token_ids) < self.max_new_tokens
+        return len(self.output_token_ids) + self.pending < self.max_new_tokens
 
     @property
     def prefill_done(self) -> bool:
         """Everything but the newest token is in the cache: the next step is a decode."""
-        return self.num_uncomputed <= 1 and bool(self.output_token_ids)
-
-    def token_at(self, index: int) -> int:
-        n = len(self.prompt_token_ids)
-        return self.prompt_token_ids[index] if index < n else self.output_token_ids[index - n]
+        return self.num_uncomputed <= 1 and bool(self.output_token_ids or self.pending)
 
     def tokens(self, start: int, stop: int) -> list[int]:
+        """Tokens ``[start, stop)`` of the sequence; a pending token is named by the
+        placeholder of the sampling row that chooses it."""
         n = len(self.prompt_token_ids)
-        if stop <= n:
-            return self.prompt_token_ids[start:stop]
-        if start >= n:
-            return self.output_token_ids[start - n : stop - n]
-        return self.prompt_token_ids[start:] + self.output_token_ids[: stop - n]
+        m = n + len(self.output_token_ids)
+        out: list[int] = []
+        if start < n:
+            out += self.prompt_token_ids[start : min(stop, n)]
+        if stop > n and start < m:
+            out += self.output_token_ids[max(start, n) - n : min(stop, m) - n]
+        if stop > m:
+            out += [fed_token(self.pending_row)] * (stop - max(start, m))
+        return out

@@ -26,11 +26,27 @@ go on.  Eviction is recomputation: slot and pages are given back, progress is re
 zero, and the request returns to the *front* of the queue; its generated tokens are kept
 and run again as if they were prompt, and because the i-th draw of a request depends only
 on its seed and i, it continues with exactly the tokens it would have produced.
+
+**The launch/harvest pipeline** (:818-933; on unless ``EngineConfig.pipeline`` or the
+environment variable ``RAPID_LLM_PIPELINE`` says otherwise).  ``step`` queues step N + 1 on
+the device before it reads what step N chose, so planning, packing and the harvest itself
+run while the device computes.  A request sampled in step N owns a *pending* token until the
+harvest: it counts in the request's length, and step N + 1 feeds it from the device
+(:func:`~rapid_llm_amd.engine.feed.fed_token`).  Ends that depend on counts (``max_gen_len``,
+``max_seq_len``) are known when planning and cost nothing.  Ends that depend on the token
+(a stop token, the repetition breaker) are seen one step late: the request has then ridden
+one more step, whose token is discarded, and its slot and pages are given back after that
+step.  Nobody is evicted or ended for want of pages on a guess: when pages are short, the
+step in flight is read first and the decision made on what is then known.  The tokens are
+those of the synchronous loop.  A step is run synchronously (harvest
+before planning) while a live request has a repetition penalty, whose history must hold the
+newest token.
 """
 
 from __future__ import annotations
 
 import itertools
+import os
 import time
 from collections import deque
 from dataclasses import dataclass, field
@@ -42,7 +58,10 @@ from ..sampling.params import SamplingParams
 from ..sampling.rng import derive_seed
 from .request import Request, RequestStatus
 
-REPEAT_POLL_INTERVAL = 8  # steps between checks of the repetition breaker (scheduler.py:1414)
+# Output tokens of a request between checks of the repetition breaker.  The reference polls
+# every 8th step of the engine (scheduler.py:1414); counting the request's own tokens makes
+# the end of a request independent of what else runs and of the pipeline.
+REPEAT_POLL_INTERVAL = 8
 
 
 @dataclass
@@ -85,6 +104,27 @@ class StepOutput:
     token_ids: list[int]  # parallel to SamplingPlan.rows
     logprobs: list[PositionLogprobs | None] | None = None  # parallel to rows, if any asked
     prompt_logprobs: list[PositionLogprobs] | None = None  # parallel to prompt_rows
+
+
+class _ReadFirst(Exception):
+    """Planning met a shortage of pages while a step is in flight."""
+
+
+class _Done:
+    """The handle of a step that an executor without ``launch`` has already run."""
+
+    def __init__(self, output: StepOutput) -> None:
+        self._output = output
+
+    def result(self) -> StepOutput:
+        return self._output
+
+
+@dataclass
+class _Inflight:
+    handle: Any  # .result() -> StepOutput
+    sampled: list[Request]  # parallel to the sampling rows of the step
+    scored: list[tuple[Request, int]]  # (request, prompt position) parallel to its prompt rows
 
 
 def detect_repetition(token_ids: Sequence[int], window: int = 32, min_reps: int = 3) -> bool:
@@ -133,6 +173,12 @@ class Scheduler:
         self._step_count = 0
         self.num_preemptions = 0
         self.last_plan: StepPlan | None = None
+        pipeline = getattr(config, "pipeline", None)
+        if pipeline is None:  # the reference's switch (rapid_llm/executor/worker.py:50-53), on by default here
+            pipeline = os.environ.get("RAPID_LLM_PIPELINE", "1").strip().lower() in ("1", "true", "on")
+        self.pipeline = bool(pipeline) and hasattr(executor, "launch")
+        self._inflight: _Inflight | None = None
+        self._held: list[Request] = []  # finished, but a step in flight still uses their slot and pages
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -155,6 +201,7 @@ class Scheduler:
         load_format: str = "auto",
         seed: int = 0,
         hf_overrides=None,
+        pipeline: bool | None = None,
     ) -> "Scheduler":
         """Names and defaults of rapid_llm/engine/scheduler.py:409-440 where it has them."""
         from .llm import build_engine
@@ -165,7 +212,7 @@ class Scheduler:
             max_chunk_size=max_chunk_size if enable_chunked_prefill else 0,
             max_gpu_num_blocks=max_gpu_num_blocks, device=device, use_cuda_graph=use_cuda_graph,
             dtype=dtype, page_size=page_size, num_pages=num_pages, load_format=load_format,
-            seed=seed, hf_overrides=hf_overrides,
+            seed=seed, hf_overrides=hf_overrides, pipeline=pipeline,
         )
 
     # ------------------------------------------------------------------ submission
@@ -226,15 +273,21 @@ class Scheduler:
         self._finish(request, "abort")
 
     def has_unfinished_requests(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.waiting or self.running or self._inflight is not None)
 
     # ------------------------------------------------------------------ bookkeeping
     def _finish(self, request: Request, reason: str) -> None:
+        """A token of the request that is still in flight belongs to nobody: the request
+        stopped before it.  Slot and pages are given back when that step has been read."""
         if request.status is RequestStatus.RUNNING:
             self.running.remove(request)
-            self.executor.finish(request.request_id)
+            if request.pending:
+                self._held.append(request)  # given back when the step in flight has been read
+            else:
+                self.executor.finish(request.request_id)
         elif request.status is RequestStatus.WAITING:
             self.waiting.remove(request)
+        request.discard = request.pending
         request.status = RequestStatus.FINISHED
         request.finish_reason = reason
         request.finish_time = time.monotonic()
@@ -250,6 +303,12 @@ class Scheduler:
         self.num_preemptions += 1
         self.waiting.appendleft(request)
         plan.preempted.append(request)
+
+    def _ends_at_harvest(self, request: Request) -> bool:
+        """The token in flight is the request's last, by count: it is not planned further."""
+        return request.pending > 0 and (
+            not request.has_room or request.seq_len >= self.config.max_seq_len
+        )
 
     def _portion(self, request: Request, budget: int) -> int:
         """Tokens of the request's next portion under what is left of the budget
@@ -270,10 +329,14 @@ class Scheduler:
         for request in sorted(self.running, key=lambda r: r.admission_number):
             if request.status is not RequestStatus.RUNNING or request.num_uncomputed != 1:
                 continue
+            if self._ends_at_harvest(request):
+                continue
             if budget < 1:
                 break
             rid = request.request_id
             while not cache.reserve(rid, request.seq_len, request.num_computed_tokens):
+                if self._inflight is not None:
+                    raise _ReadFirst  # the step in flight may end requests and free their pages
                 victims = [
                     r for r in self.running if r is not request and r.request_id not in granted
                 ]
@@ -329,9 +392,15 @@ class Scheduler:
     def _plan_with_progress(self) -> StepPlan:
         """A plan that runs something whenever anything can run."""
         plan = self.plan()
-        while not plan.work and self.running:
-            # every running request is stuck on pages it cannot get
-            youngest = max(self.running, key=lambda r: r.admission_number)
+
+        def stuck() -> list[Request]:
+            # running requests that have work and got none: they wait for pages
+            return [r for r in self.running if not self._ends_at_harvest(r)]
+
+        while not plan.work and stuck():
+            if self._inflight is not None:
+                raise _ReadFirst
+            youngest = max(stuck(), key=lambda r: r.admission_number)
             if len(self.running) == 1:
                 self._finish(youngest, "length")
                 plan.finished.append(youngest)
@@ -341,7 +410,10 @@ class Scheduler:
             more.preempted = plan.preempted + more.preempted
             more.finished = plan.finished + more.finished
             plan = more
-        if not plan.work and not plan.finished and self.waiting:
+        if (
+            not plan.work and not plan.finished and self.waiting and not self.running
+            and self._inflight is None and not self._held
+        ):
             raise RuntimeError(
                 f"request {self.waiting[0].request_id!r} cannot be admitted into an empty engine"
             )
@@ -349,17 +421,51 @@ class Scheduler:
 
     # ------------------------------------------------------------------ the loop
     def step(self) -> list[Request]:
-        """Plan one batch, run it, harvest the chosen tokens.  Returns the requests that
-        advanced or finished in this step (rapid_llm/engine/scheduler.py:1405-1460)."""
+        """Plan one batch, run it, harvest chosen tokens.  Returns the requests that advanced
+        or finished (rapid_llm/engine/scheduler.py:1405-1460).  Pipelined, the tokens harvested
+        are those of the step queued by the previous call (:818-933)."""
+        if self.pipeline and self._can_pipeline():
+            try:
+                launched, advanced = self._launch()
+            except _ReadFirst:
+                # pages are short: who is evicted or ended is decided on what is known, after
+                # the step in flight has been read (nothing was decided or queued so far)
+                advanced = self._harvest(self._inflight)
+                self._inflight = None
+                launched, ended = self._launch()
+                advanced += ended
+            else:
+                if self._inflight is not None:
+                    advanced += self._harvest(self._inflight)
+            self._inflight = launched
+            return advanced
+        advanced = []
+        if self._inflight is not None:  # leaving the pipeline: read what is in flight first
+            advanced += self._harvest(self._inflight)
+            self._inflight = None
+        launched, ended = self._launch()
+        advanced += ended
+        if launched is not None:
+            advanced += self._harvest(launched)
+        return advanced
+
+    def _can_pipeline(self) -> bool:
+        # the penalty reads the request's newest token from the host's list
+        return all(
+            r.params.repetition_penalty == 1.0 for r in itertools.chain(self.running, self.waiting)
+        )
+
+    def _launch(self) -> tuple["_Inflight | None", list[Request]]:
+        """Plan a step and queue it; returns what is in flight and the requests the planner
+        ended."""
         from ..sampling.sampler import RowSampling
         from .step import StepEntry
 
         plan = self._plan_with_progress()
         self.last_plan = plan
         self._step_count += 1
-        advanced: list[Request] = list(plan.finished)
         if not plan.work:
-            return advanced
+            return None, list(plan.finished)
         entries, sampled = [], []
         sampling = SamplingPlan()
         scored: list[tuple[Request, int]] = []  # (request, prompt position the record is for)
@@ -389,7 +495,7 @@ class Scheduler:
                         top_p=p.top_p,
                         repetition_penalty=p.repetition_penalty,
                         seed=r.seed,
-                        counter=len(r.output_token_ids),
+                        counter=len(r.output_token_ids) + r.pending,
                         generated=r.output_token_ids if p.repetition_penalty != 1.0 else (),
                     )
                 )
@@ -399,18 +505,35 @@ class Scheduler:
                 want.append(w.count - 1)
             entries.append(StepEntry(r.request_id, r.tokens(w.start, w.start + w.count), want))
             num_rows += len(want)
-        result = self.executor.execute(entries, sampling)
-        tokens, logprobs = result.token_ids, result.logprobs
+        if hasattr(self.executor, "launch"):
+            handle = self.executor.launch(entries, sampling)
+        else:
+            handle = _Done(self.executor.execute(entries, sampling))
+        # the plan is committed (rapid_llm/engine/batch_planner.py:462-470)
         for w in plan.work:
             w.request.num_computed_tokens = w.start + w.count
             self.cache.trim(w.request.request_id, w.request.num_computed_tokens)
-        for (request, q), record in zip(scored, result.prompt_logprobs or ()):
-            request.prompt_logprobs[q] = record
+        for row, request in enumerate(sampled):
+            request.pending += 1
+            request.pending_row = row
+        return _Inflight(handle, sampled, scored), list(plan.finished)
 
+    def _harvest(self, inflight: "_Inflight") -> list[Request]:
+        """Read a step's tokens back and retire whoever stopped
+        (rapid_llm/engine/scheduler.py:1405-1460)."""
+        result = inflight.handle.result()
+        tokens, logprobs = result.token_ids, result.logprobs
+        for (request, q), record in zip(inflight.scored, result.prompt_logprobs or ()):
+            request.prompt_logprobs[q] = record
         now = time.monotonic()
-        check_repeat = self._step_count % REPEAT_POLL_INTERVAL == 0
-        for i, request in enumerate(sampled):
+        advanced: list[Request] = []
+        for i, request in enumerate(inflight.sampled):
             token = int(tokens[i])
+            request.pending -= 1
+            if request.discard:
+                # the request stopped at an earlier harvest: this token belongs to nobody
+                request.discard -= 1
+                continue
             request.delta = ""
             if request.first_token_time is None:
                 request.first_token_time = now
@@ -427,10 +550,22 @@ class Scheduler:
                 piece = detok.append(token)
                 request.delta = piece
                 request.text += piece
-            if not request.has_room or request.seq_len >= self.config.max_seq_len:
+            outputs = len(request.output_token_ids)
+            if outputs >= request.max_new_tokens or request.prompt_len + outputs >= self.config.max_seq_len:
                 self._finish(request, "length")
-            elif check_repeat and request.params.stop_on_repeat and detect_repetition(request.output_token_ids):
+            elif (
+                request.params.stop_on_repeat
+                and outputs % REPEAT_POLL_INTERVAL == 0
+                and detect_repetition(request.output_token_ids)
+            ):
                 self._finish(request, "repeat")
+        held = []
+        for request in self._held:
+            if request.pending:
+                held.append(request)
+            else:
+                self.executor.finish(request.request_id)
+        self._held = held
         return advanced
 
     def run_to_completion(self) -> None:

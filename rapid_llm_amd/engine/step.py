@@ -27,10 +27,12 @@ from ..config.engine_config import EngineConfig
 from ..config.model_config import read_config_json
 from ..config.registry import config_from_dict
 from ..kernels import ops
+from ..kernels.upload import upload
 from ..models.causal_lm import CausalLM
 from ..parts.runtime import Runtime
 from ..weights.loader import load_model_dir
 from ..weights.random_init import random_params
+from .feed import fed_token  # noqa: F401  (part of the step function's input convention)
 
 _TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 # batch sizes decode graphs are captured for; other sizes are padded up with filler rows
@@ -44,7 +46,9 @@ class OutOfPages(CacheError):
 @dataclass
 class StepEntry:
     """One request's share of a step: its next tokens and the places among them whose
-    logits are wanted (indices into ``tokens``; may be empty)."""
+    logits are wanted (indices into ``tokens``; may be empty).  A single token may be given
+    as :func:`fed_token` ``(r)``: the token that row ``r`` of the latest sampling chose, which
+    the host need not have seen yet."""
 
     request_id: str
     tokens: Sequence[int]
@@ -74,6 +78,7 @@ class StepContext:
     h_seq_lens: list[int] = field(default_factory=list)
     max_position: int = 0
     max_seq_tokens: int = 0  # longest portion in the batch
+    fed_tokens: torch.Tensor | None = None  # [rows] what the latest sampling chose (see fed_token)
     extra: dict[str, Any] = field(default_factory=dict)  # per-step device metadata of kernels
 
 
@@ -144,6 +149,9 @@ class ModelRunner:
         self.computed: dict[str, int] = {}
         self.vocab_size = self.spec.vocab_size
         self._graphs: dict[tuple[int, int], tuple] = {}
+        # where the sampling kernels leave their choices, one row per sampled request of a
+        # step; the next step's embedding reads fed tokens from here
+        self.sampled = torch.zeros(max(1, self.engine.max_num_seqs), dtype=torch.int32, device=self.device)
 
     # ------------------------------------------------------------------ sizing
     def _decide_num_pages(self, groups) -> int:
@@ -232,6 +240,8 @@ class ModelRunner:
         slots = [cache.slot_of(e.request_id) for e in entries]
         for e in entries:
             lo, hi = min(e.tokens), max(e.tokens)
+            if len(e.tokens) == 1 and -self.sampled.numel() <= lo < 0:
+                continue  # a fed token: resolved on the device
             if lo < 0 or hi >= vocab:
                 raise ValueError(
                     f"request {e.request_id!r} has a token id outside [0, {vocab}): min {lo}, max {hi}"
@@ -287,6 +297,7 @@ class ModelRunner:
             cu_seqlens=part[6],
             logit_rows=part[7],
             block_tables=self.device_cache.tables,
+            fed_tokens=self.sampled,
             **meta,
         )
 
@@ -335,9 +346,7 @@ class ModelRunner:
         entry = self._graphs.get(key)
         if entry is None:
             static = torch.zeros(len(host), dtype=torch.int32, device=self.device)
-            pinned = torch.empty(len(host), dtype=torch.int32, pin_memory=True)
-            pinned.numpy()[:] = host
-            static.copy_(pinned, non_blocking=True)
+            upload(host, self.device, into=static)
             ctx = self._context(static, offs, dict(meta, max_position=bound - 1))
             ctx.extra["decode_only_tokens"] = torch.arange(rows, dtype=torch.int32, device=self.device)
             ctx.extra["context_bound"] = bound
@@ -356,11 +365,10 @@ class ModelRunner:
             # the graph's kernel nodes hold raw pointers: everything they point at that was
             # allocated outside the capture (the static inputs, the index list in ctx.extra)
             # must live as long as the graph does, so the context is kept with it
-            entry = (graph, static, pinned, logits, ctx)
+            entry = (graph, static, logits, ctx)
             self._graphs[key] = entry
-        graph, static, pinned, logits, _ctx = entry
-        pinned.numpy()[:] = host
-        static.copy_(pinned, non_blocking=True)
+        graph, static, logits, _ctx = entry
+        upload(host, self.device, into=static)
         graph.replay()
         return logits[:batch]
 
@@ -382,7 +390,7 @@ class ModelRunner:
             logits = self._graph_step(entries, meta)
         else:
             host, offs = self._pack(entries, meta)
-            dev = torch.from_numpy(host).to(self.device, non_blocking=False)
+            dev = upload(host, self.device)
             logits = self.model.forward(self._context(dev, offs, meta), self.device_cache.layers)
         for e in entries:
             done = self.computed.get(e.request_id, 0) + len(e.tokens)

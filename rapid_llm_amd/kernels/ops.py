@@ -13,6 +13,7 @@ from typing import Optional
 import torch
 
 from . import build
+from .upload import upload_ints
 
 F32, BF16 = 0, 1
 _TAG = {torch.float32: F32, torch.bfloat16: BF16}
@@ -86,14 +87,21 @@ def _ok(code: int, what: str) -> None:
 # --------------------------------------------------------------------------- #
 
 
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Optional[torch.Tensor] = None) -> None:
+    """``out[t] = table[ids[t]]``; an id ``-(r + 1)`` takes ``fed[r]``, the token a sampling
+    kernel chose in row ``r`` of the previous step."""
     tokens = ids.numel()
     vocab, hidden = table.shape
     _need(ids, "ids", torch.int32)
     _need(table, "embedding table")
     _need(out, "out", torch.float32, (tokens, hidden))
+    if fed is not None:
+        _need(fed, "fed", torch.int32)
     _ok(
-        core().rl_embed(_p(ids), _p(table), _tag(table.dtype), _p(out), tokens, hidden, vocab, _stream()),
+        core().rl_embed(
+            _p(ids), _p(fed), 0 if fed is None else fed.numel(), _p(table), _tag(table.dtype), _p(out),
+            tokens, hidden, vocab, _stream(),
+        ),
         "rl_embed",
     )
 
@@ -496,7 +504,7 @@ class AttentionPlan:
         self.num_decode = len(dec_tokens)
         self.num_tiles = len(tiles) // 4
         device = ctx.token_ids.device
-        packed = torch.tensor(dec_tokens + tiles, dtype=torch.int32).to(device)
+        packed = upload_ints(dec_tokens + tiles, device)
         self.seq_token = packed[: self.num_decode]
         self.tile_info = packed[self.num_decode :]
 
@@ -512,7 +520,7 @@ class AttentionPlan:
             rest = items[_FIRST_ROUND:]
             second = rest[::-1][:_FIRST_ROUND]
             middle = rest[: max(0, len(rest) - _FIRST_ROUND)]
-            order = torch.tensor(first + second + middle, dtype=torch.int32).to(device)
+            order = upload_ints(first + second + middle, device)
             self.orders[nkv] = order
         return order
 

@@ -117,7 +117,7 @@ class CausalLM:
     def forward(self, ctx, caches) -> torch.Tensor:
         """Run the tokens of ``ctx`` through every layer (which writes their keys and values)
         and return float32 logits ``[len(ctx.logit_rows), vocab]``."""
-        residual = self.embed.forward(ctx.token_ids)
+        residual = self.embed.forward(ctx.token_ids, ctx.fed_tokens)
         delta = None
         for place, li in enumerate(self.order):
             delta = self.blocks[li].forward(residual, delta, ctx, caches[place])

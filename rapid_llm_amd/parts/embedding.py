@@ -34,9 +34,10 @@ class TokenEmbedding(Part):
     def bind(self, params, runtime) -> None:
         self.table = params[self.name + ".weight"]
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, token_ids: torch.Tensor, fed_tokens: torch.Tensor | None = None) -> torch.Tensor:
+        """Rows of the table for the ids; an id ``-(r + 1)`` takes ``fed_tokens[r]``."""
         out = torch.empty((token_ids.numel(), self.hidden_size), dtype=torch.float32, device=token_ids.device)
-        ops.embed(token_ids, self.table, out)
+        ops.embed(token_ids, self.table, out, fed_tokens)
         return out
 
 

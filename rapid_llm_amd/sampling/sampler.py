@@ -16,6 +16,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops
+from ..kernels.upload import upload, upload_ints
 from .logprobs import PositionLogprobs
 
 
@@ -64,7 +65,7 @@ class Sampler:
     def _index(self, row_index: Sequence[int] | None) -> torch.Tensor | None:
         if row_index is None:
             return None
-        return torch.tensor(list(row_index), dtype=torch.int32).to(self.device)
+        return upload_ints(list(row_index), self.device)
 
     def sample(
         self,
@@ -72,16 +73,23 @@ class Sampler:
         rows: Sequence[RowSampling],
         want_logprobs: bool = False,
         row_index: Sequence[int] | None = None,
+        out: torch.Tensor | None = None,
     ) -> tuple[torch.Tensor, torch.Tensor | None]:
         """``logits [R, vocab]`` float32 -> chosen ids ``[n]`` int32 (on the device) and,
         if asked, the chosen tokens' log-probabilities ``[n]`` float32.  Sampling row ``b``
         reads row ``row_index[b]`` of the logits; without an index there is one sampling
-        row per row of logits, in order."""
+        row per row of logits, in order.  ``out`` (int32, at least ``n`` long) receives the
+        ids in place of a new tensor.  Nothing here waits for the device."""
         n = len(rows)
         reads = len(row_index) if row_index is not None else logits.shape[0]
         if n != reads:
             raise ValueError(f"{reads} rows of logits for {n} sampling rows")
-        out = torch.empty(n, dtype=torch.int32, device=self.device)
+        if out is None:
+            out = torch.empty(n, dtype=torch.int32, device=self.device)
+        elif out.numel() < n:
+            raise ValueError(f"{n} sampling rows do not fit an output of {out.numel()}")
+        else:
+            out = out[:n]
         if n == 0:
             return out, (torch.empty(0, dtype=torch.float32, device=self.device) if want_logprobs else None)
         index = self._index(row_index)
@@ -90,7 +98,7 @@ class Sampler:
             ops.argmax(logits, out, index)
             return out, None
         packed, words, any_penalty = _pack_rows(rows)
-        dev = torch.from_numpy(packed).to(self.device)
+        dev = upload(packed, self.device)
         logprob = torch.empty(n, dtype=torch.float32, device=self.device) if want_logprobs else None
         ops.sample(
             logits, dev[:words], dev[words:] if any_penalty else None, out, logprob, any_penalty, index
@@ -113,8 +121,9 @@ class Sampler:
         698-716).  Without, the raw logits are scored, as for the tokens of a prompt
         (:425-447)."""
         if not isinstance(targets, torch.Tensor):
-            targets = torch.tensor(list(targets), dtype=torch.int32)
-        targets = targets.to(device=self.device, dtype=torch.int32)
+            targets = upload_ints(list(targets), self.device)
+        elif targets.device != self.device or targets.dtype != torch.int32:
+            targets = targets.to(device=self.device, dtype=torch.int32)
         n = targets.shape[0]
         if rows is not None and len(rows) != n:
             raise ValueError(f"{n} targets for {len(rows)} sampling rows")
@@ -122,7 +131,7 @@ class Sampler:
         if rows is None:
             return ops.logprobs(logits, targets, k, row_index=index)
         packed, words, any_penalty = _pack_rows(rows)
-        dev = torch.from_numpy(packed).to(self.device)
+        dev = upload(packed, self.device)
         return ops.logprobs(
             logits, targets, k, dev[:words], dev[words:] if any_penalty else None, any_penalty, index
         )

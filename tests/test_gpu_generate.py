@@ -193,6 +193,45 @@ def test_stop_tokens_and_stream(tmp_path):
     assert sum(1 for s in seen) >= 5
 
 
+@pytest.mark.parametrize("dtype,graph", [("float32", False), ("bfloat16", True)])
+def test_pipeline_gives_the_tokens_of_the_synchronous_loop(tmp_path, dtype, graph):
+    """Steps queued before the last one's tokens are read (decoded tokens fed from the device,
+    stop tokens seen a step late) against every step read before the next is planned: greedy
+    and sampled requests, a stop token, portions beside decoded tokens, few pages."""
+    from rapid_llm_amd import SamplingParams
+
+    cfg, page, seed = TINY["B"]
+    model_dir = make_model_dir(tmp_path, "B", dtype)
+    prompts = [random_tokens(n, cfg["vocab_size"], seed + 7 * n) for n in (3, 40, 1, 19, 26, 8)]
+    params = [SamplingParams(temperature=0.0 if i % 2 == 0 else 0.8, top_p=0.9, max_gen_len=6 + 5 * i, seed=i,
+                             logprobs=1 if i == 1 else None)
+              for i in range(len(prompts))]
+    common = dict(max_seq_len=128, max_chunk_size=16, max_num_batched_tokens=40, max_num_seqs=4,
+                  use_cuda_graph=graph)
+    free = _llm(model_dir, dtype, page, pipeline=False, **common).generate(prompts, params)
+    stop = free[4].token_ids[9]
+    (model_dir / "generation_config.json").write_text('{"eos_token_id": [%d]}' % stop)
+    outs = {}
+    for pipeline in (False, True):
+        for pages in (200, 8):
+            llm = _llm(model_dir, dtype, page, pipeline=pipeline, num_pages=pages, **common)
+            assert llm.scheduler.pipeline == pipeline
+            outs[pipeline, pages] = llm.generate(prompts, params)
+            llm.scheduler.cache.check_invariants()
+            assert not llm.scheduler.cache.live_requests() and not llm.scheduler._held
+            if pages == 8:
+                assert llm.scheduler.num_preemptions > 0
+    base = outs[False, 200]
+    assert any(o.outputs[0].finish_reason == "eos" for o in base)
+    for key, got in outs.items():
+        if dtype == "bfloat16" and key[1] != 200:
+            continue  # another schedule rounds differently in bfloat16; float32 is exact
+        for a, b in zip(base, got):
+            assert a.token_ids == b.token_ids and a.outputs[0].finish_reason == b.outputs[0].finish_reason, key
+            if a.outputs[0].logprobs is not None:
+                assert [r.token_id for r in a.outputs[0].logprobs] == [r.token_id for r in b.outputs[0].logprobs]
+
+
 def test_command_line_batch(tmp_path, capsys):
     from rapid_llm_amd.cli import main
 

@@ -302,6 +302,22 @@ def test_gemm_bf16_swiglu_fused(shape):
     assert ops.gemm_bf16_swiglu(torch.zeros(33, k, dtype=torch.bfloat16, device=DEV), w.to(DEV)) is None
 
 
+def test_embed_takes_fed_tokens_from_the_sampling_buffer():
+    """An id -(r + 1) reads row r of the buffer the sampling kernels write; other ids are
+    the rows they name; an id that names no row of either reads row 0 and never faults."""
+    ops = _ops()
+    torch.manual_seed(9)
+    table = torch.randn(37, 24)
+    fed = torch.tensor([5, 36, 0, 11], dtype=torch.int32)
+    ids = torch.tensor([3, -1, -4, 36, -2, -9, 99], dtype=torch.int32)
+    out = torch.empty(len(ids), 24, dtype=torch.float32, device=DEV)
+    ops.embed(ids.to(DEV), table.to(DEV), out, fed.to(DEV))
+    want = table[[3, 5, 11, 36, 36, 0, 0]]
+    assert torch.equal(out.cpu(), want)
+    ops.embed(ids.to(DEV), table.to(DEV), out)  # no buffer: a negative id reads row 0
+    assert torch.equal(out.cpu(), table[[3, 0, 0, 36, 0, 0, 0]])
+
+
 def test_embed_and_argmax():
     ops = _ops()
     vocab, hidden = 503, 96

@@ -7,6 +7,7 @@ import pytest
 
 from rapid_llm_amd.cache import CacheManager, GroupSpec
 from rapid_llm_amd.config import EngineConfig
+from rapid_llm_amd.engine.feed import fed_row, fed_token
 from rapid_llm_amd.engine.request import RequestStatus
 from rapid_llm_amd.engine.scheduler import Scheduler, StepOutput, detect_repetition
 from rapid_llm_amd.sampling import PositionLogprobs, SamplingParams
@@ -65,6 +66,62 @@ class ScriptedExecutor:
         self.cache.release(request_id)
         self.computed.pop(request_id, None)
         self.fed.pop(request_id, None)
+
+
+class PipelinedExecutor(ScriptedExecutor):
+    """The same, with ``launch``: the result of a step may be read after the next step has
+    been queued.  A fed token must name the row of the previous launch in which its own
+    request was sampled; it is replaced by what that row chose, as the device would."""
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.previous = []  # (request id, token) per sampling row of the latest launch
+        self.unread = 0
+        self.max_unread = 0
+        self.history = {}  # every token fed for a request, over its evictions too: position -> token
+
+    def launch(self, entries, sampling):
+        resolved = []
+        for e in entries:
+            tokens = list(e.tokens)
+            if tokens[0] < 0:
+                assert len(tokens) == 1, "only a single token can be fed from the device"
+                rid, token = self.previous[fed_row(tokens[0])]
+                assert rid == e.request_id, "a fed token names another request's row"
+                tokens = [token]
+            assert min(tokens) >= 0
+            start = self.computed.get(e.request_id, 0)
+            for i, t in enumerate(tokens):
+                assert self.history.setdefault((e.request_id, start + i), t) == t, "a position changed its token"
+            resolved.append(type(e)(e.request_id, tokens, e.want))
+        result = self.execute(resolved, sampling)
+        rids = [e.request_id for e, n in zip(entries, [len(e.want) for e in entries])
+                if e.want and e.want[-1] == len(e.tokens) - 1]
+        sampled_rids = []
+        num_rows, k = 0, 0
+        for e in entries:
+            if k < len(sampling.rows) and e.want and sampling.logits_rows[k] == num_rows + len(e.want) - 1:
+                sampled_rids.append(e.request_id)
+                k += 1
+            num_rows += len(e.want)
+        self.previous = list(zip(sampled_rids, result.token_ids))
+        self.unread += 1
+        self.max_unread = max(self.max_unread, self.unread)
+        executor = self
+
+        class Handle:
+            def result(self_inner):
+                executor.unread -= 1
+                return result
+
+        return Handle()
+
+
+def _make_pipelined(num_pages=64, page=4, seqs=4, max_len=128, token=None, pipeline=True, **cfg):
+    ex = PipelinedExecutor(num_pages, page, seqs, max_len, token=token)
+    config = EngineConfig(max_seq_len=max_len, page_size=page, num_pages=num_pages, max_num_seqs=seqs,
+                          pipeline=pipeline, **{"max_num_batched_tokens": 64, "max_chunk_size": 16, **cfg})
+    return Scheduler(ex, config, stop_token_ids=[EOS]), ex
 
 
 def _make(num_pages=64, page=4, seqs=4, max_len=128, token=None, **cfg):
@@ -367,3 +424,118 @@ def test_sampling_params_validation():
         with pytest.raises(ValueError):
             SamplingParams(**bad)
     assert SamplingParams(temperature=0).is_greedy and not SamplingParams().is_greedy
+
+
+# ------------------------------------------------------------------ the launch/harvest pipeline
+def _workload(scheduler, seed, n=9, penalty=False):
+    import random
+
+    rng = random.Random(seed)
+    requests = []
+    for i in range(n):
+        prompt = [rng.randrange(50) for _ in range(rng.choice([1, 2, 5, 17, 30]))]
+        params = SamplingParams(
+            temperature=0.0, max_gen_len=rng.choice([1, 2, 3, 9, 24]),
+            repetition_penalty=1.3 if penalty and i % 3 == 0 else 1.0,
+            stop_on_repeat=i % 4 == 0, logprobs=0 if i % 2 else None,
+            prompt_logprobs=1 if i % 5 == 0 else None,
+        )
+        requests.append(scheduler.add_request(prompt, params))
+    return requests
+
+
+def _token_with_stops(rid, i):
+    # some requests meet a stop token early, some late, some never
+    n = int(rid.split("-")[1])
+    return EOS if (n % 3 == 1 and i == 2 + n % 5) else (n * 31 + i * 7) % 50
+
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("pool", [200, 21, 13])
+def test_pipeline_changes_no_token(seed, pool):
+    """Queueing step N + 1 before step N is read gives every request the tokens, the finish
+    reason and the records of the synchronous loop: ample pages, and pools so small that
+    requests are evicted (the schedules then differ, the results must not)."""
+    outcomes = []
+    for pipeline in (False, True):
+        s, ex = _make_pipelined(num_pages=pool, page=4, seqs=3, max_len=64, token=_token_with_stops,
+                                pipeline=pipeline, max_num_batched_tokens=24, max_chunk_size=8)
+        requests = _workload(s, seed)
+        steps = 0
+        while s.has_unfinished_requests():
+            s.step()
+            steps += 1
+            assert steps < 2000
+        assert ex.max_unread == (2 if pipeline else 1)
+        assert not ex.cache.live_requests() and not s._held and ex.unread == 0
+        ex.cache.check_invariants()
+        outcomes.append([
+            (r.output_token_ids, r.finish_reason,
+             None if r.output_logprobs is None else [x.token_id for x in r.output_logprobs],
+             None if r.prompt_logprobs is None else [x and x.token_id for x in r.prompt_logprobs])
+            for r in requests
+        ])
+        assert all(r.pending == 0 and r.discard == 0 for r in requests)
+    assert outcomes[0] == outcomes[1]
+
+
+def test_pipeline_feeds_tokens_from_the_device_and_stops_one_step_late():
+    s, ex = _make_pipelined(token=lambda rid, i: EOS if i == 3 else 40 + i)
+    r = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=10))
+    while s.has_unfinished_requests():
+        s.step()
+    assert r.output_token_ids == [40, 41, 42] and r.finish_reason == "eos"
+    # prompt, then one decoded token a step; the step after the stop token ran and was dropped
+    assert [shape for shape in ex.steps] == [[(r.request_id, 3, True)]] + [[(r.request_id, 1, True)]] * 4
+    assert not ex.cache.live_requests()
+
+
+def test_pipeline_ends_by_count_cost_no_extra_step():
+    s, ex = _make_pipelined()
+    r = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=4))
+    while s.has_unfinished_requests():
+        s.step()
+    assert len(r.output_token_ids) == 4 and r.finish_reason == "length"
+    assert len(ex.steps) == 4  # the prompt's step chooses the first token, three decodes the rest
+    s, ex = _make_pipelined(max_len=8)
+    r = s.add_request([1, 2, 3, 4, 5], SamplingParams(temperature=0.0))
+    while s.has_unfinished_requests():
+        s.step()
+    assert r.seq_len == 8 and r.finish_reason == "length" and len(ex.steps) == 3
+
+
+def test_a_penalty_falls_back_to_the_synchronous_loop():
+    outcomes = []
+    for pipeline in (False, True):
+        s, ex = _make_pipelined(pipeline=pipeline, seqs=3, token=_token_with_stops)
+        requests = _workload(s, 3, penalty=True)
+        while s.has_unfinished_requests():
+            s.step()
+        outcomes.append([(r.output_token_ids, r.finish_reason) for r in requests])
+        assert not ex.cache.live_requests()
+    assert outcomes[0] == outcomes[1]
+
+
+def test_abort_while_a_step_is_in_flight():
+    s, ex = _make_pipelined()
+    r = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=10))
+    q = s.add_request([4, 5], SamplingParams(temperature=0.0, max_gen_len=3))
+    s.step()
+    s.step()
+    assert r.pending == 1
+    s.abort(r.request_id)
+    assert r.finish_reason == "abort" and ex.cache.has(r.request_id)  # held until the step is read
+    kept = list(r.output_token_ids)
+    while s.has_unfinished_requests():
+        s.step()
+    assert r.output_token_ids == kept and not ex.cache.live_requests()
+    assert len(q.output_token_ids) == 3
+
+
+def test_request_tokens_name_the_pending_row():
+    s, ex = _make_pipelined()
+    r = s.add_request([7, 8, 9], SamplingParams(temperature=0.0, max_gen_len=5))
+    s.step()
+    assert r.pending == 1 and r.seq_len == 4 and r.tokens(2, 4) == [9, fed_token(0)]
+    s.step()  # queues the decode of the fed token, then reads the first token
+    assert r.output_token_ids == [1000] and r.pending == 1 and r.tokens(0, 5) == [7, 8, 9, 1000, fed_token(0)]
