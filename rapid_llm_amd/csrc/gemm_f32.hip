@@ -1,73 +1,155 @@
-// True float32 matrix product C[M,N] = A[M,K] * W[N,K]^T with float32 FMA only: no matrix
-// cores, no reduced-precision mode.  The sum over k runs in ascending order in every
-// thread, so an output element does not depend on M, on the tile it falls in, or on what
-// else is in the batch.
+// True float32 matrix product C[M,N] = A[M,K] * W[N,K]^T on the matrix cores' float32
+// instruction (v_mfma_f32_16x16x4_f32: float32 operands, float32 accumulation; no
+// reduced-precision mode).
+//
+// One order of summation for every output element, whatever M, the tile it falls in or what
+// else is in the batch, so that results are equal bit for bit however the rows are cut:
+//   * K is cut in chunks of 16; the chunks are dealt to the 8 waves of a workgroup as 8
+//     contiguous runs of ceil(chunks / 8);
+//   * a wave walks its chunks in ascending order; a chunk is four matrix instructions on one
+//     accumulator, instruction j taking the k  {j, 4 + j, 8 + j, 12 + j}  of the chunk (lane
+//     group g supplies k = 4 g + j, from one 16-byte load of k = 4g .. 4g + 3);
+//   * the 8 partial results are added in the order of the waves.
+// k beyond K contribute zeros.
+//
+// The transposed product is computed (W supplies the A operand, the rows of A the B operand),
+// so a lane's four results are four consecutive n of one row of C.  A workgroup owns NT x MT
+// tiles of 16 x 16; NT and MT only decide how often an operand is reused.
 #include "common.h"
 
-#define TM 64
-#define TN 64
-#define TK 16
-#define PAD 1
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A,
-                                                       const float* __restrict__ W,
-                                                       float* __restrict__ C, int M, int N, int K,
-                                                       int lda, int ldw, int ldc) {
-    __shared__ float As[TK][TM + PAD];
-    __shared__ float Ws[TK][TN + PAD];
-    const int tid = threadIdx.x;
-    const int m0 = blockIdx.y * TM;
-    const int n0 = blockIdx.x * TN;
-    const int lr = tid / 4;        // 0..63: row of the tile this thread loads
-    const int lk = (tid % 4) * 4;  // 0,4,8,12: first of its four k
-    const int ty = tid / 16, tx = tid % 16;
-    float acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+#define FW 8    // waves per workgroup = runs of K
+#define FCH 16  // k per chunk
+#define RED_TILES 4  // tiles reduced through LDS at a time
 
-    for (int k0 = 0; k0 < K; k0 += TK) {
+// four consecutive floats of a row, zeros beyond `limit` (elements left in the row)
+template <bool VEC>
+__device__ inline f32x4 load_k4(const float* p, int limit) {
+    if (VEC) {
+        if (limit >= 4) return *reinterpret_cast<const f32x4*>(p);
+        return (f32x4){0.f, 0.f, 0.f, 0.f};  // VEC: K is a multiple of 4, a piece is whole or absent
+    }
+    f32x4 v;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int k = k0 + lk + i;
-            const int am = m0 + lr, wn = n0 + lr;
-            As[lk + i][lr] = (am < M && k < K) ? A[(size_t)am * lda + k] : 0.f;
-            Ws[lk + i][lr] = (wn < N && k < K) ? W[(size_t)wn * ldw + k] : 0.f;
-        }
-        __syncthreads();
+    for (int i = 0; i < 4; ++i) v[i] = i < limit ? p[i] : 0.f;
+    return v;
+}
+
+template <int NT, int MT, bool VEC>
+__global__ __launch_bounds__(FW* RL_WAVE) void gemm_f32_kernel(
+    const float* __restrict__ A, const float* __restrict__ W, float* __restrict__ C, int M, int N,
+    int K, int lda, int ldw, int ldc) {
+    __shared__ float red[FW][RED_TILES * 256];
+
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int r16 = lane & 15;
+    const int g = lane >> 4;
+    const int n0 = blockIdx.x * NT * 16;
+    const int m0 = blockIdx.y * MT * 16;
+
+    // rows beyond the matrices read the last row; their results are dropped at the end
+    const float* wrow[NT];
+    const float* arow[MT];
+    bool aok[MT];
 #pragma unroll
-        for (int k = 0; k < TK; ++k) {
-            float a[4], b[4];
+    for (int nt = 0; nt < NT; ++nt)
+        wrow[nt] = W + (size_t)min(n0 + nt * 16 + r16, N - 1) * ldw + 4 * g;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+    for (int mt = 0; mt < MT; ++mt) {
+        aok[mt] = m0 + mt * 16 + r16 < M;
+        arow[mt] = A + (size_t)min(m0 + mt * 16 + r16, M - 1) * lda + 4 * g;
+    }
+
+    f32x4 acc[NT][MT];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = Ws[k][tx * 4 + j];
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    const int chunks = (K + FCH - 1) / FCH;
+    const int per = (chunks + FW - 1) / FW;
+    const int c_lo = min(chunks, wave * per), c_hi = min(chunks, c_lo + per);
+
+    f32x4 wv[NT], av[MT], wn[NT], an[MT];
+    auto load = [&](int c, f32x4* wd, f32x4* ad) {
+        const int k = c * FCH + 4 * g;  // this lane's first k of the chunk
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wd[nt] = load_k4<VEC>(wrow[nt] + c * FCH, K - k);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            ad[mt] = aok[mt] ? load_k4<VEC>(arow[mt] + c * FCH, K - k) : (f32x4){0.f, 0.f, 0.f, 0.f};
+    };
+    if (c_lo < c_hi) load(c_lo, wv, av);
+    for (int c = c_lo; c < c_hi; ++c) {
+        if (c + 1 < c_hi) load(c + 1, wn, an);  // the next chunk's loads fly during this one's products
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[nt][mt] =
+                        __builtin_amdgcn_mfma_f32_16x16x4f32(wv[nt][j], av[mt][j], acc[nt][mt], 0, 0, 0);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wv[nt] = wn[nt];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) av[mt] = an[mt];
+    }
+
+    // the waves' partial tiles are added in the order of the waves, RED_TILES tiles at a time
+    constexpr int TILES = NT * MT;
+#pragma unroll
+    for (int t0 = 0; t0 < TILES; t0 += RED_TILES) {
+        if (t0 > 0) __syncthreads();
+#pragma unroll
+        for (int t = t0; t < t0 + RED_TILES && t < TILES; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
-        }
+                red[wave][((t - t0) * 4 + i) * 64 + lane] = acc[t / MT][t % MT][i];
         __syncthreads();
-    }
+        const int count = min(RED_TILES, TILES - t0) * 256;
+        for (int e = threadIdx.x; e < count; e += FW * RL_WAVE) {
+            const int ln = e & 63;
+            const int i = (e >> 6) & 3;
+            const int t = t0 + (e >> 8);
+            const int n = n0 + (t / MT) * 16 + 4 * (ln >> 4) + i;
+            const int m = m0 + (t % MT) * 16 + (ln & 15);
+            if (n >= N || m >= M) continue;
+            float v = red[0][e];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m0 + ty * 4 + i;
-        if (m >= M) continue;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + tx * 4 + j;
-            if (n < N) C[(size_t)m * ldc + n] = acc[i][j];
+            for (int w = 1; w < FW; ++w) v += red[w][e];
+            C[(size_t)m * ldc + n] = v;
         }
     }
 }
 
+template <int NT, int MT>
+static int launch(const float* A, const float* W, float* C, int M, int N, int K, int lda, int ldw,
+                  int ldc, hipStream_t stream) {
+    dim3 grid((N + NT * 16 - 1) / (NT * 16), (M + MT * 16 - 1) / (MT * 16)), block(FW * RL_WAVE);
+    if (grid.y > 65535) return RL_ERR_ARG;
+    const bool vec = K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 &&
+                     (reinterpret_cast<uintptr_t>(A) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(W) & 15) == 0;
+    if (vec)
+        hipLaunchKernelGGL((gemm_f32_kernel<NT, MT, true>), grid, block, 0, stream, A, W, C, M, N, K,
+                           lda, ldw, ldc);
+    else
+        hipLaunchKernelGGL((gemm_f32_kernel<NT, MT, false>), grid, block, 0, stream, A, W, C, M, N,
+                           K, lda, ldw, ldc);
+    return rl_launch_status();
+}
+
+// Rows of A and W may be strided; the inner dimension is contiguous.  The tiling follows M:
+// few rows stream the weights once with as many workgroups as there are 16-row tiles of W;
+// many rows reuse each operand four times.
 extern "C" int rl_gemm_f32(const float* A, const float* W, float* C, int M, int N, int K, int lda,
                            int ldw, int ldc, hipStream_t stream) {
     if (M <= 0 || N <= 0) return RL_OK;
     if (K <= 0 || lda < K || ldw < K || ldc < N) return RL_ERR_ARG;
-    dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM), block(256);
-    if (grid.y > 65535) return RL_ERR_ARG;
-    hipLaunchKernelGGL(gemm_f32_kernel, grid, block, 0, stream, A, W, C, M, N, K, lda, ldw, ldc);
-    return rl_launch_status();
+    if (M <= 16) return launch<1, 1>(A, W, C, M, N, K, lda, ldw, ldc, stream);
+    if (M <= 32) return launch<2, 2>(A, W, C, M, N, K, lda, ldw, ldc, stream);
+    return launch<4, 4>(A, W, C, M, N, K, lda, ldw, ldc, stream);
 }

@@ -261,7 +261,8 @@ def test_qknorm_rope_kvwrite(dtype, shape, many):
     assert torch.isnan(kc[~written_k]).all()  # nothing else was touched
 
 
-@pytest.mark.parametrize("shape", [(1, 96, 64), (7, 503, 96), (130, 200, 333), (64, 64, 16)])
+@pytest.mark.parametrize("shape", [(1, 96, 64), (7, 503, 96), (130, 200, 333), (64, 64, 16), (33, 48, 7),
+                                   (40, 1000, 4100), (19, 70, 130)])
 def test_gemm_f32(shape):
     ops = _ops()
     m, n, k = shape
@@ -270,10 +271,33 @@ def test_gemm_f32(shape):
     ops.gemm_f32(a.to(DEV), w.to(DEV), out)
     want = (a.double() @ w.double().T).float()
     torch.testing.assert_close(out.cpu(), want, rtol=1e-5, atol=1e-5 * math.sqrt(k))
-    # a row's result does not depend on the rows beside it
-    out1 = torch.empty(1, n, device=DEV)
-    ops.gemm_f32(a[m // 2 : m // 2 + 1].to(DEV), w.to(DEV), out1)
-    assert torch.equal(out1[0], out[m // 2])
+    # a row's result does not depend on the rows beside it, nor on the tiling that their
+    # number selects (1, up to 16, up to 32, more)
+    for lo, hi in [(m // 2, m // 2 + 1), (0, min(m, 9)), (max(0, m - 20), m), (max(0, m - 33), m)]:
+        part = torch.empty(hi - lo, n, device=DEV)
+        ops.gemm_f32(a[lo:hi].to(DEV), w.to(DEV), part)
+        assert torch.equal(part, out[lo:hi]), (shape, lo, hi)
+    # views: rows of wider matrices, a start that is not 16-byte aligned
+    wide_a = torch.randn(m, k + 5).to(DEV)
+    wide_w = torch.randn(n, k + 5).to(DEV)
+    wide_out = torch.zeros(m, n + 3, device=DEV)
+    ops.gemm_f32(wide_a[:, 1 : k + 1], wide_w[:, 1 : k + 1], wide_out[:, 2 : n + 2])
+    ref = (wide_a[:, 1 : k + 1].double() @ wide_w[:, 1 : k + 1].double().T).float()
+    torch.testing.assert_close(wide_out[:, 2 : n + 2], ref, rtol=1e-5, atol=1e-5 * math.sqrt(k))
+    assert float(wide_out[:, :2].abs().max()) == 0.0 and float(wide_out[:, n + 2 :].abs().max()) == 0.0
+
+
+def test_gemm_f32_keeps_what_bfloat16_would_lose():
+    """A true float32 product: a term 2^-12 of its neighbours survives (it would vanish in a
+    product with bfloat16 or tf32-like operands)."""
+    ops = _ops()
+    k = 64
+    a = torch.ones(1, k)
+    w = torch.ones(1, k)
+    w[0, 17] = 1.0 + 2.0 ** -12
+    out = torch.empty(1, 1, device=DEV)
+    ops.gemm_f32(a.to(DEV), w.to(DEV), out)
+    assert out.item() == k + 2.0 ** -12
 
 
 @pytest.mark.parametrize("shape", [(1, 503, 96), (8, 4096, 4096), (16, 300, 1000), (64, 1000, 12288), (17, 6144, 4096), (200, 331, 80), (3, 24, 48)])
