@@ -358,7 +358,12 @@ class ModelRunner:
                 self.model.forward(ctx, self.device_cache.layers)
             current.wait_stream(side)
             torch.cuda.synchronize()
-            ctx.extra = {k: v for k, v in ctx.extra.items() if k in ("decode_only_tokens", "context_bound")}
+            # launch data that depends on the batch's shape only was uploaded by that run and is
+            # kept: nothing may be copied from the host while the graph is recorded
+            ctx.extra = {
+                k: v for k, v in ctx.extra.items()
+                if k in ("decode_only_tokens", "context_bound") or (isinstance(k, tuple) and k[0] == "f32_tiles")
+            }
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, self.device_cache.layers)

@@ -40,7 +40,7 @@ CORE_SOURCES = (
     "sampling.hip",
     "gemm_bf16.hip",
 )
-ATTENTION_SOURCES = ("attention_mfma.hip",)
+ATTENTION_SOURCES = ("attention_mfma.hip", "attention_f32.hip")
 HEADERS = ("common.h",)
 
 # head sizes built ahead of time by build_all(): every one the kernels take.  A fresh

@@ -535,6 +535,68 @@ _MIN_SPLIT_KEYS = 128
 _MAX_SPLIT_PAGES = 1024  # page ids of one split are staged in LDS
 
 
+def _f32_tiles(ctx, group: int) -> tuple[torch.Tensor, int]:
+    """Tiles of 16 (token, head of the group) rows, request by request: ``[tiles, 3]`` int32
+    (first token of the request in the step, its tokens, first row of the tile)."""
+    key = ("f32_tiles", group)
+    made = ctx.extra.get(key)
+    if made is None:
+        tiles: list[int] = []
+        at = 0
+        for n in ctx.h_seq_lens:
+            for row0 in range(0, n * group, 16):
+                tiles += [at, n, row0]
+            at += n
+        made = (upload_ints(tiles, ctx.token_ids.device), len(tiles) // 3)
+        ctx.extra[key] = made
+    return made
+
+
+def attention_f32(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    out: torch.Tensor,
+    ctx,
+    block_table: torch.Tensor,
+    page_size: int,
+    nq: int,
+    nkv: int,
+    d: int,
+    window: int,
+    scale: float,
+) -> None:
+    """float32 attention of every token of the step on the float32 matrix instruction; a
+    row's result is the same bit for bit however the step was cut."""
+    tokens = q.shape[0]
+    pages = k_cache.shape[0]
+    _need(q, "q", torch.float32, (tokens, nq * d))
+    _need(out, "out", torch.float32, (tokens, nq * d))
+    _need(k_cache, "k_cache", torch.float32, (pages, nkv, page_size, d))
+    _need(v_cache, "v_cache", torch.float32, (pages, nkv, d, page_size))
+    _need(ctx.positions, "positions", torch.int32, (tokens,))
+    _need(ctx.token_slot, "token_slot", torch.int32, (tokens,))
+    _need(block_table, "block_table", torch.int32)
+    if page_size % 4:
+        raise KernelError(f"the float32 attention reads four keys of a page at once: page size {page_size}")
+    if ctx.max_position // page_size >= block_table.shape[1]:
+        raise KernelError(
+            f"position {ctx.max_position} needs page {ctx.max_position // page_size} of a block table "
+            f"with {block_table.shape[1]} columns"
+        )
+    if nkv > 65535:
+        raise KernelError(f"{nkv} kv heads exceed the launch grid")
+    tiles, num_tiles = _f32_tiles(ctx, nq // nkv)
+    _ok(
+        attention_lib(d).rl_attn_f32(
+            _p(q), _p(k_cache), _p(v_cache), _p(out), _p(tiles), num_tiles, _p(ctx.positions),
+            _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv, window,
+            ctypes.c_float(scale), _stream(),
+        ),
+        "rl_attn_f32",
+    )
+
+
 def paged_attention(
     q: torch.Tensor,
     k_cache: torch.Tensor,
@@ -551,8 +613,12 @@ def paged_attention(
 ) -> None:
     """Attention of every token of the step over its request's cached keys.
 
-    float32 runs the FMA kernel.  bfloat16 runs the matrix-core kernels: single tokens go
+    float32 runs the float32 matrix-core kernel (head sizes in steps of 16; the FMA kernel
+    otherwise).  bfloat16 runs the bfloat16 matrix-core kernels: single tokens go
     to the split-key decode kernel, portions to the tiled prefill kernel."""
+    if q.dtype == torch.float32 and d % 16 == 0:
+        attention_f32(q, k_cache, v_cache, out, ctx, block_table, page_size, nq, nkv, d, window, scale)
+        return
     if q.dtype != torch.bfloat16:
         attention_generic(
             q, k_cache, v_cache, out, ctx.positions, ctx.token_slot, block_table, page_size,

@@ -116,6 +116,29 @@ def test_paged_attention(case, dtype):
         torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("case", ATTN_CASES[:7], ids=lambda c: f"h{c[0]}kv{c[1]}d{c[2]}p{c[3]}w{c[4]}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_attention_generic(case, dtype):
+    """The FMA kernel that serves what the matrix-core kernels refuse, called by itself."""
+    ops = _ops()
+    nq, nkv, d, page, window, seqs = case
+    q, kc, vc, table, ctx, want = _paged_problem(seqs, nq, nkv, d, page, dtype, seed=3 + d, window=window)
+    out = torch.full_like(q, float("nan"))
+    ops.attention_generic(q, kc, vc, out, ctx.positions, ctx.token_slot, table, page, nq, nkv, d, window,
+                          1.0 / math.sqrt(d), ctx.max_position)
+    tol = dict(rtol=1e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(out.float().cpu(), want, **tol)
+
+
+def test_attention_f32_head_size_off_the_grid_takes_the_generic_kernel():
+    ops = _ops()
+    nq, nkv, d, page = 6, 2, 24, 4
+    q, kc, vc, table, ctx, want = _paged_problem([(9, 1), (0, 21)], nq, nkv, d, page, torch.float32, seed=2)
+    out = torch.full_like(q, float("nan"))
+    ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, 0, 1.0 / math.sqrt(d))
+    torch.testing.assert_close(out.cpu(), want, rtol=1e-5, atol=2e-6)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("far", [3, 257, 640])
 def test_attention_finds_a_far_key(dtype, far):
