@@ -230,7 +230,7 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
     const int col = lane & 15;  // row of the attention problem = query head of the group
     const int g = lane >> 4;
 
-    const int t = seq_token[seq];
+    const int t = seq_token ? seq_token[seq] : seq;  // null: the step holds single tokens only
     const int pos = positions[t];
     const int* table = block_table + (size_t)token_slot[t] * table_stride;
     const int kend = pos + 1;
@@ -487,7 +487,7 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o,
                                   const int* __restrict__ seq_token, int nq, int nsplit) {
     const int seq = blockIdx.x, head = blockIdx.y;
     const size_t slot0 = ((size_t)seq * nq + head) * nsplit;
-    const int t = seq_token[seq];
+    const int t = seq_token ? seq_token[seq] : seq;
     const int d = threadIdx.x;
     if (d >= D) return;
     float mm = -INFINITY, wsum = 0.f, o = 0.f;

@@ -21,6 +21,20 @@ __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict_
     if (id < 0 || id >= vocab) id = 0;
     const W* row = table + (size_t)id * hidden;
     float* dst = out + (size_t)t * hidden;
+    constexpr int VEC = 16 / sizeof(W);  // elements of one 16-byte read
+    if (hidden % VEC == 0) {
+        struct alignas(16) Pack {
+            W v[VEC];
+        };
+        for (int i = threadIdx.x * VEC; i < hidden; i += blockDim.x * VEC) {
+            const Pack p = *reinterpret_cast<const Pack*>(row + i);
+#pragma unroll
+            for (int j = 0; j < VEC; j += 4)
+                *reinterpret_cast<float4*>(dst + i + j) = make_float4(
+                    to_float(p.v[j]), to_float(p.v[j + 1]), to_float(p.v[j + 2]), to_float(p.v[j + 3]));
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]);
 }
 

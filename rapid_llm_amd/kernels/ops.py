@@ -478,7 +478,7 @@ class AttentionPlan:
         if fixed is not None:
             # a step of single tokens whose index list is already on the device (graphs)
             self.num_decode = fixed.numel()
-            self.seq_token = fixed
+            self.seq_token = None  # request i is token i: the kernels skip the lookup
             self.max_decode_ctx = max(ctx.h_seq_starts) + 1
             self.num_tiles = 0
             self.tile_info = None
