@@ -83,6 +83,44 @@ def prefill_flops(cfg, tokens: int) -> float:
     return linear + attn
 
 
+def measured_peaks() -> int:
+    """Practical peaks of this device, beside the published ones the fractions are quoted
+    against: a 4 GiB read by a plain streaming kernel, a 2 GiB library copy, and the library's square
+    products of 8,192."""
+    import torch
+
+    def timed(fn, n=10) -> float:
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / n
+
+    from rapid_llm_amd.kernels import ops
+
+    out = {}
+    x = torch.ones(1 << 31, dtype=torch.bfloat16, device="cuda")  # 4 GiB
+    out["read_gbps"] = round(
+        max(x.numel() * 2 / timed(lambda: ops.read_buffer(x, blocks)) for blocks in (1024, 2048, 4096, 8192, 32768)) / 1e9, 1
+    )
+    half = x[: 1 << 30]
+    y = torch.empty_like(half)
+    out["copy_gbps_read_plus_write"] = round(2 * half.numel() * 2 / timed(lambda: y.copy_(half)) / 1e9, 1)
+    del x, y, half
+    n = 8192
+    for name, dtype in (("bf16", torch.bfloat16), ("fp32", torch.float32)):
+        a = torch.randn(n, n, device="cuda", dtype=dtype)
+        b = torch.randn(n, n, device="cuda", dtype=dtype)
+        torch.backends.cuda.matmul.allow_tf32 = False
+        out[f"gemm_{name}_tflops"] = round(2 * n**3 / timed(lambda: torch.matmul(a, b.t())) / 1e12, 1)
+    out["published"] = {"hbm_gbps": HBM_GBPS, "bf16_tflops": PEAK_TFLOPS["bfloat16"], "fp32_tflops": PEAK_TFLOPS["float32"]}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -96,7 +134,11 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-pipeline", action="store_true", help="read every step's tokens before queueing the next")
+    ap.add_argument("--peaks", action="store_true",
+                    help="measure what the device reaches with library kernels (a large read, copy and square products) and exit")
     args = ap.parse_args()
+    if args.peaks:
+        return measured_peaks()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2

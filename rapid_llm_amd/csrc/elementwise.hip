@@ -653,3 +653,32 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
     }
     return rl_launch_status();
 }
+
+// --------------------------------------------------------------------------- //
+// A plain read of a buffer, for measuring what the memory system delivers: every thread
+// keeps eight 16-byte loads in flight; nothing is written unless the data match a pattern
+// that never occurs (so that the loads cannot be dropped).
+// --------------------------------------------------------------------------- //
+__global__ __launch_bounds__(256) void read_kernel(const uint4* __restrict__ src, size_t n16,
+                                                   unsigned* __restrict__ sink) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    unsigned acc = 0;
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = src[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < n16; i += stride) acc += src[i].x;
+    if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
+extern "C" int rl_read_buffer(const void* src, size_t bytes, unsigned* sink, int blocks,
+                              hipStream_t stream) {
+    if (bytes < 16 || blocks < 1 || (reinterpret_cast<uintptr_t>(src) & 15)) return RL_ERR_ARG;
+    hipLaunchKernelGGL(read_kernel, dim3(blocks), dim3(256), 0, stream, (const uint4*)src,
+                       bytes / 16, sink);
+    return rl_launch_status();
+}

@@ -106,6 +106,17 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, fed: Option
     )
 
 
+def read_buffer(buf: torch.Tensor, blocks: int = 4096) -> None:
+    """Stream a buffer through the compute units once (a measurement of read bandwidth)."""
+    if not buf.is_cuda or not buf.is_contiguous():
+        raise KernelError("read_buffer takes a contiguous GPU tensor")
+    sink = torch.zeros(1, dtype=torch.int32, device=buf.device)
+    _ok(
+        core().rl_read_buffer(_p(buf), ctypes.c_size_t(buf.numel() * buf.element_size()), _p(sink), blocks, _stream()),
+        "rl_read_buffer",
+    )
+
+
 def add_rmsnorm(
     residual: torch.Tensor,
     delta: Optional[torch.Tensor],
