@@ -14,6 +14,18 @@
 // packed [gate | up] matrix and the epilogue writes silu(gate) * up
 // (rapid_llm/kernels/ops/activation/swiglu.py:91-121), so the [M, 2I] intermediate never
 // exists.
+//
+// Two optional epilogues fold the residual norm between two products into the products
+// themselves, so that a decode step needs no norm kernel (rapid_llm/kernels/ops/layernorm/
+// skip_rmsnorm.py:51-85 is what they compute together):
+//   * "residual": the producer adds its result (rounded to bfloat16, as a stored result
+//     would be) to the float32 residual rows in place, writes the rows times the norm's
+//     weight as bfloat16, and leaves the sum of squares of its 16 columns of every row in
+//     `partial[workgroup][row]`;
+//   * "scaled input": the consumer reads those rows as its X and multiplies its own result
+//     by  rsqrt(sum of the partials / width + eps)  of the row: the norm's factor is a
+//     scalar per row and commutes with the product.
+// Sums run in a fixed order (the workgroups' partials in index order).
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -62,11 +74,24 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
 // split over workgroups and staggered K offsets did not help.
 #define WT_PITCH 272  // bytes between the 16 rows of the LDS tile: 256 + 16, conflict-free reads
 
+struct SkinnyExtra {
+    // scaled input (null: X is used as it is)
+    const float* x_partial;  // [x_parts][16] sums of squares
+    int x_parts;
+    float x_inv_size, x_eps;
+    // residual epilogue (null: the result is stored)
+    float* residual;      // [M, N] float32, updated in place
+    const float* norm_w;  // [N]
+    bf16_t* xt;           // [M, N] residual * norm_w
+    float* partial;       // [workgroups][16]
+};
+
 template <int NT, typename OutT, bool SWIGLU>
 __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, OutT* __restrict__ out, int M,
-    int N, int K, int ldx, int ldw, int ldo) {
+    int N, int K, int ldx, int ldw, int ldo, SkinnyExtra ex) {
     __shared__ float red[GW][NT * 256];
+
     __shared__ __attribute__((aligned(16))) unsigned char wtile[GW][16 * WT_PITCH];
 
     const int lane = threadIdx.x & (RL_WAVE - 1);
@@ -120,6 +145,23 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
+    // What the residual epilogue needs from memory is asked for now and arrives while the
+    // weights stream: the residual and norm weights of the results this thread will write.
+    // (Asking for a scaled input's partial sums this early was measured and lost 1.5 us a
+    // product: loads return in order, and the weights then wait behind them.)
+    static_assert(NT * 64 <= GW * RL_WAVE, "every result of the workgroup has a thread of its own");
+    float res_in[4] = {0.f, 0.f, 0.f, 0.f}, nw_in[4] = {0.f, 0.f, 0.f, 0.f};
+    if (!SWIGLU && ex.residual && threadIdx.x < NT * 64) {
+        const int ln = threadIdx.x & 63, ot = threadIdx.x >> 6, m = ln & 15;
+        const int nbase = (blockIdx.x * NT + ot) * 16 + 4 * (ln >> 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (m < M && nbase + i < N) {
+                res_in[i] = ex.residual[(size_t)m * N + nbase + i];
+                nw_in[i] = ex.norm_w[nbase + i];
+            }
+    }
+
     // whole chunks of 128: no predicates.  The bound is the same for every lane of a wave.
     const int kfull = K & ~(KSTEP - 1);
     for (int kw = wave * KSTEP; kw < kfull; kw += GW * KSTEP) {
@@ -161,63 +203,109 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
         }
     }
 
+    // the norm's factor of every row of a scaled input: thread (run j, row m) adds the
+    // partials j, j + 32, .. in order, then every row's 32 runs are added in order
+    // (the epilogues' small arrays live where the weight tiles were: an occupancy of three
+    // workgroups per compute unit hangs on a few hundred bytes of LDS)
+    float(*row_part)[16] = reinterpret_cast<float(*)[16]>(&wtile[0][0]);  // [32][16]
+    float* row_scale = reinterpret_cast<float*>(&wtile[0][0]) + 32 * 16;   // [16]
+    float* sq = row_scale + 16;                                            // [NT * 64]
+    static_assert(sizeof(wtile) >= (32 * 16 + 16 + NT * 64) * sizeof(float), "epilogue arrays fit");
+    if (ex.x_partial) {
+        const int m = threadIdx.x & 15, j = threadIdx.x >> 4;  // 512 threads: 32 runs
+        float run = 0.f;
+        for (int p = j; p < ex.x_parts; p += 32) run += ex.x_partial[p * 16 + m];
+        __syncthreads();  // every wave has left the main loop: the weight tiles are free
+        row_part[j][m] = run;
+    }
     // partial tiles of the waves -> LDS; lane-major so that reads below are conflict-free
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) red[wave][(nt * 4 + i) * 64 + lane] = acc[nt][i];
     __syncthreads();
+    if (ex.x_partial) {
+        if (threadIdx.x < 16) {
+            float ss = 0.f;
+            for (int j = 0; j < 32; ++j) ss += row_part[j][threadIdx.x];
+            row_scale[threadIdx.x] = rsqrtf(ss * ex.x_inv_size + ex.x_eps);
+        }
+        __syncthreads();
+    }
 
     // thread -> (tile pair / tile, lane of the tile); sums the waves in order
     constexpr int OUT_TILES = SWIGLU ? NT / 2 : NT;
-    for (int e = threadIdx.x; e < OUT_TILES * 64; e += GW * RL_WAVE) {
+    for (int e = threadIdx.x; e < OUT_TILES * 64; e += GW * RL_WAVE) {  // at most one round
         const int ln = e & 63;
         const int ot = e >> 6;
         const int m = ln & 15;
         const int nbase = (blockIdx.x * OUT_TILES + ot) * 16 + 4 * (ln >> 4);
-        if (m >= M) continue;
+        const float scale = ex.x_partial ? row_scale[m] : 1.f;
+        float sumsq = 0.f;
+        if (m < M) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int n = nbase + i;
-            if (n >= N) continue;
-            float v;
-            if (SWIGLU) {
-                float gate = 0.f, up = 0.f;
+            for (int i = 0; i < 4; ++i) {
+                const int n = nbase + i;
+                if (n >= N) continue;
+                float v;
+                if (SWIGLU) {
+                    float gate = 0.f, up = 0.f;
 #pragma unroll
-                for (int w = 0; w < GW; ++w) {
-                    gate += red[w][((2 * ot) * 4 + i) * 64 + ln];
-                    up += red[w][((2 * ot + 1) * 4 + i) * 64 + ln];
+                    for (int w = 0; w < GW; ++w) {
+                        gate += red[w][((2 * ot) * 4 + i) * 64 + ln];
+                        up += red[w][((2 * ot + 1) * 4 + i) * 64 + ln];
+                    }
+                    // the activation reads its operands rounded to bfloat16, as the unfused
+                    // path does where the product's result is stored before the activation
+                    gate = bf16_to_float(float_to_bf16(gate * scale));
+                    up = bf16_to_float(float_to_bf16(up * scale));
+                    v = gate / (1.f + expf(-gate)) * up;
+                } else {
+                    v = 0.f;
+#pragma unroll
+                    for (int w = 0; w < GW; ++w) v += red[w][(ot * 4 + i) * 64 + ln];
+                    v *= scale;
                 }
-                // the activation reads its operands rounded to bfloat16, as the unfused
-                // path does where the product's result is stored before the activation
-                gate = bf16_to_float(float_to_bf16(gate));
-                up = bf16_to_float(float_to_bf16(up));
-                v = gate / (1.f + expf(-gate)) * up;
-            } else {
-                v = 0.f;
-#pragma unroll
-                for (int w = 0; w < GW; ++w) v += red[w][(ot * 4 + i) * 64 + ln];
+                if (!SWIGLU && ex.residual) {
+                    const size_t at = (size_t)m * N + n;
+                    const float r = res_in[i] + bf16_to_float(float_to_bf16(v));
+                    ex.residual[at] = r;
+                    ex.xt[at] = float_to_bf16(r * nw_in[i]);
+                    sumsq += r * r;
+                } else {
+                    store_out<OutT>(out + (size_t)m * ldo + n, v);
+                }
             }
-            store_out<OutT>(out + (size_t)m * ldo + n, v);
+        }
+        if (!SWIGLU && ex.residual) sq[e] = sumsq;
+    }
+    if (!SWIGLU && ex.residual) {
+        __syncthreads();
+        // row m of this workgroup's columns: the epilogue threads with lane % 16 == m, in order
+        if (threadIdx.x < 16) {
+            float ss = 0.f;
+            for (int e = threadIdx.x; e < OUT_TILES * 64; e += 16) ss += sq[e];
+            ex.partial[(size_t)blockIdx.x * 16 + threadIdx.x] = ss;
         }
     }
 }
 
 template <int NT, typename OutT, bool SWIGLU>
 static int launch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
-                  int ldw, int ldo, hipStream_t stream) {
+                  int ldw, int ldo, const SkinnyExtra& ex, hipStream_t stream) {
     constexpr int rows_per_block = (SWIGLU ? NT / 2 : NT) * 16;
     dim3 grid((N + rows_per_block - 1) / rows_per_block), block(GW * RL_WAVE);
     hipLaunchKernelGGL((gemm_skinny_kernel<NT, OutT, SWIGLU>), grid, block, 0, stream, X, W, out,
-                       M, N, K, ldx, ldw, ldo);
+                       M, N, K, ldx, ldw, ldo, ex);
     return rl_launch_status();
 }
 
 template <typename OutT, bool SWIGLU>
 static int dispatch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
-                    int ldw, int ldo, int nt, hipStream_t stream) {
+                    int ldw, int ldo, int nt, const SkinnyExtra& ex, hipStream_t stream) {
 #define RL_CASE(NTV)                                                                           \
-    if (nt == NTV) return launch<NTV, OutT, SWIGLU>(X, W, out, M, N, K, ldx, ldw, ldo, stream);
+    if (nt == NTV)                                                                             \
+        return launch<NTV, OutT, SWIGLU>(X, W, out, M, N, K, ldx, ldw, ldo, ex, stream);
     if (SWIGLU) {
         RL_CASE(2) RL_CASE(4)
     } else {
@@ -227,28 +315,70 @@ static int dispatch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, i
     return RL_ERR_ARG;
 }
 
+static bool skinny_args_ok(int M, int K, int ldx, int ldw) {
+    return M <= 16 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K;
+}
+
+// x_partial (optional): X holds rows whose norm factor is still to be applied,
+// rsqrt(sum over x_parts of x_partial[part][row] / x_size + x_eps); the result is multiplied
+// by it.
+static SkinnyExtra scaled_input(const float* x_partial, int x_parts, int x_size, float x_eps) {
+    SkinnyExtra ex = {};
+    if (x_partial) {
+        ex.x_partial = x_partial;
+        ex.x_parts = x_parts;
+        ex.x_inv_size = 1.f / (float)x_size;
+        ex.x_eps = x_eps;
+    }
+    return ex;
+}
+
 // out_type: RL_F32 or RL_BF16.  nt: weight-row tiles per workgroup (see the host wrapper).
 extern "C" int rl_gemm_skinny(const void* X, const void* W, void* out, int M, int N, int K,
                               int ldx, int ldw, int ldo, int out_type, int nt,
+                              const float* x_partial, int x_parts, int x_size, float x_eps,
                               hipStream_t stream) {
     if (M <= 0 || N <= 0) return RL_OK;
-    if (M > 16 || K < 8 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < N)
+    if (!skinny_args_ok(M, K, ldx, ldw) || ldo < N || (x_partial && (x_parts < 1 || x_size < 1)))
         return RL_ERR_ARG;
+    const SkinnyExtra ex = scaled_input(x_partial, x_parts, x_size, x_eps);
     if (out_type == RL_F32)
         return dispatch<float, false>((const bf16_t*)X, (const bf16_t*)W, (float*)out, M, N, K,
-                                      ldx, ldw, ldo, nt, stream);
+                                      ldx, ldw, ldo, nt, ex, stream);
     if (out_type == RL_BF16)
         return dispatch<bf16_t, false>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, N, K,
-                                       ldx, ldw, ldo, nt, stream);
+                                       ldx, ldw, ldo, nt, ex, stream);
     return RL_ERR_ARG;
 }
 
 // out[M, I] = silu(X Wg^T) * (X Wu^T) with W = [Wg | Wu] stacked by rows, [2I, K].
 extern "C" int rl_gemm_skinny_swiglu(const void* X, const void* W, void* out, int M, int I, int K,
-                                     int ldx, int ldw, int ldo, int nt, hipStream_t stream) {
+                                     int ldx, int ldw, int ldo, int nt, const float* x_partial,
+                                     int x_parts, int x_size, float x_eps, hipStream_t stream) {
     if (M <= 0 || I <= 0) return RL_OK;
-    if (M > 16 || K < 8 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo < I)
+    if (!skinny_args_ok(M, K, ldx, ldw) || ldo < I || (x_partial && (x_parts < 1 || x_size < 1)))
         return RL_ERR_ARG;
     return dispatch<bf16_t, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx,
-                                  ldw, ldo, nt, stream);
+                                  ldw, ldo, nt, scaled_input(x_partial, x_parts, x_size, x_eps),
+                                  stream);
+}
+
+// The product with the residual epilogue: residual[M, N] += X W^T (rounded to bfloat16),
+// xt[M, N] = residual * norm_w as bfloat16, partial[workgroup][16] = sums of squares of the
+// workgroup's columns per row.  Returns the number of workgroups through *parts (the caller
+// sizes `partial` with rl_gemm_skinny_parts).
+extern "C" int rl_gemm_skinny_parts(int N, int nt) { return (N + nt * 16 - 1) / (nt * 16); }
+
+extern "C" int rl_gemm_skinny_residual(const void* X, const void* W, int M, int N, int K, int ldx,
+                                       int ldw, int nt, float* residual, const float* norm_w,
+                                       void* xt, float* partial, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return RL_OK;
+    if (!skinny_args_ok(M, K, ldx, ldw) || !residual || !norm_w || !xt || !partial) return RL_ERR_ARG;
+    SkinnyExtra ex = {};
+    ex.residual = residual;
+    ex.norm_w = norm_w;
+    ex.xt = (bf16_t*)xt;
+    ex.partial = partial;
+    return dispatch<bf16_t, false>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K,
+                                   ldx, ldw, N, nt, ex, stream);
 }

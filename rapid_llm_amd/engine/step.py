@@ -79,6 +79,9 @@ class StepContext:
     max_position: int = 0
     max_seq_tokens: int = 0  # longest portion in the batch
     fed_tokens: torch.Tensor | None = None  # [rows] what the latest sampling chose (see fed_token)
+    # a step of few rows in bfloat16: parts may hand their last product on unfinished, so that
+    # the norm that follows is folded into the products around it (parts/lazy.py)
+    defer_products: bool = False
     extra: dict[str, Any] = field(default_factory=dict)  # per-step device metadata of kernels
 
 
@@ -298,6 +301,7 @@ class ModelRunner:
             logit_rows=part[7],
             block_tables=self.device_cache.tables,
             fed_tokens=self.sampled,
+            defer_products=self.dtype == torch.bfloat16 and meta["num_tokens"] <= ops.SKINNY_MAX_ROWS,
             **meta,
         )
 

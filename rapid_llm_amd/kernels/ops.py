@@ -433,8 +433,23 @@ def _skinny_tiles(rows: int, out_features: int) -> int:
     return 2 if rows > 4 and -(-out_features // 32) >= _MIN_BLOCKS else 1
 
 
-def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """``x[M,K] @ w[N,K]^T`` with bfloat16 operands and float32 accumulation.
+def _scaled_args(scaled, rows: int, k: int) -> tuple:
+    """The kernels' arguments for an X whose norm factor is still to be applied."""
+    if scaled is None:
+        return (None, 0, 0, ctypes.c_float(0.0))
+    _need(scaled.partial, "partial sums of squares", torch.float32)
+    if scaled.partial.dim() != 2 or scaled.partial.shape[1] != 16 or scaled.size != k or rows > 16:
+        raise KernelError(
+            f"scaled rows of width {scaled.size} with partials {tuple(scaled.partial.shape)} do not fit "
+            f"a product of {rows} rows over {k}"
+        )
+    return (_p(scaled.partial), scaled.partial.shape[0], scaled.size, ctypes.c_float(scaled.eps))
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, scaled=None) -> torch.Tensor:
+    """``x[M,K] @ w[N,K]^T`` with bfloat16 operands and float32 accumulation.  ``scaled``
+    (few rows only): the rows of ``x`` still lack their norm's factor, which is applied to
+    the result (see ``gemm_bf16_residual``).
 
     Up to 16 rows (decode) run the hand-written bandwidth-bound kernel, which can write
     float32 directly.  More rows go to the library product, as the reference's dense products do
@@ -451,16 +466,50 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
         nt = _skinny_tiles(m, n)
         _ok(
-            core().rl_gemm_skinny(_p(x), _p(w), _p(out), m, n, k, k, k, n, _tag(out_dtype), nt, _stream()),
+            core().rl_gemm_skinny(
+                _p(x), _p(w), _p(out), m, n, k, k, k, n, _tag(out_dtype), nt, *_scaled_args(scaled, m, k), _stream()
+            ),
             "rl_gemm_skinny",
         )
         return out
+    if scaled is not None:
+        raise KernelError(f"scaled rows need the few-row product: {m} rows over {k}")
     return torch.matmul(x, w.t())
 
 
-def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor | None:
+def gemm_bf16_residual(
+    x: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """The few-row product with the residual epilogue: ``residual += x w^T`` (the product
+    rounded to bfloat16 first, as a stored result would be) in place; returns
+    ``(residual * norm_weight`` as bfloat16, ``partial [workgroups, 16]`` float32``)`` with the
+    sums of squares of each workgroup's columns of every row.  A consumer that takes the rows
+    as ``scaled`` input finishes the norm."""
+    _need(x, "x", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    m, k = x.shape
+    n = w.shape[0]
+    if k != w.shape[1] or m > SKINNY_MAX_ROWS or k % 8:
+        raise KernelError(f"gemm_bf16_residual takes up to {SKINNY_MAX_ROWS} rows over a multiple of 8: x {tuple(x.shape)}, w {tuple(w.shape)}")
+    _need(residual, "residual", torch.float32, (m, n))
+    _need(norm_weight, "norm weight", torch.float32, (n,))
+    lib = core()
+    nt = _skinny_tiles(m, n)
+    rows = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    partial = torch.empty((lib.rl_gemm_skinny_parts(n, nt), 16), dtype=torch.float32, device=x.device)
+    _ok(
+        lib.rl_gemm_skinny_residual(
+            _p(x), _p(w), m, n, k, k, k, nt, _p(residual), _p(norm_weight), _p(rows), _p(partial), _stream()
+        ),
+        "rl_gemm_skinny_residual",
+    )
+    return rows, partial
+
+
+def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> torch.Tensor | None:
     """``silu(x Wg^T) * (x Wu^T)`` for the packed ``[gate | up]`` matrix in one kernel, for
-    few rows; ``None`` when the shape is not one the fused kernel takes."""
+    few rows; ``None`` when the shape is not one the fused kernel takes.  ``scaled``: as in
+    ``gemm_bf16``."""
     m, k = x.shape
     two_i = w_gate_up.shape[0]
     if m > SKINNY_MAX_ROWS or k % 8 or two_i % 2 or x.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16:
@@ -471,7 +520,9 @@ def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor |
     out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
     nt = _skinny_tiles(m, inter) * 2  # pairs of (gate, up) tiles
     _ok(
-        core().rl_gemm_skinny_swiglu(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, _stream()),
+        core().rl_gemm_skinny_swiglu(
+            _p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, *_scaled_args(scaled, m, k), _stream()
+        ),
         "rl_gemm_skinny_swiglu",
     )
     return out

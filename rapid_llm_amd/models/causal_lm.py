@@ -20,6 +20,7 @@ from ..parts.base import (
     ParamSpec,
 )
 from ..parts.embedding import OutputProjection, TokenEmbedding
+from ..parts.lazy import plain, run_norm
 from .spec import ModelSpec
 
 
@@ -120,10 +121,13 @@ class CausalLM:
         residual = self.embed.forward(ctx.token_ids, ctx.fed_tokens)
         delta = None
         for place, li in enumerate(self.order):
-            delta = self.blocks[li].forward(residual, delta, ctx, caches[place])
+            block = self.blocks[li]
+            if not getattr(block, "accepts_deferred", False):
+                delta = plain(delta)
+            delta = block.forward(residual, delta, ctx, caches[place])
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=residual.device)
-        h = self.final_norm.forward(residual, delta, ctx, rows=ctx.logit_rows)
+        h = run_norm(self.final_norm, residual, delta, ctx, rows=ctx.logit_rows)
         return self.output.forward(h)
 
 

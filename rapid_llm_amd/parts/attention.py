@@ -93,6 +93,10 @@ class GQAAttention(Mixer):
         return CacheNeed("kv", window=self.window, num_kv_heads=self.nkv, head_dim=self.d)
 
     # ---- step ------------------------------------------------------------------
+    @property
+    def accepts_scaled_rows(self) -> bool:
+        return self.qkv.weight.dtype == torch.bfloat16
+
     def forward(self, x, ctx, cache):
         tokens = x.shape[0]
         qkv = self.qkv(x)
@@ -109,7 +113,7 @@ class GQAAttention(Mixer):
                 qkv, cache.k, cache.v, out, ctx, table, cache.page_size, self.nq, self.nkv, self.d,
                 self.window, self.scale, self.q_norm_w, self.k_norm_w, cos, sin, eps, cache.owns_pages,
             )
-            return self.o(out)
+            return self.o.deferred(out, ctx)
         q = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         ops.qknorm_rope_kvwrite(
             qkv, q,
@@ -123,7 +127,7 @@ class GQAAttention(Mixer):
             q, cache.k, cache.v, out, ctx, table, cache.page_size,
             self.nq, self.nkv, self.d, self.window, self.scale,
         )
-        return self.o(out)
+        return self.o.deferred(out, ctx)
 
 
 MIXERS.register("gqa_attention", GQAAttention)

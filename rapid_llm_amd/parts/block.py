@@ -8,9 +8,12 @@ next norm kernel, as the reference threads ``(hidden, residual)`` through its la
 from __future__ import annotations
 
 from .base import BLOCKS, Block
+from .lazy import run_norm
 
 
 class PreNormBlock(Block):
+    accepts_deferred = True  # the incoming delta may be a DeferredProduct
+
     def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm) -> None:
         self.mixer = mixer
         self.feed_forward = feed_forward
@@ -21,9 +24,9 @@ class PreNormBlock(Block):
         return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
 
     def forward(self, residual, delta, ctx, cache):
-        x = self.mixer_norm.forward(residual, delta, ctx)
+        x = run_norm(self.mixer_norm, residual, delta, ctx, consumer=self.mixer)
         a = self.mixer.forward(x, ctx, cache)
-        x = self.feed_forward_norm.forward(residual, a, ctx)
+        x = run_norm(self.feed_forward_norm, residual, a, ctx, consumer=self.feed_forward)
         return self.feed_forward.forward(x, ctx)
 
 

@@ -15,6 +15,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from .lazy import DeferredProduct, ScaledRows
 
 
 class Linear:
@@ -30,8 +31,32 @@ class Linear:
             )
         self.weight = weight
 
-    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    # ---- folding a neighbouring norm into the product (decode steps, bfloat16) ----------
+    def skinny(self, x) -> bool:
+        """Whether ``x`` runs through the hand-written few-row kernel, which has the epilogues."""
+        return (
+            self.weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+            and x.shape[0] <= ops.SKINNY_MAX_ROWS and self.in_features % 8 == 0
+        )
+
+    def deferred(self, x: torch.Tensor, ctx):
+        """The product, or a :class:`DeferredProduct` of it where the step allows it."""
+        if getattr(ctx, "defer_products", False) and isinstance(x, torch.Tensor) and self.skinny(x):
+            return DeferredProduct(self, x)
+        return self(x)
+
+    def add_to_residual(self, x: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> ScaledRows:
+        """``residual += x W^T`` in place; returns the new rows times ``norm_weight`` and the
+        pieces of their sums of squares."""
+        rows, partial = ops.gemm_bf16_residual(x, self.weight, residual, norm_weight)
+        return ScaledRows(rows, partial, self.out_features, eps)
+
+    def __call__(self, x, out_dtype: torch.dtype | None = None) -> torch.Tensor:
         w = self.weight
+        if isinstance(x, ScaledRows):
+            if not self.skinny(x):
+                raise ValueError("scaled rows reached a product that cannot apply their factor")
+            return ops.gemm_bf16(x.rows, w, out_dtype or x.dtype, scaled=x)
         rows = x.shape[0]
         out_dtype = out_dtype or x.dtype
         if w.dtype == torch.float32:

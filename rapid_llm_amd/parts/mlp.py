@@ -11,6 +11,7 @@ import torch
 
 from ..kernels import ops
 from .base import FEED_FORWARDS, FeedForward, ParamSpec, Source
+from .lazy import ScaledRows
 from .linear import Linear
 
 
@@ -45,12 +46,17 @@ class SwiGLU(FeedForward):
         self.gate_up.bind(params[self.name + ".gate_up"])
         self.down.bind(params[self.name + ".down"])
 
+    @property
+    def accepts_scaled_rows(self) -> bool:
+        return self.gate_up.weight.dtype == torch.bfloat16
+
     def forward(self, x, ctx):
         w = self.gate_up.weight
         if w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
-            act = ops.gemm_bf16_swiglu(x, w)  # few rows: product and activation in one kernel
+            # few rows: product and activation in one kernel
+            act = ops.gemm_bf16_swiglu(x.rows, w, scaled=x) if isinstance(x, ScaledRows) else ops.gemm_bf16_swiglu(x, w)
             if act is not None:
-                return self.down(act)
+                return self.down.deferred(act, ctx)
         gu = self.gate_up(x)
         act = torch.empty((x.shape[0], self.intermediate_size), dtype=gu.dtype, device=x.device)
         ops.swiglu(gu, act)

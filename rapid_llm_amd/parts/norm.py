@@ -12,9 +12,12 @@ import torch
 
 from ..kernels import ops
 from .base import NORMS, Norm, ParamSpec, Source
+from .lazy import DeferredProduct
 
 
 class RMSNorm(Norm):
+    fuses_products = True  # takes a DeferredProduct as delta, may return ScaledRows
+
     def __init__(self, size: int, eps: float, checkpoint_name: str, name: str = "norm") -> None:
         self.size = size
         self.eps = float(eps)
@@ -37,7 +40,16 @@ class RMSNorm(Norm):
         self.weight = params[self.name + ".weight"]
         self.dtype = runtime.dtype
 
-    def forward(self, residual, delta, ctx, rows=None):
+    def forward(self, residual, delta, ctx, rows=None, scaled_ok=False):
+        if isinstance(delta, DeferredProduct):
+            if (
+                scaled_ok and rows is None and delta.linear.out_features == self.size
+                and self.dtype == torch.bfloat16 and delta.linear.skinny(delta.x)
+            ):
+                # the producer's kernel adds into the residual and leaves what the consumer's
+                # kernel needs to finish the norm: no kernel of this norm's own runs
+                return delta.linear.add_to_residual(delta.x, residual, self.weight, self.eps)
+            delta = delta.materialize()
         n = residual.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=self.dtype, device=residual.device)
         ops.add_rmsnorm(residual, delta, self.weight, out, self.eps, rows)

@@ -349,6 +349,53 @@ def test_gemm_bf16_swiglu_fused(shape):
     assert ops.gemm_bf16_swiglu(torch.zeros(33, k, dtype=torch.bfloat16, device=DEV), w.to(DEV)) is None
 
 
+@pytest.mark.parametrize("shape", [(1, 96, 64), (8, 4096, 4096), (16, 304, 1000), (5, 4096, 12288), (3, 40, 48)])
+def test_products_fold_the_norm_between_them(shape):
+    """producer: residual += x W^T, rows * weight, pieces of the sums of squares; consumer:
+    takes those rows and scales its own result.  Together they are the product, the residual
+    add, the norm and the next product (and the fused activation) of the unfused path."""
+    from rapid_llm_amd.parts.lazy import ScaledRows
+
+    ops = _ops()
+    m, hidden, k = shape
+    torch.manual_seed(m + hidden)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(hidden, k) / math.sqrt(k)).bfloat16()
+    residual = torch.randn(m, hidden)
+    norm_w = 1 + 0.1 * torch.randn(hidden)
+    eps = 3e-6
+    res = residual.clone().to(DEV)
+    rows, partial = ops.gemm_bf16_residual(x.to(DEV), w.to(DEV), res, norm_w.to(DEV))
+    delta = (x.float() @ w.float().T).bfloat16().float()
+    want_res = residual + delta
+    # the product is rounded to bfloat16 before the add; sums in another order may round a
+    # few results one step the other way
+    torch.testing.assert_close(res.cpu() - residual, delta, rtol=2.0 ** -7, atol=1e-5)
+    assert float((res.cpu() - want_res).abs().gt(1e-5).float().mean()) < 0.01
+    torch.testing.assert_close(rows.float().cpu(), (res.cpu() * norm_w).bfloat16().float(), rtol=8e-3, atol=1e-6)
+    ss = partial.sum(0).cpu()[:m]
+    torch.testing.assert_close(ss, (res.cpu() ** 2).sum(-1), rtol=1e-5, atol=1e-5)
+    assert partial.shape[1] == 16 and float(partial[:, m:].abs().max() if m < 16 else 0.0) == 0.0
+    # the consumer: a plain product, and the packed gate/up product with its activation
+    scaled = ScaledRows(rows, partial, hidden, eps)
+    normed = plain_rmsnorm(res.cpu(), norm_w, eps)
+    n2 = 208
+    w2 = (torch.randn(n2, hidden) / math.sqrt(hidden)).bfloat16()
+    for out_dtype, tol in ((torch.bfloat16, 2e-2), (torch.float32, 1e-2)):
+        got = ops.gemm_bf16(rows, w2.to(DEV), out_dtype, scaled=scaled)
+        want = normed.bfloat16().float() @ w2.float().T
+        torch.testing.assert_close(got.float().cpu(), want, rtol=tol, atol=tol)
+    wgu = (torch.randn(2 * n2, hidden) / math.sqrt(hidden)).bfloat16()
+    act = ops.gemm_bf16_swiglu(rows, wgu.to(DEV), scaled=scaled)
+    gu = (normed.bfloat16().float() @ wgu.float().T).bfloat16().float()
+    want = torch.nn.functional.silu(gu[:, :n2]) * gu[:, n2:]
+    torch.testing.assert_close(act.float().cpu(), want, rtol=3e-2, atol=3e-2)
+    # run again: the same bits (fixed orders of summation)
+    res2 = residual.clone().to(DEV)
+    rows2, partial2 = ops.gemm_bf16_residual(x.to(DEV), w.to(DEV), res2, norm_w.to(DEV))
+    assert torch.equal(rows2, rows) and torch.equal(partial2, partial) and torch.equal(res2, res)
+
+
 def test_embed_takes_fed_tokens_from_the_sampling_buffer():
     """An id -(r + 1) reads row r of the buffer the sampling kernels write; other ids are
     the rows they name; an id that names no row of either reads row 0 and never faults."""
