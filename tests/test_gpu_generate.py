@@ -2,7 +2,6 @@
 and sampling kernels; the plain implementation re-runs the whole sequence for every token."""
 
 import pytest
-import torch
 
 from plain_model import plain_forward, plain_load
 from plain_sampler import plain_sample

@@ -3,7 +3,6 @@ a toy mixer with state of its own and a toy architecture, registered, built and 
 without a change to the framework; a run order that names a layer twice; a layer that reads
 another layer's cache."""
 
-import json
 import math
 from dataclasses import dataclass
 

@@ -1,6 +1,5 @@
 """Tiny configurations of the Qwen3 dense decoder that differ in every size and option."""
 
-import json
 import random
 from pathlib import Path
 
