@@ -482,12 +482,15 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
 // One thread per channel; the loads of MERGE_STEP splits are issued together and folded into a
 // running (max, weight, output), in the order of the splits.
 #define MERGE_STEP 8
+// by_token: the partial results lie at the token's place in the step, not at the launch's own
+// count of its rows (the prefill kernel's splits).
 __global__ void attn_merge_kernel(const float* __restrict__ part_o,
                                   const float* __restrict__ part_ml, bf16_t* __restrict__ out,
-                                  const int* __restrict__ seq_token, int nq, int nsplit) {
+                                  const int* __restrict__ seq_token, int nq, int nsplit,
+                                  int by_token) {
     const int seq = blockIdx.x, head = blockIdx.y;
-    const size_t slot0 = ((size_t)seq * nq + head) * nsplit;
     const int t = seq_token ? seq_token[seq] : seq;
+    const size_t slot0 = ((size_t)(by_token ? t : seq) * nq + head) * nsplit;
     const int d = threadIdx.x;
     if (d >= D) return;
     float mm = -INFINITY, wsum = 0.f, o = 0.f;
@@ -575,7 +578,7 @@ extern "C" int rl_attn_decode(const void* q, const void* k_cache, const void* v_
     if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
     if (nsplit > 1) {
         hipLaunchKernelGGL(attn_merge_kernel, dim3(num_seqs, nq), dim3(D < 64 ? 64 : D), 0,
-                           stream, part_o, part_ml, (bf16_t*)out, seq_token, nq, nsplit);
+                           stream, part_o, part_ml, (bf16_t*)out, seq_token, nq, nsplit, 0);
     }
     return rl_launch_status();
 }
@@ -614,12 +617,18 @@ attn_prefill_kernel(
     const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out,
     const int* __restrict__ tile_info, const int* __restrict__ work_order,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int window, float scale_log2) {
+    int page_size, int nq, int nkv, int window, float scale_log2, int nsplit,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
     __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_KEYS * K_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Vs[D * V_LD];
 
     const int G = nq / nkv;
-    const int item = work_order ? work_order[blockIdx.x] : blockIdx.x;
+    // nsplit > 1: the keys of every tile are cut into nsplit runs of whole 64-key steps, one
+    // workgroup each; the runs' results go to part_o / part_ml (indexed by the token's place in
+    // the step) and are folded by the merge kernel, as the decode kernel's splits are
+    const int split = blockIdx.x % nsplit;
+    const int wg = blockIdx.x / nsplit;
+    const int item = work_order ? work_order[wg] : wg;
     const int tile = item / nkv;
     const int hk = item % nkv;
     const int tok0 = tile_info[4 * tile + 0];
@@ -752,13 +761,20 @@ attn_prefill_kernel(
         }
     };
 
-    const int first_base = tile_kstart & ~(PF_KEYS - 1);
-    if (first_base < tile_kend) stage_load(first_base);
-    for (int base = first_base; base < tile_kend; base += PF_KEYS) {
+    int first_base = tile_kstart & ~(PF_KEYS - 1);
+    int run_end = tile_kend;
+    if (nsplit > 1) {
+        const int steps = (tile_kend - first_base + PF_KEYS - 1) / PF_KEYS;
+        const int per = (steps + nsplit - 1) / nsplit;
+        run_end = min(tile_kend, first_base + (split + 1) * per * PF_KEYS);
+        first_base += split * per * PF_KEYS;
+    }
+    if (first_base < run_end) stage_load(first_base);
+    for (int base = first_base; base < run_end; base += PF_KEYS) {
         __syncthreads();  // the previous tile has been consumed
         stage_store(base);
         __syncthreads();
-        if (base + PF_KEYS < tile_kend) stage_load(base + PF_KEYS);
+        if (base + PF_KEYS < run_end) stage_load(base + PF_KEYS);
         if (base > wave_max_pos) continue;  // every key of the tile is ahead of this wave's rows
         // masks are needed where the diagonal or a window's edge crosses the tile
         const bool need_mask =
@@ -845,6 +861,22 @@ attn_prefill_kernel(
         const float lt = row_sum4(l[n]);
         const float inv = lt > 0.f ? 1.f / lt : 0.f;
         if (!r_ok[n]) continue;
+        if (nsplit > 1) {
+            const size_t slot = ((size_t)r_tok[n] * nq + r_head[n]) * nsplit + split;
+            if (lt > 0.f) {
+                float* prow = part_o + slot * D;
+#pragma unroll
+                for (int b = 0; b < DB; ++b)
+                    *reinterpret_cast<float4*>(prow + 16 * b + 4 * g) =
+                        make_float4(acc[n][b][0] * inv, acc[n][b][1] * inv, acc[n][b][2] * inv,
+                                    acc[n][b][3] * inv);
+            }
+            if (g == 0) {
+                part_ml[slot * 2] = lt > 0.f ? m[n] : -INFINITY;
+                part_ml[slot * 2 + 1] = lt;
+            }
+            continue;
+        }
         bf16_t* orow = out + ((size_t)r_tok[n] * nq + r_head[n]) * D;
 #pragma unroll
         for (int b = 0; b < DB; ++b) {
@@ -860,19 +892,31 @@ attn_prefill_kernel(
 
 extern "C" int rl_attn_prefill_rows() { return PF_ROWS; }
 
+// nsplit > 1 cuts every tile's keys into that many runs (for launches of few, long tiles);
+// part_o [tokens of the step, nq, nsplit, D] and part_ml [.., 2] then hold the runs' results
+// and prefill_tokens [num_prefill_tokens] names the tokens the merge kernel writes.
 extern "C" int rl_attn_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                                const int* tile_info, const int* work_order, int num_tiles,
                                const int* token_slot,
                                const int* block_table, int table_stride, int page_size, int nq,
-                               int nkv, int window, float scale, hipStream_t stream) {
+                               int nkv, int window, float scale, int nsplit, float* part_o,
+                               float* part_ml, const int* prefill_tokens, int num_prefill_tokens,
+                               hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
-    if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535) return RL_ERR_ARG;
+    if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || nsplit < 1)
+        return RL_ERR_ARG;
+    if (nsplit > 1 && (!part_o || !part_ml || !prefill_tokens || num_prefill_tokens < 1 || nq > 65535))
+        return RL_ERR_ARG;
     const float scale_log2 = scale * 1.4426950408889634f;
-    if ((long)num_tiles * nkv > 0x7fffffffL) return RL_ERR_ARG;
-    dim3 grid(num_tiles * nkv), block(PF_WAVES * RL_WAVE);
+    if ((long)num_tiles * nkv * nsplit > 0x7fffffffL) return RL_ERR_ARG;
+    dim3 grid(num_tiles * nkv * nsplit), block(PF_WAVES * RL_WAVE);
     hipLaunchKernelGGL(attn_prefill_kernel, grid, block, 0, stream, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_info,
                        work_order, token_slot, block_table, table_stride, page_size, nq, nkv, window,
-                       scale_log2);
+                       scale_log2, nsplit, part_o, part_ml);
+    if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
+    if (nsplit > 1)
+        hipLaunchKernelGGL(attn_merge_kernel, dim3(num_prefill_tokens, nq), dim3(D < 64 ? 64 : D), 0,
+                           stream, part_o, part_ml, (bf16_t*)out, prefill_tokens, nq, nsplit, 1);
     return rl_launch_status();
 }

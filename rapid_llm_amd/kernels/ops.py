@@ -533,7 +533,8 @@ class AttentionPlan:
     (query heads per kv head): which requests are single tokens (decode kernel) and how the
     portions of the others are cut into row tiles (prefill kernel)."""
 
-    __slots__ = ("num_decode", "seq_token", "max_decode_ctx", "num_tiles", "tile_info", "tile_keys", "orders")
+    __slots__ = ("num_decode", "seq_token", "max_decode_ctx", "num_tiles", "tile_info", "tile_keys", "orders",
+                 "_prefill_tokens", "_prefill_list")
 
     def __init__(self, ctx, group: int, tile_rows: int) -> None:
         fixed = ctx.extra.get("decode_only_tokens")
@@ -546,8 +547,10 @@ class AttentionPlan:
             self.tile_info = None
             self.tile_keys = []
             self.orders = {}
+            self._prefill_list, self._prefill_tokens = [], None
             return
         dec_tokens: list[int] = []
+        self._prefill_list, self._prefill_tokens = [], None
         tile_list: list[tuple[int, int, int, int]] = []
         self.max_decode_ctx = 0
         at = 0
@@ -558,6 +561,7 @@ class AttentionPlan:
             else:
                 for row0 in range(0, n * group, tile_rows):
                     tile_list.append((at, start, n, row0))
+                self._prefill_list.extend(range(at, at + n))
             at += n
         tiles = [v for t in tile_list for v in t]
         # keys each tile reads: what its workgroups cost
@@ -569,6 +573,12 @@ class AttentionPlan:
         packed = upload_ints(dec_tokens + tiles, device)
         self.seq_token = packed[: self.num_decode]
         self.tile_info = packed[self.num_decode :]
+
+    def prefill_tokens(self, device) -> torch.Tensor:
+        """Indices in the step of the tokens that belong to portions (not single tokens)."""
+        if self._prefill_tokens is None:
+            self._prefill_tokens = upload_ints(self._prefill_list, device)
+        return self._prefill_tokens
 
     def work_order(self, nkv: int, device) -> torch.Tensor:
         """Order in which the (tile, kv head) pairs of the prefill kernel are handed out.
@@ -595,6 +605,15 @@ _TARGET_BLOCKS = 256
 _FIRST_ROUND = 256  # workgroups that start first, one on each compute unit
 _MIN_SPLIT_KEYS = 128
 _MAX_SPLIT_PAGES = 1024  # page ids of one split are staged in LDS
+# The prefill kernel cuts its tiles' keys into runs when a launch has fewer workgroups than
+# this and tiles of at least twice that many keys (a portion of one long prompt).
+_PREFILL_SPLIT_BELOW = 512
+_PREFILL_SPLIT_KEYS = 512
+_PREFILL_MAX_SPLITS = 8
+
+
+def tile_rows_of(lib) -> int:
+    return lib.rl_attn_prefill_rows()
 
 
 def _f32_tiles(ctx, group: int) -> tuple[torch.Tensor, int]:
@@ -705,12 +724,27 @@ def paged_attention(
     group = nq // nkv
     plan = attention_plan(ctx, group, d)
     if plan.num_tiles:
+        # few, long tiles (a portion of one long prompt): their keys are cut into runs so that
+        # the launch fills the chip; the runs are folded by the merge kernel
+        nsplit = 1
+        items = plan.num_tiles * nkv
+        longest = max(plan.tile_keys)
+        if window > 0:
+            longest = min(longest, window + tile_rows_of(lib))
+        if items < _PREFILL_SPLIT_BELOW and longest >= 2 * _PREFILL_SPLIT_KEYS:
+            nsplit = min(_PREFILL_MAX_SPLITS, -(-_PREFILL_SPLIT_BELOW // items), longest // _PREFILL_SPLIT_KEYS)
+        part_o = part_ml = tokens_list = None
+        if nsplit > 1:
+            part_o = torch.empty((tokens, nq, nsplit, d), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((tokens, nq, nsplit, 2), dtype=torch.float32, device=q.device)
+            tokens_list = plan.prefill_tokens(q.device)
         _ok(
             lib.rl_attn_prefill(
                 _p(q), _p(k_cache), _p(v_cache), _p(out), _p(plan.tile_info),
                 _p(plan.work_order(nkv, q.device)), plan.num_tiles,
                 _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv,
-                window, ctypes.c_float(scale), _stream(),
+                window, ctypes.c_float(scale), nsplit, _p(part_o), _p(part_ml), _p(tokens_list),
+                0 if tokens_list is None else tokens_list.numel(), _stream(),
             ),
             "rl_attn_prefill",
         )

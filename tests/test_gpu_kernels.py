@@ -97,6 +97,8 @@ ATTN_CASES = [
     (10, 5, 112, 12, 40, [(333, 1), (77, 50)]),
     (8, 2, 128, 16, 0, [(20000, 1), (16000, 150), (9000, 1)]),  # long contexts: many splits, a long prefix
     (4, 1, 64, 8, 3000, [(12000, 1), (5000, 40)]),               # a window deep in a long context
+    (8, 2, 128, 16, 0, [(3584, 512)]),   # one portion of a long prompt: few, long tiles, their keys cut into runs
+    (6, 3, 64, 8, 0, [(1500, 300), (40, 1), (2100, 33)]),  # the same beside a single token, odd lengths
 ]
 
 
