@@ -1,9 +1,11 @@
 // Paged causal attention in true float32 on the matrix cores' float32 instruction
 // (v_mfma_f32_16x16x4_f32), compiled for one head size RL_HEAD_DIM (a multiple of 16).
 //
-// One wave per (tile of 16 rows, kv head).  Rows are (token, query head of the kv group)
-// pairs of ONE request, so grouped heads and neighbouring tokens share every key that is
-// read.  As in the bfloat16 kernels the transposed products are computed,
+// One workgroup of four waves per (tile of 16 rows, kv head).  Rows are (token, query head of
+// the kv group) pairs of ONE request, so grouped heads and neighbouring tokens share every key
+// that is read.  The key tiles are dealt to the waves by their absolute index (tile i goes to
+// wave i % 4), each wave keeps a softmax state of its own, and the four states are folded in
+// the order of the waves: a single token's long context is then read by four waves at once.  As in the bfloat16 kernels the transposed products are computed,
 //   S^T[keys, rows] = K[keys, d] Q^T[d, rows],   O^T[d, rows] += V^T[d, keys] P^T[keys, rows],
 // which leaves a lane with the scores of keys 4g .. 4g + 3 of its own row: exactly its
 // operand of the second product, whose other operand is one 16-byte read of the transposed
@@ -11,9 +13,9 @@
 //
 // A row's result does not depend on the tile it falls in, on the other rows there, or on how
 // a prompt was cut into steps: keys are taken in tiles of 16 at absolute positions 0, 16, ..,
-// in ascending order; within a tile the order of every sum is fixed by the key's position;
-// a tile that holds no visible key of a row leaves that row's state as it is, exactly
-// (factor 1, terms 0).  Masked keys contribute exactly zero
+// each wave takes its tiles in ascending order; within a tile the order of every sum is fixed
+// by the key's position; a tile that holds no visible key of a row leaves that row's state as
+// it is, exactly (factor 1, terms 0), and so does a wave without visible keys in the fold.  Masked keys contribute exactly zero
 // (rapid_llm/kernels/ops/attention/flashdecoding.py:223-237); scores are (q . k) / sqrt(d)
 // (rapid_llm/modules/attention.py:62), softmax over keys in float32
 // (rapid_llm/kernels/ops/attention/flashattention2_nopad.py:138-168).
@@ -27,6 +29,7 @@ namespace f32attn {
 
 constexpr int D = RL_HEAD_DIM;
 constexpr int DB = D / 16;  // 16-channel chunks of the first product = blocks of the output
+constexpr int AW = 4;       // waves per workgroup: key tile i belongs to wave i % AW
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ inline f32x4 ld4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
@@ -43,7 +46,7 @@ __device__ inline float row_sum(float v) {
 
 // tile_info: [tiles][3] = index of the request's first token in the step, its tokens in the
 // step, first row of the tile.  The request's first position is read from `positions`.
-__global__ __launch_bounds__(RL_WAVE) void attn_f32_kernel(
+__global__ __launch_bounds__(AW* RL_WAVE) void attn_f32_kernel(
     const float* __restrict__ q, const float* __restrict__ k_cache,
     const float* __restrict__ v_cache, float* __restrict__ out,
     const int* __restrict__ tile_info, const int* __restrict__ positions,
@@ -53,7 +56,10 @@ __global__ __launch_bounds__(RL_WAVE) void attn_f32_kernel(
     const int hk = blockIdx.y;
     const int G = nq / nkv;
     const int at = tile_info[3 * tile], n = tile_info[3 * tile + 1], row0 = tile_info[3 * tile + 2];
-    const int lane = threadIdx.x;
+    __shared__ float fold_ml[AW - 1][2][RL_WAVE];
+    __shared__ float fold_acc[AW - 1][DB * 4][RL_WAVE];
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
     const int r16 = lane & 15;
     const int g = lane >> 4;
     const int start = positions[at];
@@ -123,24 +129,26 @@ __global__ __launch_bounds__(RL_WAVE) void attn_f32_kernel(
         return (part[0] + part[1]) + (part[2] + part[3]);
     };
 
-    // Software pipeline over the tiles: while tile t goes through softmax and the second
-    // product, the scores of tile t + 1 are already being multiplied and the operands of
-    // tile t + 2 are in flight.  A lone wave (decode) has nothing else to hide latency with.
+    // Software pipeline over the wave's tiles: while tile t goes through softmax and the
+    // second product, the scores of its next tile are already being multiplied and the
+    // operands of the one after are in flight.
+    constexpr int STEP = 16 * AW;
+    const int mine = lo + 16 * ((wave - lo / 16) & (AW - 1));  // first tile >= lo with index % AW == wave
     Frags cur, nxt;
     f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f}, s_next = s;
-    if (lo < hi) {
-        load(lo, cur);
+    if (mine < hi) {
+        load(mine, cur);
         s = scores(cur);
     }
-    if (lo + 16 < hi) load(lo + 16, nxt);
-    for (int kb = lo; kb < hi; kb += 16) {
+    if (mine + STEP < hi) load(mine + STEP, nxt);
+    for (int kb = mine; kb < hi; kb += STEP) {
         f32x4 vcur[DB];
 #pragma unroll
         for (int b = 0; b < DB; ++b) vcur[b] = cur.v[b];
-        if (kb + 16 < hi) {
+        if (kb + STEP < hi) {
             s_next = scores(nxt);
             cur = nxt;
-            if (kb + 32 < hi) load(kb + 32, nxt);
+            if (kb + 2 * STEP < hi) load(kb + 2 * STEP, nxt);
         }
         // ---- this lane's keys kb + 4g + i of its own row ------------------------------------
         float tmax = -INFINITY;
@@ -181,6 +189,31 @@ __global__ __launch_bounds__(RL_WAVE) void attn_f32_kernel(
         }
         s = s_next;
     }
+    // ---- fold the waves' states in their order (a wave without visible keys has m = -inf,
+    // l = 0 and zero sums: it changes nothing, exactly) ----------------------------------------
+    if (wave > 0) {
+        fold_ml[wave - 1][0][lane] = m;
+        fold_ml[wave - 1][1][lane] = l;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fold_acc[wave - 1][4 * b + i][lane] = acc[b][i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < AW - 1; ++w) {
+        const float m_w = fold_ml[w][0][lane], l_w = fold_ml[w][1][lane];
+        const float m_new = fmaxf(m, m_w);
+        if (m_new == -INFINITY) continue;
+        const float fa = expf(m - m_new), fb = expf(m_w - m_new);
+        l = l * fa + l_w * fb;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[b][i] = acc[b][i] * fa + fold_acc[w][4 * b + i][lane] * fb;
+        m = m_new;
+    }
     if (!row_ok) return;
     // acc[b][i] is channel 16b + 4g + i of the lane's row
     float* orow = out + ((size_t)(at + tok) * nq + head) * D + 4 * g;
@@ -202,7 +235,7 @@ extern "C" int rl_attn_f32(const float* q, const float* k_cache, const float* v_
                            hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535) return RL_ERR_ARG;
-    hipLaunchKernelGGL(f32attn::attn_f32_kernel, dim3(num_tiles, nkv), dim3(RL_WAVE), 0, stream, q,
+    hipLaunchKernelGGL(f32attn::attn_f32_kernel, dim3(num_tiles, nkv), dim3(f32attn::AW * RL_WAVE), 0, stream, q,
                        k_cache, v_cache, out, tile_info, positions, token_slot, block_table,
                        table_stride, page_size, nq, nkv, window, scale);
     return rl_launch_status();
