@@ -72,7 +72,11 @@ __global__ __launch_bounds__(FW* RL_WAVE) void gemm_f32_kernel(
     const int per = (chunks + FW - 1) / FW;
     const int c_lo = min(chunks, wave * per), c_hi = min(chunks, c_lo + per);
 
-    f32x4 wv[NT], av[MT], wn[NT], an[MT];
+    // With one tile (few rows: the weights are streamed once) four chunks are asked for
+    // together, so that the four lane groups read 256 contiguous bytes of every row and more
+    // loads are in flight; the products still run chunk by chunk in ascending order
+    constexpr int U = (NT * MT == 1) ? 4 : 1;
+    f32x4 wv[U][NT], av[U][MT], wn[U][NT], an[U][MT];
     auto load = [&](int c, f32x4* wd, f32x4* ad) {
         const int k = c * FCH + 4 * g;  // this lane's first k of the chunk
 #pragma unroll
@@ -81,21 +85,33 @@ __global__ __launch_bounds__(FW* RL_WAVE) void gemm_f32_kernel(
         for (int mt = 0; mt < MT; ++mt)
             ad[mt] = aok[mt] ? load_k4<VEC>(arow[mt] + c * FCH, K - k) : (f32x4){0.f, 0.f, 0.f, 0.f};
     };
-    if (c_lo < c_hi) load(c_lo, wv, av);
-    for (int c = c_lo; c < c_hi; ++c) {
-        if (c + 1 < c_hi) load(c + 1, wn, an);  // the next chunk's loads fly during this one's products
+    auto load_group = [&](int c, f32x4 (*wd)[NT], f32x4 (*ad)[MT]) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int u = 0; u < U; ++u)
+            if (c + u < c_hi) load(c + u, wd[u], ad[u]);
+    };
+    if (c_lo < c_hi) load_group(c_lo, wv, av);
+    for (int c = c_lo; c < c_hi; c += U) {
+        if (c + U < c_hi) load_group(c + U, wn, an);  // the next group's loads fly during this one's products
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+        for (int u = 0; u < U; ++u) {
+            if (c + u >= c_hi) break;
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    acc[nt][mt] =
-                        __builtin_amdgcn_mfma_f32_16x16x4f32(wv[nt][j], av[mt][j], acc[nt][mt], 0, 0, 0);
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) wv[nt] = wn[nt];
+                for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) av[mt] = an[mt];
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[u][nt][j], av[u][mt][j],
+                                                                          acc[nt][mt], 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) wv[u][nt] = wn[u][nt];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) av[u][mt] = an[u][mt];
+        }
     }
 
     // the waves' partial tiles are added in the order of the waves, RED_TILES tiles at a time
