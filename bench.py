@@ -7,7 +7,8 @@ greedy sampling kernel, tokens fed back.  The default run has the layer sizes of
 Qwen3-8B (BASELINE.json ``configs[2]``), a batch of 8, every request with a 2,048-token
 prompt, context 4,096.  One JSON line is printed: decoded tokens a second (``value``), the
 2,048-token prefill (``prefill``), the decode step against the HBM roofline (``roofline``)
-and decoding at batch 1 and 64 (``points``).
+and decoding at batch 1 and 64 (``points``, which also holds the true 32-bit path's decode
+and prefill speed, measured in a second process).
 
 Metric definitions follow rapid_llm's docs/benchmark_models.md:141-149: decode tok/s is
 batch / mean step time; prefill tok/s is prompt tokens / prefill latency; both timed
@@ -121,6 +122,30 @@ def measured_peaks() -> int:
     return 0
 
 
+def float32_points(args) -> dict:
+    """The same model through the true 32-bit path, in a process of its own (the float32
+    weights need their own 33 GB): decode tok/s at the main batch size and prefill tok/s."""
+    import subprocess
+
+    cmd = [
+        sys.executable, os.path.abspath(__file__), "--dtype", "float32", "--batch", str(args.batch),
+        "--steps", "16", "--warmup", "4", "--points", "",
+    ]
+    if args.layers is not None:
+        cmd += ["--layers", str(args.layers)]
+    try:
+        done = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        line = json.loads(done.stdout.strip().splitlines()[-1])
+        out = {f"fp32_decode_b{args.batch}": line["value"]}
+        if line.get("prefill"):
+            out["fp32_prefill"] = line["prefill"]["value"]
+        print(f"[bench] float32 path: {out}", file=sys.stderr, flush=True)
+        return out
+    except Exception as err:  # the main line must not be lost to the float32 run
+        print(f"[bench] the float32 run gave no result: {err!r}", file=sys.stderr, flush=True)
+        return {}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -134,6 +159,7 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-pipeline", action="store_true", help="read every step's tokens before queueing the next")
+    ap.add_argument("--no-fp32", action="store_true", help="skip the float32 points (a second process)")
     ap.add_argument("--peaks", action="store_true",
                     help="measure what the device reaches with library kernels (a large read, copy and square products) and exit")
     args = ap.parse_args()
@@ -302,6 +328,8 @@ def main() -> int:
         s, _ = decode(b, args.point_steps, max(2, args.warmup // 2))
         pts[f"decode_b{b}"] = round(b / s, 2)
         print(f"[bench] decode batch {b}: {pts[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
+    if args.dtype == "bfloat16" and not args.no_fp32 and points:
+        pts.update(float32_points(args))
     result["points"] = pts
     print(json.dumps(result), flush=True)
     return 0
