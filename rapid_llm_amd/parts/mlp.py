@@ -60,7 +60,7 @@ class SwiGLU(FeedForward):
         gu = self.gate_up(x)
         act = torch.empty((x.shape[0], self.intermediate_size), dtype=gu.dtype, device=x.device)
         ops.swiglu(gu, act)
-        return self.down(act)
+        return self.down.deferred(act, ctx)
 
 
 FEED_FORWARDS.register("swiglu", SwiGLU)
