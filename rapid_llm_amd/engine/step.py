@@ -152,6 +152,8 @@ class ModelRunner:
         self.computed: dict[str, int] = {}
         self.vocab_size = self.spec.vocab_size
         self._graphs: dict[tuple[int, int], tuple] = {}
+        # a part that does not promise to be replayable keeps every step eager
+        self.graphs_allowed = self.model.replayable()
         # where the sampling kernels leave their choices, one row per sampled request of a
         # step; the next step's embedding reads fed tokens from here
         self.sampled = torch.zeros(max(1, self.engine.max_num_seqs), dtype=torch.int32, device=self.device)
@@ -393,6 +395,7 @@ class ModelRunner:
         meta = self._prepare(entries)
         if (
             (self.engine.use_graph if use_graph is None else use_graph)
+            and self.graphs_allowed
             and len(entries) <= GRAPH_BATCHES[-1]
             and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
         ):

@@ -92,6 +92,11 @@ class CausalLM:
         for part in self.all_parts():
             part.bind(params, runtime)
 
+    def replayable(self) -> bool:
+        """Whether a step of this model may be recorded into a graph: every part and every
+        block says so (``Part.replayable``)."""
+        return all(getattr(p, "replayable", False) for p in (*self.all_parts(), *self.blocks))
+
     # ---- cache -----------------------------------------------------------------
     def cache_needs(self) -> list[CacheNeed]:
         """One need per place in the run order.  ``LayerSpec.share_cache_with`` names a layer;

@@ -24,6 +24,8 @@ from .linear import Linear
 
 
 class GQAAttention(Mixer):
+    replayable = True
+
     def __init__(
         self,
         hidden_size: int,

@@ -93,6 +93,15 @@ class CacheNeed:
 class Part:
     """Common protocol: declare tensors, receive them, run."""
 
+    #: A part whose ``forward`` may be recorded once into a HIP graph and replayed for later
+    #: steps declares ``replayable = True``.  It promises that everything ``forward`` does on
+    #: the host depends only on what is fixed for a recorded step (the number of rows, the
+    #: context bound in ``ctx.extra["context_bound"]``), that every per-step value (ids,
+    #: positions, slots, block tables, state) is read on the device from the tensors of
+    #: ``ctx`` and of the cache, and that nothing waits for the device or copies from the host.
+    #: A model with a part that does not declare it runs every step eagerly.
+    replayable = False
+
     def param_specs(self) -> list[ParamSpec]:
         return []
 

@@ -12,6 +12,7 @@ from .lazy import run_norm
 
 
 class PreNormBlock(Block):
+    replayable = True
     accepts_deferred = True  # the incoming delta may be a DeferredProduct
 
     def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm) -> None:

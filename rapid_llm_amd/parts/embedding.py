@@ -15,6 +15,8 @@ from .linear import Linear
 
 
 class TokenEmbedding(Part):
+    replayable = True
+
     def __init__(self, vocab_size: int, hidden_size: int, checkpoint_name: str, name: str = "embed") -> None:
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.checkpoint_name = checkpoint_name
@@ -43,6 +45,8 @@ class TokenEmbedding(Part):
 
 class OutputProjection(Part):
     """``logits = h W^T`` in float32, over the rows that were asked for only."""
+
+    replayable = True
 
     def __init__(
         self,

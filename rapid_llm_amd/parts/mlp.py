@@ -16,6 +16,8 @@ from .linear import Linear
 
 
 class SwiGLU(FeedForward):
+    replayable = True
+
     def __init__(
         self,
         hidden_size: int,

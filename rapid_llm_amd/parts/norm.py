@@ -16,6 +16,7 @@ from .lazy import DeferredProduct
 
 
 class RMSNorm(Norm):
+    replayable = True
     fuses_products = True  # takes a DeferredProduct as delta, may return ScaledRows
 
     def __init__(self, size: int, eps: float, checkpoint_name: str, name: str = "norm") -> None:

@@ -17,6 +17,7 @@ from .base import POSITION_ENCODINGS, PositionEncoding
 
 
 class NoPositionEncoding(PositionEncoding):
+    replayable = True
     kind = "none"
 
     def __init__(self, **_ignored) -> None:
@@ -25,6 +26,7 @@ class NoPositionEncoding(PositionEncoding):
 
 
 class RotaryHalfSplit(PositionEncoding):
+    replayable = True
     kind = "rope_half_split"
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None) -> None:

@@ -440,6 +440,44 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
         NORMS.unregister("toy_plain_norm")
 
 
+def test_toy_architecture_generates_through_the_entry_point(tmp_path):
+    """The toy model under the scheduler, graphs and pipeline left at their defaults: the toy
+    mixer walks host lists and does not declare itself replayable, so every step runs eagerly;
+    slots (and with them the mixer's state) pass from finished requests to waiting ones."""
+    from safetensors.torch import load_file
+
+    from rapid_llm_amd import LLM, SamplingParams, write_random_model
+    from rapid_llm_amd.config import register_architecture, unregister_architecture
+    from rapid_llm_amd.parts import FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS
+
+    _toy_parts()
+    register_architecture("ToyForCausalLM", ToyConfig, _toy_spec, replace=True)
+    try:
+        cfg = ToyConfig(hidden=48, vocab=97, heads=3, head_dim=16, inter=80, decay=0.8, period=9.0)
+        folder = write_random_model(cfg.to_dict(), 5, tmp_path / "toy", dtype="float32")
+        weights = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
+        llm = LLM(str(folder), dtype="float32", max_seq_len=64, page_size=8, num_pages=24, max_num_seqs=2,
+                  max_chunk_size=6, max_num_batched_tokens=16)
+        runner = llm.scheduler.runner
+        assert not runner.graphs_allowed and runner.engine.use_graph
+        prompts = [random_tokens(n, cfg.vocab, 70 + i) for i, n in enumerate((9, 14, 3, 11, 6))]
+        new = 7
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_gen_len=new))
+        assert not runner._graphs
+        for prompt, out in zip(prompts, outs):
+            toks = list(prompt)
+            for _ in range(new):
+                toks.append(int(_toy_plain(weights, cfg, toks)[-1].argmax()))
+            assert out.outputs[0].token_ids == toks[len(prompt):]
+        runner.cache.check_invariants()
+    finally:
+        unregister_architecture("ToyForCausalLM")
+        MIXERS.unregister("toy_decaying_sum")
+        FEED_FORWARDS.unregister("toy_routed")
+        POSITION_ENCODINGS.unregister("toy_phase")
+        NORMS.unregister("toy_plain_norm")
+
+
 def test_unknown_part_kinds_are_named():
     from rapid_llm_amd.models import CausalLM, LayerSpec, ModelSpec, PartSpec
 
