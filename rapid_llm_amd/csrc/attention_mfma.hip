@@ -42,6 +42,7 @@ static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple 
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int DC = (D + 31) / 32;     // 32-channel chunks of the first product
 constexpr int DB = D / 16;            // 16-channel blocks of the output
@@ -72,16 +73,22 @@ __device__ inline f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-// maximum over the four lanes (groups) that hold the same row
+// Maximum and sum over the four lanes (one in each row of 16) that hold the same query row:
+// two lane swaps of gfx950 (the halves of the wave, then neighbouring rows of 16) instead of
+// two trips through the LDS crossbar.
 __device__ inline float row_max4(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16, RL_WAVE));
-    v = fmaxf(v, __shfl_xor(v, 32, RL_WAVE));
-    return v;
+    const unsigned u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned w = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ inline float row_sum4(float v) {
-    v += __shfl_xor(v, 16, RL_WAVE);
-    v += __shfl_xor(v, 32, RL_WAVE);
-    return v;
+    const unsigned u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned w = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 // --------------------------------------------------------------------------- //
@@ -591,13 +598,14 @@ extern "C" int rl_attn_decode_fusable() { return D % 64 == 0 ? 1 : 0; }
 #ifndef RL_PF_NQ
 #define RL_PF_NQ 2
 #endif
-#define PF_WAVES 4
+#define PF_WAVES 4                       // waves that share the rows of a tile
 #define PF_NQ RL_PF_NQ                   // 16-row blocks per wave
 #define PF_ROWS (PF_WAVES * PF_NQ * 16)  // rows per workgroup
 #define PF_KEYS 64                       // keys per LDS tile and per softmax step
-#define PF_THREADS (PF_WAVES * RL_WAVE)
+#define PF_THREADS (PF_WAVES * RL_WAVE)  // threads of one wave group
 #define K_LD (D + 8)                     // padded row of the K tile (bfloat16 elements)
 #define V_LD (PF_KEYS + 8)               // padded row of the V^T tile
+#define PF_TILE_ELEMS (PF_KEYS * K_LD + D * V_LD)  // one group's K and V^T tiles in LDS
 
 // Softmax is the arithmetic that competes with the matrix cores here, so a step covers 64
 // keys (one maximum, one rescale and one sum for 16 scores per lane), scores are masked only
@@ -611,16 +619,28 @@ extern "C" int rl_attn_decode_fusable() { return D % 64 == 0 ? 1 : 0; }
 // Two waves per SIMD at most: the accumulators then live in ordinary vector registers, which
 // the rescale and the epilogue read directly (at the default budget of 128 the compiler parks
 // them in accumulation registers and moves them back and forth around every rescale).
-__global__ __launch_bounds__(PF_WAVES* RL_WAVE) __attribute__((amdgpu_waves_per_eu(1, 2))) void
+//
+// GROUPS == 2: the two waves of a SIMD belong to one workgroup.  Two groups of four waves hold
+// the same rows and take the 64-key steps of the tile alternately (group 0 the even ones), each
+// with K and V^T tiles of its own in LDS; at the end group 1 hands its softmax state and
+// accumulators to group 0 through LDS.  A tile is then walked in half as many steps, which
+// pays when the longest tile bounds the launch's time (one prompt from its start: every
+// workgroup is resident at once and the last rows see the most keys).  GROUPS == 1: the two
+// waves of a SIMD belong to two workgroups with tiles of their own, which drift apart so that
+// one's matrix products overlap the other's softmax; better when there is enough work to keep
+// every unit busy (2,048 tokens of Qwen3-8B from the start: 78 against 86 us; 8,192 tokens:
+// 819 against 731 us).
+template <int GROUPS>
+__global__ __launch_bounds__(GROUPS* PF_THREADS) __attribute__((amdgpu_waves_per_eu(1, 2))) void
 attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out,
     const int* __restrict__ tile_info, const int* __restrict__ work_order,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int window, float scale_log2, int nsplit,
+    int page_size, unsigned page_magic, int nq, int nkv, int window, float scale_log2, int nsplit,
     float* __restrict__ part_o, float* __restrict__ part_ml) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[PF_KEYS * K_LD];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * V_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t tiles[GROUPS * PF_TILE_ELEMS];
+    __shared__ float fold_ml[GROUPS > 1 ? PF_WAVES * PF_NQ * 2 * RL_WAVE : 1];
 
     const int G = nq / nkv;
     // nsplit > 1: the keys of every tile are cut into nsplit runs of whole 64-key steps, one
@@ -639,11 +659,14 @@ attn_prefill_kernel(
     const int seq_end = start + qlen;  // keys at or beyond this were never written
     const int* table = block_table + (size_t)token_slot[tok0] * table_stride;
 
-    const int tid = threadIdx.x;
+    const int grp = GROUPS > 1 ? threadIdx.x / PF_THREADS : 0;  // wave group: which steps
+    const int tid = threadIdx.x - grp * PF_THREADS;             // thread within the group
     const int lane = tid & (RL_WAVE - 1);
     const int wave = tid / RL_WAVE;
     const int col = lane & 15;
     const int g = lane >> 4;
+    bf16_t* const Ks = tiles + grp * PF_TILE_ELEMS;
+    bf16_t* const Vs = Ks + PF_KEYS * K_LD;
 
     // rows of this lane: one per 16-row block
     int r_tok[PF_NQ], r_head[PF_NQ], r_pos[PF_NQ];
@@ -691,31 +714,37 @@ attn_prefill_kernel(
     constexpr int KCH = (D / 8 + TPK - 1) / TPK;
     constexpr int KG = PF_KEYS / 4;  // groups of four keys
     constexpr int VCH = (D + PF_THREADS / KG - 1) / (PF_THREADS / KG);
-    uint4 kreg[KCH];
-    uint2 vreg[VCH];
-    auto stage_load = [&](int base) {
+    // native vector types: an array of them is taken apart into registers, whereas an array
+    // of uint4 structs stayed in memory and each tile's keys were waited for as soon as asked for
+    bf16x8 kreg[KCH];
+    u32x2 vreg[VCH];
+    // The page ids of a step are asked for one step before its keys and values, so that no
+    // wave waits for a table entry in front of its products.  key / page_size is a multiply
+    // by page_magic = ceil(2^32 / page_size), exact for key < 2^32 / page_size (host-checked).
+    int k_key = 0, k_page = 0, v_key = 0, v_page = 0;
+    auto stage_pages = [&](int base) {
+        k_key = min(base + tid / TPK, seq_end - 1);  // clamped; masked by position below
+        k_page = table[__umulhi((unsigned)k_key, page_magic)];
+        v_key = min(base + 4 * (tid % KG), (seq_end - 1) & ~3);
+        v_page = table[__umulhi((unsigned)v_key, page_magic)];
+    };
+    auto stage_load = [&]() {
         {
-            const int kk = tid / TPK;
-            const int key = min(base + kk, seq_end - 1);  // clamped; masked by position below
-            const int page = table[key / page_size];
-            const bf16_t* krow =
-                k_cache + (((size_t)page * nkv + hk) * page_size + key % page_size) * D;
+            const int in_page = k_key - (int)__umulhi((unsigned)k_key, page_magic) * page_size;
+            const bf16_t* krow = k_cache + (((size_t)k_page * nkv + hk) * page_size + in_page) * D;
 #pragma unroll
             for (int i = 0; i < KCH; ++i) {
                 const int ch = tid % TPK + i * TPK;
-                if (ch < D / 8) kreg[i] = *reinterpret_cast<const uint4*>(krow + 8 * ch);
+                if (ch < D / 8) kreg[i] = load16(krow + 8 * ch);
             }
         }
         {
-            const int kg = tid % KG;
-            const int keyc = min(base + 4 * kg, (seq_end - 1) & ~3);
-            const int page = table[keyc / page_size];
-            const bf16_t* vbase =
-                v_cache + (((size_t)page * nkv + hk) * D) * page_size + keyc % page_size;
+            const int in_page = v_key - (int)__umulhi((unsigned)v_key, page_magic) * page_size;
+            const bf16_t* vbase = v_cache + (((size_t)v_page * nkv + hk) * D) * page_size + in_page;
 #pragma unroll
             for (int i = 0; i < VCH; ++i) {
                 const int d = tid / KG + i * (PF_THREADS / KG);
-                if (d < D) vreg[i] = *reinterpret_cast<const uint2*>(vbase + (size_t)d * page_size);
+                if (d < D) vreg[i] = *reinterpret_cast<const u32x2*>(vbase + (size_t)d * page_size);
             }
         }
     };
@@ -730,7 +759,7 @@ attn_prefill_kernel(
 #pragma unroll
             for (int i = 0; i < KCH; ++i) {
                 const int ch = tid % TPK + i * TPK;
-                if (ch < D / 8) *reinterpret_cast<uint4*>(&Ks[lrow * K_LD + 8 * ch]) = kreg[i];
+                if (ch < D / 8) *reinterpret_cast<bf16x8*>(&Ks[lrow * K_LD + 8 * ch]) = kreg[i];
             }
         }
         {
@@ -750,12 +779,12 @@ attn_prefill_kernel(
             for (int i = 0; i < VCH; ++i) {
                 const int d = tid / KG + i * (PF_THREADS / KG);
                 if (d < D) {
-                    uint2 v = vreg[i];
+                    u32x2 v = vreg[i];
                     if (!all_in) {
                         v.x &= keep_x;
                         v.y &= keep_y;
                     }
-                    *reinterpret_cast<uint2*>(&Vs[d * V_LD + 4 * kg]) = v;
+                    *reinterpret_cast<u32x2*>(&Vs[d * V_LD + 4 * kg]) = v;
                 }
             }
         }
@@ -769,13 +798,29 @@ attn_prefill_kernel(
         run_end = min(tile_kend, first_base + (split + 1) * per * PF_KEYS);
         first_base += split * per * PF_KEYS;
     }
-    if (first_base < run_end) stage_load(first_base);
-    for (int base = first_base; base < run_end; base += PF_KEYS) {
+    constexpr int STRIDE = GROUPS * PF_KEYS;  // the groups advance together
+    if (first_base + grp * PF_KEYS < run_end) {
+        stage_pages(first_base + grp * PF_KEYS);
+        stage_load();
+        if (first_base + grp * PF_KEYS + STRIDE < run_end) stage_pages(first_base + grp * PF_KEYS + STRIDE);
+    }
+    // q has arrived before the loop starts: inside it, waiting for q would mean waiting for
+    // everything asked for since, the next step's keys and values included
+#pragma unroll
+    for (int n = 0; n < PF_NQ; ++n)
+#pragma unroll
+        for (int c = 0; c < DC; ++c) asm volatile("" : "+v"(qf[n][c]));
+    for (int both = first_base; both < run_end; both += STRIDE) {
+        const int base = both + grp * PF_KEYS;  // this group's step
+        const bool live = base < run_end;       // group 1 may have no last step
         __syncthreads();  // the previous tile has been consumed
-        stage_store(base);
+        if (live) stage_store(base);
         __syncthreads();
-        if (base + PF_KEYS < run_end) stage_load(base + PF_KEYS);
-        if (base > wave_max_pos) continue;  // every key of the tile is ahead of this wave's rows
+        if (base + STRIDE < run_end) {
+            stage_load();  // of the step whose page ids were asked for a step ago
+            if (base + 2 * STRIDE < run_end) stage_pages(base + 2 * STRIDE);
+        }
+        if (!live || base > wave_max_pos) continue;  // no key of the step is visible to this wave's rows
         // masks are needed where the diagonal or a window's edge crosses the tile
         const bool need_mask =
             (base + PF_KEYS - 1 > wave_min_pos) || (window > 0 && base < wave_max_pos - window + 1);
@@ -856,6 +901,47 @@ attn_prefill_kernel(
             }
         }
     }
+    if (GROUPS > 1) {
+        // group 1's state travels through the LDS that held the tiles: element j of a lane at
+        // [wave][j][lane]; group 0 folds it into its own
+        float* fold_acc = reinterpret_cast<float*>(tiles);
+        constexpr int PER_LANE = PF_NQ * DB * 4;
+        static_assert(GROUPS == 1 ||
+                          sizeof(float) * PF_WAVES * PER_LANE * RL_WAVE <= sizeof(bf16_t) * GROUPS * PF_TILE_ELEMS,
+                      "the accumulators of one group fit where the tiles were");
+        __syncthreads();  // every wave has read its last tile
+        if (grp == 1) {
+#pragma unroll
+            for (int n = 0; n < PF_NQ; ++n) {
+                fold_ml[((wave * PF_NQ + n) * 2 + 0) * RL_WAVE + lane] = m[n];
+                fold_ml[((wave * PF_NQ + n) * 2 + 1) * RL_WAVE + lane] = l[n];
+#pragma unroll
+                for (int b = 0; b < DB; ++b)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        fold_acc[(wave * PER_LANE + (n * DB + b) * 4 + i) * RL_WAVE + lane] = acc[n][b][i];
+            }
+        }
+        __syncthreads();
+        if (grp == 1) return;
+#pragma unroll
+        for (int n = 0; n < PF_NQ; ++n) {
+            const float m1 = fold_ml[((wave * PF_NQ + n) * 2 + 0) * RL_WAVE + lane];
+            const float l1 = fold_ml[((wave * PF_NQ + n) * 2 + 1) * RL_WAVE + lane];
+            const float m_new = fmaxf(m[n], m1);
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+            const float a0 = __builtin_amdgcn_exp2f(m[n] - m_safe);
+            const float a1 = __builtin_amdgcn_exp2f(m1 - m_safe);
+            m[n] = m_new;
+            l[n] = l[n] * a0 + l1 * a1;
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[n][b][i] = acc[n][b][i] * a0 +
+                                   fold_acc[(wave * PER_LANE + (n * DB + b) * 4 + i) * RL_WAVE + lane] * a1;
+        }
+    }
 #pragma unroll
     for (int n = 0; n < PF_NQ; ++n) {
         const float lt = row_sum4(l[n]);
@@ -892,6 +978,7 @@ attn_prefill_kernel(
 
 extern "C" int rl_attn_prefill_rows() { return PF_ROWS; }
 
+// groups: 1 or 2 wave groups per workgroup (a compute unit then holds 2 or 1 workgroups).
 // nsplit > 1 cuts every tile's keys into that many runs (for launches of few, long tiles);
 // part_o [tokens of the step, nq, nsplit, D] and part_ml [.., 2] then hold the runs' results
 // and prefill_tokens [num_prefill_tokens] names the tokens the merge kernel writes.
@@ -899,21 +986,24 @@ extern "C" int rl_attn_prefill(const void* q, const void* k_cache, const void* v
                                const int* tile_info, const int* work_order, int num_tiles,
                                const int* token_slot,
                                const int* block_table, int table_stride, int page_size, int nq,
-                               int nkv, int window, float scale, int nsplit, float* part_o,
+                               int nkv, int window, float scale, int groups, int nsplit, float* part_o,
                                float* part_ml, const int* prefill_tokens, int num_prefill_tokens,
                                hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
-    if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || nsplit < 1)
+    if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || nsplit < 1 ||
+        (groups != 1 && groups != 2))
         return RL_ERR_ARG;
     if (nsplit > 1 && (!part_o || !part_ml || !prefill_tokens || num_prefill_tokens < 1 || nq > 65535))
         return RL_ERR_ARG;
     const float scale_log2 = scale * 1.4426950408889634f;
+    const unsigned page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     if ((long)num_tiles * nkv * nsplit > 0x7fffffffL) return RL_ERR_ARG;
-    dim3 grid(num_tiles * nkv * nsplit), block(PF_WAVES * RL_WAVE);
-    hipLaunchKernelGGL(attn_prefill_kernel, grid, block, 0, stream, (const bf16_t*)q,
-                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_info,
-                       work_order, token_slot, block_table, table_stride, page_size, nq, nkv, window,
-                       scale_log2, nsplit, part_o, part_ml);
+    dim3 grid(num_tiles * nkv * nsplit), block(groups * PF_THREADS);
+    auto kernel = groups == 2 ? attn_prefill_kernel<2> : attn_prefill_kernel<1>;
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache,
+                       (const bf16_t*)v_cache, (bf16_t*)out, tile_info, work_order, token_slot,
+                       block_table, table_stride, page_size, page_magic, nq, nkv, window, scale_log2,
+                       nsplit, part_o, part_ml);
     if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
     if (nsplit > 1)
         hipLaunchKernelGGL(attn_merge_kernel, dim3(num_prefill_tokens, nq), dim3(D < 64 ? 64 : D), 0,

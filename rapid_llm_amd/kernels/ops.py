@@ -580,20 +580,23 @@ class AttentionPlan:
             self._prefill_tokens = upload_ints(self._prefill_list, device)
         return self._prefill_tokens
 
-    def work_order(self, nkv: int, device) -> torch.Tensor:
-        """Order in which the (tile, kv head) pairs of the prefill kernel are handed out.
-        The first round, one workgroup on every compute unit, takes the longest; the second
-        round, which joins them on the same units, the shortest in ascending order, so that a
-        unit's two workgroups add up alike; the rest follow longest first and fill the gaps."""
-        order = self.orders.get(nkv)
+    def work_order(self, nkv: int, device, resident: int = 1) -> torch.Tensor:
+        """Order in which the (tile, kv head) pairs of the prefill kernel are handed out:
+        longest first, so that the short ones fill the gaps at the end.  Where a compute unit
+        holds two workgroups at a time (``resident == 2``), the first round, one workgroup on
+        every unit, takes the longest, and the second round, which joins them on the same
+        units, the shortest in ascending order, so that a unit's two workgroups add up alike."""
+        order = self.orders.get((nkv, resident))
         if order is None:
             items = sorted(range(self.num_tiles * nkv), key=lambda i: (-self.tile_keys[i // nkv], i))
-            first = items[:_FIRST_ROUND]
-            rest = items[_FIRST_ROUND:]
-            second = rest[::-1][:_FIRST_ROUND]
-            middle = rest[: max(0, len(rest) - _FIRST_ROUND)]
-            order = upload_ints(first + second + middle, device)
-            self.orders[nkv] = order
+            if resident == 2:
+                first = items[:_FIRST_ROUND]
+                rest = items[_FIRST_ROUND:]
+                second = rest[::-1][:_FIRST_ROUND]
+                middle = rest[: max(0, len(rest) - _FIRST_ROUND)]
+                items = first + second + middle
+            order = upload_ints(items, device)
+            self.orders[(nkv, resident)] = order
         return order
 
 
@@ -614,6 +617,34 @@ _PREFILL_MAX_SPLITS = 8
 
 def tile_rows_of(lib) -> int:
     return lib.rl_attn_prefill_rows()
+
+
+_PREFILL_STEP_KEYS = 64  # keys per step of the prefill kernel
+_PREFILL_SLOTS = 512  # wave groups of four the chip holds at a time (two on each compute unit)
+# what a step costs more when the two wave groups of a compute unit walk one tile in lockstep
+# than when they belong to two tiles and drift apart (measured: 3.17 against 2.83 us)
+_PREFILL_PAIRED_COST = 1.12
+
+
+def _prefill_shape(plan: "AttentionPlan", nkv: int, window: int, tile_rows: int) -> tuple[int, int]:
+    """(wave groups per workgroup, runs the keys of every tile are cut into) for a launch of
+    the prefill kernel.  Few, long tiles (a portion of one long prompt) have their keys cut
+    into runs, folded by the merge kernel, so that the launch fills the chip.  Two wave groups
+    share each tile when the longest tile would otherwise outlast the work there is for
+    every other slot."""
+    keys = plan.tile_keys
+    if window > 0:
+        keys = [min(k, window + tile_rows) for k in keys]
+    items = plan.num_tiles * nkv
+    longest = max(keys)
+    nsplit = 1
+    if items < _PREFILL_SPLIT_BELOW and longest >= 2 * _PREFILL_SPLIT_KEYS:
+        nsplit = min(_PREFILL_MAX_SPLITS, -(-_PREFILL_SPLIT_BELOW // items), longest // _PREFILL_SPLIT_KEYS)
+    steps = [-(-k // _PREFILL_STEP_KEYS) for k in keys]
+    longest_steps = -(-max(steps) // nsplit)
+    share = nkv * sum(steps) / _PREFILL_SLOTS  # steps per slot if the work were spread evenly
+    paired = max(-(-longest_steps // 2), share) * _PREFILL_PAIRED_COST
+    return (2 if paired < max(longest_steps, share) else 1), nsplit
 
 
 def _f32_tiles(ctx, group: int) -> tuple[torch.Tensor, int]:
@@ -720,19 +751,14 @@ def paged_attention(
             f"position {ctx.max_position} needs page {ctx.max_position // page_size} of a block "
             f"table with {block_table.shape[1]} columns"
         )
+    if ctx.max_position >= (1 << 32) // page_size:
+        # the prefill kernel divides positions by the page size with one multiplication
+        raise KernelError(f"position {ctx.max_position} is too large for pages of {page_size} tokens")
     lib = attention_lib(d)
     group = nq // nkv
     plan = attention_plan(ctx, group, d)
     if plan.num_tiles:
-        # few, long tiles (a portion of one long prompt): their keys are cut into runs so that
-        # the launch fills the chip; the runs are folded by the merge kernel
-        nsplit = 1
-        items = plan.num_tiles * nkv
-        longest = max(plan.tile_keys)
-        if window > 0:
-            longest = min(longest, window + tile_rows_of(lib))
-        if items < _PREFILL_SPLIT_BELOW and longest >= 2 * _PREFILL_SPLIT_KEYS:
-            nsplit = min(_PREFILL_MAX_SPLITS, -(-_PREFILL_SPLIT_BELOW // items), longest // _PREFILL_SPLIT_KEYS)
+        groups, nsplit = _prefill_shape(plan, nkv, window, tile_rows_of(lib))
         part_o = part_ml = tokens_list = None
         if nsplit > 1:
             part_o = torch.empty((tokens, nq, nsplit, d), dtype=torch.float32, device=q.device)
@@ -741,9 +767,9 @@ def paged_attention(
         _ok(
             lib.rl_attn_prefill(
                 _p(q), _p(k_cache), _p(v_cache), _p(out), _p(plan.tile_info),
-                _p(plan.work_order(nkv, q.device)), plan.num_tiles,
+                _p(plan.work_order(nkv, q.device, 2 // groups)), plan.num_tiles,
                 _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv,
-                window, ctypes.c_float(scale), nsplit, _p(part_o), _p(part_ml), _p(tokens_list),
+                window, ctypes.c_float(scale), groups, nsplit, _p(part_o), _p(part_ml), _p(tokens_list),
                 0 if tokens_list is None else tokens_list.numel(), _stream(),
             ),
             "rl_attn_prefill",

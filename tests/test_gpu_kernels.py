@@ -118,6 +118,49 @@ def test_paged_attention(case, dtype):
         torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
 
 
+PREFILL_SHAPE_CASES = [
+    # nq, nkv, d, page, window, seqs: portions only
+    (8, 2, 128, 16, 0, [(0, 200), (700, 90), (0, 3)]),     # tiles of one step (the second wave group idle) and of many
+    (6, 3, 64, 8, 0, [(130, 61), (1000, 130)]),            # odd numbers of steps
+    (6, 2, 48, 4, 70, [(0, 300), (500, 40)]),              # a window: steps before it are never read
+    (4, 4, 256, 32, 0, [(40, 100)]),                       # the largest tiles in LDS
+    (5, 5, 16, 4, 0, [(0, 77), (90, 2)]),                  # the smallest
+]
+
+
+@pytest.mark.parametrize("case", PREFILL_SHAPE_CASES, ids=lambda c: f"h{c[0]}kv{c[1]}d{c[2]}p{c[3]}w{c[4]}")
+@pytest.mark.parametrize("shape", [(1, 1), (2, 1), (1, 3), (2, 3), (2, 8)], ids=lambda s: f"g{s[0]}n{s[1]}")
+def test_prefill_attention_in_every_launch_shape(case, shape, monkeypatch):
+    """One or two wave groups on a tile, its keys whole or cut into runs: the host picks by the
+    launch's size, here every combination is forced on the same problems."""
+    ops = _ops()
+    monkeypatch.setattr(ops, "_prefill_shape", lambda *a, **k: shape)
+    nq, nkv, d, page, window, seqs = case
+    q, kc, vc, table, ctx, want = _paged_problem(seqs, nq, nkv, d, page, torch.bfloat16, seed=d + page, window=window)
+    out = torch.full_like(q, float("nan"))
+    ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, window, 1.0 / math.sqrt(d))
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+
+
+def test_prefill_shape_follows_the_launch():
+    """Two wave groups where the longest tile would outlast everyone else's work (one prompt from
+    its start), one where there is work for every slot; key runs for few, long tiles."""
+    ops = _ops()
+
+    def shape(seqs, nkv=8, group=4, window=0):
+        ctx = SimpleNamespace(h_seq_starts=[a for a, _ in seqs], h_seq_lens=[n for _, n in seqs],
+                              token_ids=torch.zeros(1, dtype=torch.int32, device=DEV), extra={})
+        return ops._prefill_shape(ops.AttentionPlan(ctx, group, 128), nkv, window, 128)
+
+    assert shape([(0, 2048)]) == (2, 1)
+    assert shape([(0, 8192)]) == (1, 1)
+    assert shape([(3584, 512)]) == (1, 4)
+    assert shape([(0, 2048)] * 4) == (1, 1)
+    assert shape([(0, 20)]) == (1, 1)  # one step: nothing to share
+
+
 @pytest.mark.parametrize("case", ATTN_CASES[:7], ids=lambda c: f"h{c[0]}kv{c[1]}d{c[2]}p{c[3]}w{c[4]}")
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_attention_generic(case, dtype):
