@@ -70,8 +70,19 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
 // MB): strided reads 16.2 / 10.5 / 22.8 / 46.9; this kernel 14.7 / 9.4 / 20.5 / 41.0; weights
 // stored pre-tiled so that every instruction reads 1 KB contiguous 14.3 / 9.2 / 19.9 / 41.2
 // (no better, and the library product of the prefill could not read them); a plain read of
-// the same bytes 10 / 6.5 / 16 / 34.  Deeper unrolling, non-temporal loads, more waves, K
-// split over workgroups and staggered K offsets did not help.
+// the same bytes 10 / 6.5 / 16 / 34.  Non-temporal loads, more waves, K split over workgroups
+// and staggered K offsets did not help.  Two chunks in flight per wave, in two sets of
+// registers (see the main loop), then gave 14.0 / 9.4 / 21.9 / 38.4 where one chunk at a time
+// gave 14.9 / 9.7 / 22.2 / 42.6 in the same run.
+// sum over the four lanes l, l + 16, l + 32, l + 48 (two lane swaps of gfx950), left in all four
+__device__ inline float sum_rows_of_16(float v) {
+    const unsigned u = __float_as_uint(v);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned w = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 #define WT_PITCH 272  // bytes between the 16 rows of the LDS tile: 256 + 16, conflict-free reads
 
 struct SkinnyExtra {
@@ -86,13 +97,14 @@ struct SkinnyExtra {
     float* partial;       // [workgroups][16]
 };
 
-template <int NT, typename OutT, bool SWIGLU>
+template <int NT, typename OutT, bool SWIGLU, bool SCALED>
 __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, OutT* __restrict__ out, int M,
     int N, int K, int ldx, int ldw, int ldo, SkinnyExtra ex) {
     __shared__ float red[GW][NT * 256];
 
     __shared__ __attribute__((aligned(16))) unsigned char wtile[GW][16 * WT_PITCH];
+    __shared__ float wave_part[SCALED ? GW : 1][16];  // a scaled input's sums of squares by wave
 
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -164,29 +176,74 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
 
     // whole chunks of 128: no predicates.  The bound is the same for every lane of a wave.
     const int kfull = K & ~(KSTEP - 1);
-    for (int kw = wave * KSTEP; kw < kfull; kw += GW * KSTEP) {
-        uint4 raw[NT][4];
-        bf16x8 x[4];
+    // Two chunks in flight per wave, in two sets of registers used in turn: the loads of the
+    // chunk after next are issued before this chunk's products.  Inside the loop no load
+    // stands behind a condition (behind one the compiler counts it as absent and makes the
+    // oldest operand wait for the newest load); what is left, one chunk or two, follows it.
+    // Rows beyond M read row 0 (their results are never stored), so no load is predicated.
+    constexpr int XP_AHEAD = 8;  // partial sums a thread asks for ahead: 256 parts in all
+    float x_part[XP_AHEAD];
+    {
+        bf16x8 wa[NT][4], wb[NT][4], xa[4], xb[4];
+        auto load = [&](bf16x8 (&r)[NT][4], bf16x8 (&xx)[4], int kw) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) raw[nt][j] = *reinterpret_cast<const uint4*>(wld[nt][j] + kw);
+                for (int j = 0; j < 4; ++j) r[nt][j] = ld16(wld[nt][j] + kw);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) x[j] = xok ? ld16(xrow + kw + 8 * j) : z8();
+            for (int j = 0; j < 4; ++j) xx[j] = ld16(xrow + kw + 8 * j);
+        };
+        auto products = [&](bf16x8 (&r)[NT][4], bf16x8 (&xx)[4]) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            // the tiles of a wave go through the same piece of LDS one after the other
+            for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                *reinterpret_cast<uint4*>(mytile + (4 * j + g) * WT_PITCH + 16 * r16) = raw[nt][j];
-            bf16x8 a[4];
+                for (int j = 0; j < 4; ++j)
+                    *reinterpret_cast<bf16x8*>(mytile + (4 * j + g) * WT_PITCH + 16 * r16) = r[nt][j];
+                bf16x8 a[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                a[j] = __builtin_bit_cast(
-                    bf16x8, *reinterpret_cast<const uint4*>(mytile + r16 * WT_PITCH + 64 * g + 16 * j));
+                for (int j = 0; j < 4; ++j)
+                    a[j] = *reinterpret_cast<const bf16x8*>(mytile + r16 * WT_PITCH + 64 * g + 16 * j);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], x[j], acc[nt], 0, 0, 0);
+                for (int j = 0; j < 4; ++j)
+                    acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], xx[j], acc[nt], 0, 0, 0);
+            }
+        };
+        // A scaled input's partial sums of squares (thread (run j, row m) owns the partials
+        // j, j + 32, ..) are asked for behind the wave's last weights, without a condition,
+        // and arrive with them; they are added after the last products.  Asked for after the
+        // loop, their whole latency stood in the open in front of the epilogue (5 us a product
+        // where a compute unit holds one workgroup).
+        auto partial_loads = [&]() {
+            if constexpr (SCALED) {
+                const int m = threadIdx.x & 15, j = threadIdx.x >> 4;  // 512 threads: 32 runs
+#pragma unroll
+                for (int i = 0; i < XP_AHEAD; ++i)
+                    x_part[i] = ex.x_partial[min(j + 32 * i, ex.x_parts - 1) * 16 + m];
+            }
+        };
+        constexpr int S = GW * KSTEP;
+        int kw = wave * KSTEP;
+        if (kw >= kfull) partial_loads();
+        if (kw < kfull) {
+            int left = (kfull - kw + S - 1) / S;  // chunks of this wave, the loaded one included
+            load(wa, xa, kw);
+            while (left > 2) {
+                load(wb, xb, kw + S);
+                products(wa, xa);
+                load(wa, xa, kw + 2 * S);
+                products(wb, xb);
+                kw += 2 * S;
+                left -= 2;
+            }
+            if (left == 2) {
+                load(wb, xb, kw + S);
+                partial_loads();
+                products(wa, xa);
+                products(wb, xb);
+            } else {
+                partial_loads();
+                products(wa, xa);
+            }
         }
     }
     // the last, partial chunk (K is a multiple of 8: a piece is whole or absent)
@@ -203,35 +260,28 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
         }
     }
 
-    // the norm's factor of every row of a scaled input: thread (run j, row m) adds the
-    // partials j, j + 32, .. in order, then every row's 32 runs are added in order
-    // (the epilogues' small arrays live where the weight tiles were: an occupancy of three
-    // workgroups per compute unit hangs on a few hundred bytes of LDS)
-    float(*row_part)[16] = reinterpret_cast<float(*)[16]>(&wtile[0][0]);  // [32][16]
-    float* row_scale = reinterpret_cast<float*>(&wtile[0][0]) + 32 * 16;   // [16]
-    float* sq = row_scale + 16;                                            // [NT * 64]
-    static_assert(sizeof(wtile) >= (32 * 16 + 16 + NT * 64) * sizeof(float), "epilogue arrays fit");
-    if (ex.x_partial) {
-        const int m = threadIdx.x & 15, j = threadIdx.x >> 4;  // 512 threads: 32 runs
+    // The norm's factor of every row of a scaled input: thread (run j, row m) adds its partials
+    // j, j + 32, .. in order; the four runs of a wave are added by lane swaps, the eight waves'
+    // sums by every thread that needs the row's factor, in the order of the waves.  No barrier
+    // beyond the one that the waves' partial tiles need anyway.
+    // (the residual epilogue's small array lives where the weight tiles were)
+    float* sq = reinterpret_cast<float*>(&wtile[0][0]);  // [NT * 64]
+    static_assert(sizeof(wtile) >= NT * 64 * sizeof(float), "epilogue array fits");
+    if constexpr (SCALED) {
+        const int m = threadIdx.x & 15, j = threadIdx.x >> 4;
         float run = 0.f;
-        for (int p = j; p < ex.x_parts; p += 32) run += ex.x_partial[p * 16 + m];
-        __syncthreads();  // every wave has left the main loop: the weight tiles are free
-        row_part[j][m] = run;
+#pragma unroll
+        for (int i = 0; i < XP_AHEAD; ++i) run += (j + 32 * i < ex.x_parts) ? x_part[i] : 0.f;
+        for (int p = j + 32 * XP_AHEAD; p < ex.x_parts; p += 32) run += ex.x_partial[p * 16 + m];
+        run = sum_rows_of_16(run);
+        if (g == 0) wave_part[wave][m] = run;
     }
     // partial tiles of the waves -> LDS; lane-major so that reads below are conflict-free
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) red[wave][(nt * 4 + i) * 64 + lane] = acc[nt][i];
-    __syncthreads();
-    if (ex.x_partial) {
-        if (threadIdx.x < 16) {
-            float ss = 0.f;
-            for (int j = 0; j < 32; ++j) ss += row_part[j][threadIdx.x];
-            row_scale[threadIdx.x] = rsqrtf(ss * ex.x_inv_size + ex.x_eps);
-        }
-        __syncthreads();
-    }
+    __syncthreads();  // also: every wave has left the main loop, the weight tiles are free
 
     // thread -> (tile pair / tile, lane of the tile); sums the waves in order
     constexpr int OUT_TILES = SWIGLU ? NT / 2 : NT;
@@ -240,7 +290,13 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
         const int ot = e >> 6;
         const int m = ln & 15;
         const int nbase = (blockIdx.x * OUT_TILES + ot) * 16 + 4 * (ln >> 4);
-        const float scale = ex.x_partial ? row_scale[m] : 1.f;
+        float scale = 1.f;
+        if constexpr (SCALED) {
+            float ss = 0.f;
+#pragma unroll
+            for (int w = 0; w < GW; ++w) ss += wave_part[w][m];
+            scale = rsqrtf(ss * ex.x_inv_size + ex.x_eps);
+        }
         float sumsq = 0.f;
         if (m < M) {
 #pragma unroll
@@ -290,12 +346,12 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     }
 }
 
-template <int NT, typename OutT, bool SWIGLU>
+template <int NT, typename OutT, bool SWIGLU, bool SCALED>
 static int launch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
                   int ldw, int ldo, const SkinnyExtra& ex, hipStream_t stream) {
     constexpr int rows_per_block = (SWIGLU ? NT / 2 : NT) * 16;
     dim3 grid((N + rows_per_block - 1) / rows_per_block), block(GW * RL_WAVE);
-    hipLaunchKernelGGL((gemm_skinny_kernel<NT, OutT, SWIGLU>), grid, block, 0, stream, X, W, out,
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, OutT, SWIGLU, SCALED>), grid, block, 0, stream, X, W, out,
                        M, N, K, ldx, ldw, ldo, ex);
     return rl_launch_status();
 }
@@ -305,9 +361,13 @@ static int dispatch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, i
                     int ldw, int ldo, int nt, const SkinnyExtra& ex, hipStream_t stream) {
 #define RL_CASE(NTV)                                                                           \
     if (nt == NTV)                                                                             \
-        return launch<NTV, OutT, SWIGLU>(X, W, out, M, N, K, ldx, ldw, ldo, ex, stream);
-    if (SWIGLU) {
-        RL_CASE(2) RL_CASE(4)
+        return ex.x_partial                                                                    \
+                   ? launch<NTV, OutT, SWIGLU, true>(X, W, out, M, N, K, ldx, ldw, ldo, ex, stream) \
+                   : launch<NTV, OutT, SWIGLU, false>(X, W, out, M, N, K, ldx, ldw, ldo, ex, stream);
+    // the gate/up variant holds a (gate, up) pair of tiles; two pairs would not fit the registers
+    // of two chunks in flight
+    if constexpr (SWIGLU) {
+        RL_CASE(2)
     } else {
         RL_CASE(1) RL_CASE(2)
     }

@@ -423,14 +423,19 @@ def sample_uniform(seed: int, counter: int) -> float:
 
 
 SKINNY_MAX_ROWS = 16  # rows up to which the hand-written bandwidth-bound product is used
-_MIN_BLOCKS = 512  # workgroups a skinny product should keep when it widens its tiles
-
-
 def _skinny_tiles(rows: int, out_features: int) -> int:
-    """Weight-row tiles per workgroup: two where the launch still has a couple of workgroups
-    per compute unit and more than a few rows share each weight tile (measured: 5% on the
-    widest matrices at 8 rows, a loss everywhere else)."""
-    return 2 if rows > 4 and -(-out_features // 32) >= _MIN_BLOCKS else 1
+    """Weight-row tiles of 16 per workgroup of the skinny product: one, which leaves the most
+    workgroups, except where two were measured faster (Qwen3-8B shapes, microseconds, one tile
+    against two): from 8 rows on when one tile would leave some compute units with two
+    workgroups and some with one (6,144 outputs: 14.0 / 12.5 at 8 rows, 17.2 / 15.9 at 16, but
+    11.8 / 12.5 at 1 row); and with more than 12 rows on matrices of a thousand tiles and more
+    (151,936 outputs: 275 / 244 at 16 rows, but 216 / 233 at 8)."""
+    blocks = -(-out_features // 16)
+    if rows >= 8 and 256 < blocks < 512:
+        return 2
+    if rows > 12 and blocks >= 1024:
+        return 2
+    return 1
 
 
 def _scaled_args(scaled, rows: int, k: int) -> tuple:
@@ -518,7 +523,7 @@ def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> t
     _need(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, k))
     inter = two_i // 2
     out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
-    nt = _skinny_tiles(m, inter) * 2  # pairs of (gate, up) tiles
+    nt = 2  # one (gate, up) pair of tiles per workgroup
     _ok(
         core().rl_gemm_skinny_swiglu(
             _p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, *_scaled_args(scaled, m, k), _stream()
