@@ -52,15 +52,11 @@ __global__ __launch_bounds__(FW* RL_WAVE) void gemm_f32_kernel(
     // rows beyond the matrices read the last row; their results are dropped at the end
     const float* wrow[NT];
     const float* arow[MT];
-    bool aok[MT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
         wrow[nt] = W + (size_t)min(n0 + nt * 16 + r16, N - 1) * ldw + 4 * g;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        aok[mt] = m0 + mt * 16 + r16 < M;
-        arow[mt] = A + (size_t)min(m0 + mt * 16 + r16, M - 1) * lda + 4 * g;
-    }
+    for (int mt = 0; mt < MT; ++mt) arow[mt] = A + (size_t)min(m0 + mt * 16 + r16, M - 1) * lda + 4 * g;
 
     f32x4 acc[NT][MT];
 #pragma unroll
@@ -74,44 +70,79 @@ __global__ __launch_bounds__(FW* RL_WAVE) void gemm_f32_kernel(
 
     // With one tile (few rows: the weights are streamed once) four chunks are asked for
     // together, so that the four lane groups read 256 contiguous bytes of every row and more
-    // loads are in flight; the products still run chunk by chunk in ascending order
+    // loads are in flight; the products still run chunk by chunk in ascending order.
     constexpr int U = (NT * MT == 1) ? 4 : 1;
-    f32x4 wv[U][NT], av[U][MT], wn[U][NT], an[U][MT];
-    auto load = [&](int c, f32x4* wd, f32x4* ad) {
+    // a chunk's operands: rows beyond A read A's last row (their results are dropped), so
+    // that no load depends on the lane
+    auto load = [&](int c, f32x4 (&wd)[NT], f32x4 (&ad)[MT]) {  // a whole chunk: no predicate
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) wd[nt] = *reinterpret_cast<const f32x4*>(wrow[nt] + c * FCH);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) ad[mt] = *reinterpret_cast<const f32x4*>(arow[mt] + c * FCH);
+    };
+    auto load_checked = [&](int c, f32x4 (&wd)[NT], f32x4 (&ad)[MT]) {
         const int k = c * FCH + 4 * g;  // this lane's first k of the chunk
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) wd[nt] = load_k4<VEC>(wrow[nt] + c * FCH, K - k);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            ad[mt] = aok[mt] ? load_k4<VEC>(arow[mt] + c * FCH, K - k) : (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int mt = 0; mt < MT; ++mt) ad[mt] = load_k4<VEC>(arow[mt] + c * FCH, K - k);
     };
-    auto load_group = [&](int c, f32x4 (*wd)[NT], f32x4 (*ad)[MT]) {
+    auto products = [&](f32x4 (&wd)[NT], f32x4 (&ad)[MT]) {
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (c + u < c_hi) load(c + u, wd[u], ad[u]);
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[nt][mt] =
+                        __builtin_amdgcn_mfma_f32_16x16x4f32(wd[nt][j], ad[mt][j], acc[nt][mt], 0, 0, 0);
     };
-    if (c_lo < c_hi) load_group(c_lo, wv, av);
-    for (int c = c_lo; c < c_hi; c += U) {
-        if (c + U < c_hi) load_group(c + U, wn, an);  // the next group's loads fly during this one's products
+    auto load_group = [&](int c, f32x4 (&wd)[U][NT], f32x4 (&ad)[U][MT]) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (c + u >= c_hi) break;
+        for (int u = 0; u < U; ++u) load(c + u, wd[u], ad[u]);
+        // the loads stay here, in front of the other group's products (left to itself the
+        // scheduler moves them down to their use and nothing is in flight during the products)
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto group_products = [&](f32x4 (&wd)[U][NT], f32x4 (&ad)[U][MT]) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[u][nt][j], av[u][mt][j],
-                                                                          acc[nt][mt], 0, 0, 0);
+        for (int u = 0; u < U; ++u) products(wd[u], ad[u]);
+    };
+    // Groups of whole chunks go through two sets of registers in turn: the group after next
+    // is asked for before this one is multiplied.  Inside the loop no load stands behind a
+    // condition (behind one the compiler counts it as absent and makes the oldest operand wait
+    // for the newest load); what the loop leaves, and the chunks that are not whole or do not
+    // fill a group, follow one by one.  The order of the sum is that of the chunks either way.
+    int c = c_lo;
+    {
+        const int whole = VEC ? min(c_hi, K / FCH) : c_lo;  // unaligned rows: every chunk is checked
+        int left = whole > c_lo ? (whole - c_lo) / U : 0;
+        if (left > 0) {
+            f32x4 wa[U][NT], aa[U][MT], wb[U][NT], ab[U][MT];
+            load_group(c, wa, aa);
+            while (left > 2) {
+                load_group(c + U, wb, ab);
+                group_products(wa, aa);
+                load_group(c + 2 * U, wa, aa);
+                group_products(wb, ab);
+                c += 2 * U;
+                left -= 2;
+            }
+            if (left == 2) {
+                load_group(c + U, wb, ab);
+                group_products(wa, aa);
+                group_products(wb, ab);
+                c += 2 * U;
+            } else {
+                group_products(wa, aa);
+                c += U;
+            }
         }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) wv[u][nt] = wn[u][nt];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) av[u][mt] = an[u][mt];
-        }
+    }
+    for (; c < c_hi; ++c) {
+        f32x4 w1[NT], a1[MT];
+        load_checked(c, w1, a1);
+        products(w1, a1);
     }
 
     // the waves' partial tiles are added in the order of the waves, RED_TILES tiles at a time
