@@ -129,27 +129,8 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_f32_kernel(
         return (part[0] + part[1]) + (part[2] + part[3]);
     };
 
-    // Software pipeline over the wave's tiles: while tile t goes through softmax and the
-    // second product, the scores of its next tile are already being multiplied and the
-    // operands of the one after are in flight.
-    constexpr int STEP = 16 * AW;
-    const int mine = lo + 16 * ((wave - lo / 16) & (AW - 1));  // first tile >= lo with index % AW == wave
-    Frags cur, nxt;
-    f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f}, s_next = s;
-    if (mine < hi) {
-        load(mine, cur);
-        s = scores(cur);
-    }
-    if (mine + STEP < hi) load(mine + STEP, nxt);
-    for (int kb = mine; kb < hi; kb += STEP) {
-        f32x4 vcur[DB];
-#pragma unroll
-        for (int b = 0; b < DB; ++b) vcur[b] = cur.v[b];
-        if (kb + STEP < hi) {
-            s_next = scores(nxt);
-            cur = nxt;
-            if (kb + 2 * STEP < hi) load(kb + 2 * STEP, nxt);
-        }
+    // softmax and second product of the tile at kb, given its scores and its values
+    auto finish_tile = [&](int kb, f32x4 s, const f32x4 (&vcur)[DB]) {
         // ---- this lane's keys kb + 4g + i of its own row ------------------------------------
         float tmax = -INFINITY;
 #pragma unroll
@@ -187,7 +168,46 @@ __global__ __launch_bounds__(AW* RL_WAVE) void attn_f32_kernel(
             for (int j = 0; j < 4; ++j)
                 acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[j], p[j], acc[b], 0, 0, 0);
         }
-        s = s_next;
+    };
+
+    // Software pipeline over the wave's tiles: while a tile goes through softmax and the second
+    // product, the scores of the next have been multiplied and the operands of the one after
+    // are in flight.  The last two tiles stand outside the loop, so that inside it the loads
+    // are issued without a condition and stay where they are written (behind a condition the
+    // compiler counts a load as absent and makes every older operand wait for it; left to
+    // itself the scheduler moves loads down to their use).
+    constexpr int STEP = 16 * AW;
+    const int mine = lo + 16 * ((wave - lo / 16) & (AW - 1));  // first tile >= lo with index % AW == wave
+    if (mine < hi) {
+        int left = (hi - mine + STEP - 1) / STEP;  // tiles of this wave, the current one included
+        int kb = mine;
+        Frags nxt;
+        f32x4 vcur[DB], vnext[DB];
+        load(kb, nxt);
+        f32x4 sc = scores(nxt);
+#pragma unroll
+        for (int b = 0; b < DB; ++b) vcur[b] = nxt.v[b];
+        if (left > 1) load(kb + STEP, nxt);
+        while (left > 2) {
+            const f32x4 s_next = scores(nxt);
+#pragma unroll
+            for (int b = 0; b < DB; ++b) vnext[b] = nxt.v[b];
+            load(kb + 2 * STEP, nxt);
+            __builtin_amdgcn_sched_barrier(0);
+            finish_tile(kb, sc, vcur);
+            sc = s_next;
+#pragma unroll
+            for (int b = 0; b < DB; ++b) vcur[b] = vnext[b];
+            kb += STEP;
+            --left;
+        }
+        if (left == 2) {
+            const f32x4 s_next = scores(nxt);
+            finish_tile(kb, sc, vcur);
+            finish_tile(kb + STEP, s_next, nxt.v);
+        } else {
+            finish_tile(kb, sc, vcur);
+        }
     }
     // ---- fold the waves' states in their order (a wave without visible keys has m = -inf,
     // l = 0 and zero sums: it changes nothing, exactly) ----------------------------------------
