@@ -604,7 +604,7 @@ extern "C" int rl_attn_decode_fusable() { return D % 64 == 0 ? 1 : 0; }
 #define PF_KEYS 64                       // keys per LDS tile and per softmax step
 #define PF_THREADS (PF_WAVES * RL_WAVE)  // threads of one wave group
 #define K_LD (D + 8)                     // padded row of the K tile (bfloat16 elements)
-#define V_LD (PF_KEYS + 8)               // padded row of the V^T tile
+#define V_LD (PF_KEYS + 16)              // padded row of the V^T tile (16 measured 3% faster than 8, 24 or 40)
 #define PF_TILE_ELEMS (PF_KEYS * K_LD + D * V_LD)  // one group's K and V^T tiles in LDS
 
 // Softmax is the arithmetic that competes with the matrix cores here, so a step covers 64
