@@ -187,6 +187,86 @@ extern "C" int rl_add_rmsnorm(float* residual, const void* delta, const float* w
     return rl_launch_status();
 }
 
+// The same norm where the delta arrives as `nparts` float32 runs of a product's K
+// (parts[run][row][hidden], see rl_gemm_mid_parts): the runs are added in order, the sum is
+// rounded to the activation type as a stored product would be, then added to the residual.
+template <typename T, int CHUNKS>
+__global__ void add_parts_rmsnorm_kernel(float* __restrict__ residual, const float* __restrict__ parts,
+                                         int nparts, size_t part_stride,
+                                         const float* __restrict__ weight, T* __restrict__ out,
+                                         int hidden, float eps) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    float4* res = reinterpret_cast<float4*>(residual + (size_t)row * hidden);
+    const int nvec = hidden >> 2;
+    const float4* w4 = reinterpret_cast<const float4*>(weight);
+    float4 val[CHUNKS], wt[CHUNKS];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) wt[c] = w4[i];
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) {
+            const float4* pr = reinterpret_cast<const float4*>(parts + (size_t)row * hidden) + i;
+            float4 d = *pr;
+            for (int r = 1; r < nparts; ++r) {
+                const float4 e = *reinterpret_cast<const float4*>(
+                    reinterpret_cast<const float*>(pr) + (size_t)r * part_stride);
+                d.x += e.x;
+                d.y += e.y;
+                d.z += e.z;
+                d.w += e.w;
+            }
+            float4 v = res[i];
+            v.x += to_float(from_float<T>(d.x));
+            v.y += to_float(from_float<T>(d.y));
+            v.z += to_float(from_float<T>(d.z));
+            v.w += to_float(from_float<T>(d.w));
+            res[i] = v;
+            val[c] = v;
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float rrms = rsqrtf(ss / (float)hidden + eps);
+    Vec4<T>* o = reinterpret_cast<Vec4<T>*>(out + (size_t)row * hidden);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * blockDim.x;
+        if (i < nvec) {
+            const float4 w = wt[c];
+            Vec4<T> y;
+            y.v[0] = from_float<T>(val[c].x * rrms * w.x);
+            y.v[1] = from_float<T>(val[c].y * rrms * w.y);
+            y.v[2] = from_float<T>(val[c].z * rrms * w.z);
+            y.v[3] = from_float<T>(val[c].w * rrms * w.w);
+            o[i] = y;
+        }
+    }
+}
+
+// parts [nparts, rows, hidden] float32, contiguous; bfloat16 rows out; hidden a multiple of 4 up to 16 K
+extern "C" int rl_add_rmsnorm_parts(float* residual, const float* parts, int nparts,
+                                    const float* weight, void* out, int rows, int hidden, float eps,
+                                    hipStream_t stream) {
+    if (rows <= 0) return RL_OK;
+    if (nparts < 1 || hidden % 4 || hidden > 16 * 1024) return RL_ERR_ARG;
+    const int nvec = hidden / 4;
+    const int threads = ((nvec + RL_WAVE - 1) / RL_WAVE) * RL_WAVE;
+    const size_t stride = (size_t)rows * hidden;
+    if (threads <= 1024)
+        hipLaunchKernelGGL((add_parts_rmsnorm_kernel<bf16_t, 1>), dim3(rows), dim3(threads), 0, stream,
+                           residual, parts, nparts, stride, weight, (bf16_t*)out, hidden, eps);
+    else
+        hipLaunchKernelGGL((add_parts_rmsnorm_kernel<bf16_t, 4>), dim3(rows), dim3(1024), 0, stream,
+                           residual, parts, nparts, stride, weight, (bf16_t*)out, hidden, eps);
+    return rl_launch_status();
+}
+
 // --------------------------------------------------------------------------- //
 // SwiGLU on the packed [gate | up] row: out[:, j] = silu(x[:, j]) * x[:, I + j]
 // rapid_llm/kernels/ops/activation/swiglu.py:91-121

@@ -442,3 +442,147 @@ extern "C" int rl_gemm_skinny_residual(const void* X, const void* W, int M, int 
     return dispatch<bf16_t, false>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K,
                                    ldx, ldw, N, nt, ex, stream);
 }
+
+// =========================================================================== //
+// 17 .. 64 rows: the runs of K of a product whose result feeds the residual
+// =========================================================================== //
+// The library's product reads X once for every 16 or 32 weight rows at these sizes and
+// stays near 3 TB/s.  Here a workgroup is four waves with 16 weight rows each; the chunk of X
+// they all need ([64 rows x 128 k], double-buffered) goes through LDS once per workgroup, the
+// weights stream as in the skinny product (two chunks in flight per wave, no load behind a
+// condition).  A matrix of 4,096 rows gives only 64 such workgroups, so K is cut into `ks`
+// runs (grid.y) whose float32 results [ks][M][N] are added by the norm kernel that consumes
+// them (rl_add_rmsnorm_parts).  Measured against the library at 64 rows (Qwen3-8B shapes,
+// microseconds): 4,096 x 4,096 11.8 / 14.9, 4,096 x 12,288 26.6 / 38.1; at 32 rows 9.9 / 13.9
+// and 23.0 / 28.6.  The wide products (6,144 and 24,576 rows) gain nothing (18.3 / 18.1 and
+// 55 / 46) and stay with the library.
+#define MW 4  // waves per workgroup
+
+template <int MB>
+__global__ __launch_bounds__(MW* RL_WAVE) void gemm_mid_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, float* __restrict__ part, int M,
+    int N, int K, int ldx, int ldw, int chunks_per_run) {
+    __shared__ __attribute__((aligned(16))) unsigned char xs[2][MB * 16 * WT_PITCH];
+    __shared__ __attribute__((aligned(16))) unsigned char wtile[MW][16 * WT_PITCH];
+    const int tid = threadIdx.x, lane = tid & (RL_WAVE - 1), wave = tid / RL_WAVE;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n0 = (blockIdx.x * MW + wave) * 16;
+    const int run = blockIdx.y;
+    const int c_lo = run * chunks_per_run, c_hi = min(K / KSTEP, c_lo + chunks_per_run);
+    // weights: instruction j reads row 4j + g of the wave's tile at bytes 16 r16 (as the skinny
+    // product does); rows beyond the matrix read its last row, their results are dropped
+    const bf16_t* wld[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) wld[j] = W + (size_t)min(n0 + 4 * j + g, N - 1) * ldw + 8 * r16;
+    // X: thread reads bytes 16 (tid % 16) of rows tid / 16 + 16 i; rows beyond M read the last
+    const bf16_t* xld[MB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i) xld[i] = X + (size_t)min(tid / 16 + 16 * i, M - 1) * ldx + 8 * (tid % 16);
+    unsigned char* mytile = wtile[wave];
+    f32x4 acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    bf16x8 wa[4], wb[4], xa[MB], xb[MB];
+    auto load = [&](bf16x8 (&w)[4], bf16x8 (&x)[MB], int c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = ld16(wld[j] + c * KSTEP);
+#pragma unroll
+        for (int i = 0; i < MB; ++i) x[i] = ld16(xld[i] + c * KSTEP);
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay in front of the other chunk's products
+    };
+    auto stage = [&](bf16x8 (&x)[MB], int buf) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            *reinterpret_cast<bf16x8*>(xs[buf] + (tid / 16 + 16 * i) * WT_PITCH + 16 * (tid % 16)) = x[i];
+    };
+    auto products = [&](bf16x8 (&w)[4], int buf) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<bf16x8*>(mytile + (4 * j + g) * WT_PITCH + 16 * r16) = w[j];
+        bf16x8 a[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            a[j] = *reinterpret_cast<const bf16x8*>(mytile + r16 * WT_PITCH + 64 * g + 16 * j);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            bf16x8 xf[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                xf[j] = *reinterpret_cast<const bf16x8*>(xs[buf] + (mb * 16 + r16) * WT_PITCH + 64 * g + 16 * j);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], xf[j], acc[mb], 0, 0, 0);
+        }
+    };
+    // Chunk c's X lives in buffer (c - c_lo) & 1.  One barrier per chunk: the X of chunk c + 1 is
+    // written to the other buffer after the barrier that all readers of chunk c - 1 have passed.
+    // The bounds are the same for every thread of the workgroup.
+    int left = c_hi - c_lo;
+    if (left > 0) {
+        int c = c_lo;
+        load(wa, xa, c);
+        stage(xa, 0);
+        while (left > 2) {
+            load(wb, xb, c + 1);
+            __syncthreads();
+            products(wa, 0);
+            stage(xb, 1);
+            load(wa, xa, c + 2);
+            __syncthreads();
+            products(wb, 1);
+            stage(xa, 0);
+            c += 2;
+            left -= 2;
+        }
+        if (left == 2) {
+            load(wb, xb, c + 1);
+            __syncthreads();
+            products(wa, 0);
+            stage(xb, 1);
+            __syncthreads();
+            products(wb, 1);
+        } else {
+            __syncthreads();
+            products(wa, 0);
+        }
+    }
+    // acc[mb][i]: row 16 mb + r16 of X, weight row n0 + 4 g + i
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = mb * 16 + r16;
+        if (m >= M) continue;
+        float* dst = part + ((size_t)run * M + m) * N + n0 + 4 * g;
+        if (n0 + 4 * g + 3 < N) {
+            *reinterpret_cast<float4*>(dst) = make_float4(acc[mb][0], acc[mb][1], acc[mb][2], acc[mb][3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n0 + 4 * g + i < N) dst[i] = acc[mb][i];
+        }
+    }
+}
+
+// part [ks, M, N] float32: run r holds X[:, r-th run of K] W[:, the same]^T.  K a multiple of
+// 128, N a multiple of 4, 1 <= M <= 64.
+extern "C" int rl_gemm_mid_parts(const void* X, const void* W, float* part, int M, int N, int K,
+                                 int ldx, int ldw, int ks, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return RL_OK;
+    if (M > 64 || K < KSTEP || K % KSTEP || N % 4 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ks < 1 ||
+        ks > K / KSTEP || !part)
+        return RL_ERR_ARG;
+    const int chunks = K / KSTEP, per = (chunks + ks - 1) / ks;
+    if ((per * (ks - 1)) >= chunks) return RL_ERR_ARG;  // every run holds a chunk
+    dim3 grid((N + MW * 16 - 1) / (MW * 16), ks), block(MW * RL_WAVE);
+    const bf16_t* x = (const bf16_t*)X;
+    const bf16_t* w = (const bf16_t*)W;
+    if (M <= 16)
+        hipLaunchKernelGGL((gemm_mid_kernel<1>), grid, block, 0, stream, x, w, part, M, N, K, ldx, ldw, per);
+    else if (M <= 32)
+        hipLaunchKernelGGL((gemm_mid_kernel<2>), grid, block, 0, stream, x, w, part, M, N, K, ldx, ldw, per);
+    else if (M <= 48)
+        hipLaunchKernelGGL((gemm_mid_kernel<3>), grid, block, 0, stream, x, w, part, M, N, K, ldx, ldw, per);
+    else
+        hipLaunchKernelGGL((gemm_mid_kernel<4>), grid, block, 0, stream, x, w, part, M, N, K, ldx, ldw, per);
+    return rl_launch_status();
+}

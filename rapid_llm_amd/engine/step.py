@@ -303,7 +303,7 @@ class ModelRunner:
             logit_rows=part[7],
             block_tables=self.device_cache.tables,
             fed_tokens=self.sampled,
-            defer_products=self.dtype == torch.bfloat16 and meta["num_tokens"] <= ops.SKINNY_MAX_ROWS,
+            defer_products=self.dtype == torch.bfloat16 and meta["num_tokens"] <= ops.MID_MAX_ROWS,
             **meta,
         )
 

@@ -511,6 +511,56 @@ def gemm_bf16_residual(
     return rows, partial
 
 
+MID_MAX_ROWS = 64  # rows up to which a product's runs of K may be left to the norm that follows
+_MID_BLOCK_ROWS = 64  # weight rows per workgroup of the mid-size product
+_MID_TARGET_BLOCKS = 256  # workgroups to reach by cutting K
+_MID_MAX_BLOCKS = 128  # wider matrices than this many workgroups stay with the library
+
+
+def mid_runs(n: int, k: int) -> int:
+    """Runs of K for the mid-size product of an ``[n, k]`` matrix, 0 where it does not apply:
+    enough to put a workgroup on every compute unit, at least four chunks of 128 each."""
+    blocks = -(-n // _MID_BLOCK_ROWS)
+    if k % 128 or n % 4 or blocks > _MID_MAX_BLOCKS:
+        return 0
+    chunks = k // 128
+    ks = max(1, min(_MID_TARGET_BLOCKS // blocks, chunks // 4, 8))
+    while ks > 1 and -(-chunks // ks) * (ks - 1) >= chunks:  # every run holds a chunk
+        ks -= 1
+    return ks
+
+
+def gemm_bf16_parts(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x[M,K] @ w[N,K]^T`` for 17 to 64 rows as float32 runs of K, ``[runs, M, N]``: their sum
+    is the product.  For products whose result goes into the residual: the norm that follows
+    adds the runs (``add_rmsnorm_parts``)."""
+    _need(x, "x", torch.bfloat16)
+    _need(w, "w", torch.bfloat16)
+    m, k = x.shape
+    n = w.shape[0]
+    ks = mid_runs(n, k)
+    if k != w.shape[1] or m > MID_MAX_ROWS or ks < 1:
+        raise KernelError(f"gemm_bf16_parts does not take x {tuple(x.shape)}, w {tuple(w.shape)}")
+    parts = torch.empty((ks, m, n), dtype=torch.float32, device=x.device)
+    _ok(core().rl_gemm_mid_parts(_p(x), _p(w), _p(parts), m, n, k, k, k, ks, _stream()), "rl_gemm_mid_parts")
+    return parts
+
+
+def add_rmsnorm_parts(residual: torch.Tensor, parts: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float) -> None:
+    """``residual += bfloat16(sum of parts)`` in place, ``out = norm(residual) * weight``."""
+    runs, tokens, hidden = parts.shape
+    _need(residual, "residual", torch.float32, (tokens, hidden))
+    _need(parts, "parts", torch.float32)
+    _need(weight, "norm weight", torch.float32, (hidden,))
+    _need(out, "out", torch.bfloat16, (tokens, hidden))
+    _ok(
+        core().rl_add_rmsnorm_parts(
+            _p(residual), _p(parts), runs, _p(weight), _p(out), tokens, hidden, ctypes.c_float(eps), _stream()
+        ),
+        "rl_add_rmsnorm_parts",
+    )
+
+
 def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> torch.Tensor | None:
     """``silu(x Wg^T) * (x Wu^T)`` for the packed ``[gate | up]`` matrix in one kernel, for
     few rows; ``None`` when the shape is not one the fused kernel takes.  ``scaled``: as in

@@ -39,9 +39,22 @@ class Linear:
             and x.shape[0] <= ops.SKINNY_MAX_ROWS and self.in_features % 8 == 0
         )
 
+    def midsize(self, x) -> bool:
+        """Whether ``x`` (more rows than the few-row kernel takes) may run as float32 runs of K
+        that a norm adds (narrow matrices only: the wide ones are faster in the library)."""
+        return (
+            self.weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+            and ops.SKINNY_MAX_ROWS < x.shape[0] <= ops.MID_MAX_ROWS
+            and ops.mid_runs(self.out_features, self.in_features) > 0
+        )
+
+    def partial_sums(self, x: torch.Tensor) -> torch.Tensor:
+        """``[runs, M, out]`` float32 whose sum over the runs is ``x W^T``."""
+        return ops.gemm_bf16_parts(x, self.weight)
+
     def deferred(self, x: torch.Tensor, ctx):
         """The product, or a :class:`DeferredProduct` of it where the step allows it."""
-        if getattr(ctx, "defer_products", False) and isinstance(x, torch.Tensor) and self.skinny(x):
+        if getattr(ctx, "defer_products", False) and isinstance(x, torch.Tensor) and (self.skinny(x) or self.midsize(x)):
             return DeferredProduct(self, x)
         return self(x)
 

@@ -50,6 +50,14 @@ class RMSNorm(Norm):
                 # the producer's kernel adds into the residual and leaves what the consumer's
                 # kernel needs to finish the norm: no kernel of this norm's own runs
                 return delta.linear.add_to_residual(delta.x, residual, self.weight, self.eps)
+            if (
+                rows is None and delta.linear.out_features == self.size and self.dtype == torch.bfloat16
+                and self.size % 4 == 0 and self.size <= 16 * 1024 and delta.linear.midsize(delta.x)
+            ):
+                # the product arrives as float32 runs of K, which this norm's kernel adds
+                out = torch.empty((residual.shape[0], self.size), dtype=self.dtype, device=residual.device)
+                ops.add_rmsnorm_parts(residual, delta.linear.partial_sums(delta.x), self.weight, out, self.eps)
+                return out
             delta = delta.materialize()
         n = residual.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=self.dtype, device=residual.device)

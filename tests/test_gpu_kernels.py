@@ -441,6 +441,47 @@ def test_products_fold_the_norm_between_them(shape):
     assert torch.equal(rows2, rows) and torch.equal(partial2, partial) and torch.equal(res2, res)
 
 
+@pytest.mark.parametrize("shape", [(17, 4096, 4096), (64, 4096, 12288), (33, 200, 256), (48, 1000, 1280), (20, 64, 128)])
+def test_product_in_runs_of_k_and_the_norm_that_adds_them(shape):
+    """17 to 64 rows: the product of a narrow matrix as float32 runs of K, and the norm kernel
+    that adds the runs, against the library product followed by the ordinary norm."""
+    ops = _ops()
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n)
+    x = (torch.randn((m, k), generator=gen)).bfloat16()
+    w = (torch.randn((n, k), generator=gen) * 0.05).bfloat16()
+    assert ops.mid_runs(n, k) >= 1
+    parts = ops.gemm_bf16_parts(x.to(DEV), w.to(DEV))
+    assert parts.shape[1:] == (m, n) and parts.shape[0] == ops.mid_runs(n, k)
+    want = x.float() @ w.float().T
+    torch.testing.assert_close(parts.sum(0).cpu(), want, rtol=2e-3, atol=2e-3 * float(want.abs().max()))
+    # the norm that adds them
+    res = torch.randn((m, n), generator=gen)
+    norm_w = 1 + 0.1 * torch.randn(n, generator=gen)
+    eps = 1e-5
+    got_res = res.to(DEV).clone()
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    ops.add_rmsnorm_parts(got_res, parts, norm_w.to(DEV), out, eps)
+    delta = parts.sum(0).bfloat16().float().cpu()
+    want_res = res + delta
+    torch.testing.assert_close(got_res.cpu(), want_res, rtol=0, atol=2.0 ** -7 * float(delta.abs().max()))
+    want_out = want_res * torch.rsqrt(want_res.pow(2).mean(-1, keepdim=True) + eps) * norm_w
+    torch.testing.assert_close(out.float().cpu(), want_out, rtol=2e-2, atol=2e-2)
+    # the same twice: no order of summation is left to chance
+    res2 = res.to(DEV).clone()
+    out2 = torch.empty_like(out)
+    ops.add_rmsnorm_parts(res2, ops.gemm_bf16_parts(x.to(DEV), w.to(DEV)), norm_w.to(DEV), out2, eps)
+    assert torch.equal(res2, got_res) and torch.equal(out2, out)
+
+
+def test_wide_matrices_stay_with_the_library():
+    ops = _ops()
+    assert ops.mid_runs(24576, 4096) == 0 and ops.mid_runs(151936, 4096) == 0
+    assert ops.mid_runs(4096, 4096) == 4 and ops.mid_runs(4096, 12288) == 4
+    assert ops.mid_runs(4096, 200) == 0  # K must be a multiple of 128
+    assert ops.mid_runs(64, 128) == 1
+
+
 def test_embed_takes_fed_tokens_from_the_sampling_buffer():
     """An id -(r + 1) reads row r of the buffer the sampling kernels write; other ids are
     the rows they name; an id that names no row of either reads row 0 and never faults."""
