@@ -844,27 +844,23 @@ attn_prefill_kernel(
                 for (int c = 0; c < DC; ++c) s[n][hb] = mfma(kf[c], qf[n][c], s[n][hb]);
             }
         }
-        // ---- softmax of 64 keys per row ---------------------------------------------------
+        // ---- softmax of 64 keys per row: maxima first, for both row blocks ---------------------
         bf16x8 p[PF_NQ][2];
+        float m_safe_n[PF_NQ];
 #pragma unroll
         for (int n = 0; n < PF_NQ; ++n) {
-            float x[16];
-#pragma unroll
-            for (int hb = 0; hb < 4; ++hb)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) x[4 * hb + i] = s[n][hb][i];
             if (need_mask) {
                 const int pos = r_pos[n];
                 const int wlo = (window > 0) ? pos - window + 1 : 0;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int key = base + 32 * (e >> 3) + 8 * g + (e & 7);
-                    if (!(key <= pos && key >= wlo)) x[e] = -INFINITY;
+                    if (!(key <= pos && key >= wlo)) s[n][e >> 2][e & 3] = -INFINITY;
                 }
             }
-            float mx = x[0];
+            float mx = s[n][0][0];
 #pragma unroll
-            for (int e = 1; e < 16; ++e) mx = fmaxf(mx, x[e]);
+            for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s[n][e >> 2][e & 3]);
             mx = row_max4(mx) * scale_log2;  // the scale is positive: max commutes with it
             const float m_new = fmaxf(m[n], mx);
             // a row that has seen no visible key yet keeps m = -inf; exp2 of (-inf) - 0 is 0
@@ -881,20 +877,36 @@ attn_prefill_kernel(
                 }
                 m[n] = m_new;
             }
-            float psum = 0.f;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float pe = __builtin_amdgcn_exp2f(fmaf(x[e], scale_log2, -m_safe));
-                psum += pe;
-                p[n][e >> 3][e & 7] = (__bf16)pe;
-            }
-            l[n] += psum;  // per-lane partial sum; the four groups are added at the end
+            m_safe_n[n] = m_safe;
         }
-        // ---- O^T += V^T P^T -------------------------------------------------------------------
+        // ---- the weights of the first 32 keys, then of the last 32; the products follow half by
+        // half, so that the first half's matrix instructions run beside the second half's
+        // exponentials (8,192 tokens: 701 -> 681 us) ---------------------------------------------
+        float psum[PF_NQ];
 #pragma unroll
-        for (int b = 0; b < DB; ++b) {
+        for (int n = 0; n < PF_NQ; ++n) {
+            psum[n] = 0.f;
 #pragma unroll
-            for (int hf = 0; hf < 2; ++hf) {
+            for (int e = 0; e < 8; ++e) {
+                const float pe = __builtin_amdgcn_exp2f(fmaf(s[n][e >> 2][e & 3], scale_log2, -m_safe_n[n]));
+                psum[n] += pe;
+                p[n][0][e] = (__bf16)pe;
+            }
+        }
+#pragma unroll
+        for (int n = 0; n < PF_NQ; ++n) {
+#pragma unroll
+            for (int e = 8; e < 16; ++e) {
+                const float pe = __builtin_amdgcn_exp2f(fmaf(s[n][e >> 2][e & 3], scale_log2, -m_safe_n[n]));
+                psum[n] += pe;
+                p[n][1][e & 7] = (__bf16)pe;
+            }
+            l[n] += psum[n];  // per-lane partial sum; the four groups are added at the end
+        }
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+            for (int b = 0; b < DB; ++b) {
                 const bf16x8 v = load16(&Vs[(16 * b + col) * V_LD + 32 * hf + 8 * g]);
 #pragma unroll
                 for (int n = 0; n < PF_NQ; ++n) acc[n][b] = mfma(v, p[n][hf], acc[n][b]);
