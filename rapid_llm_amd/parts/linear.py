@@ -7,7 +7,9 @@ Which product runs is decided by the weight's storage type:
   checkpoint stores in 32-bit is used at full precision in a bfloat16 engine too.
 * bfloat16 weight: few rows (decode) go to the hand-written bandwidth-bound matrix-core
   kernel; many rows go to the library product, as in the reference, whose dense products
-  are ``F.linear`` (rapid_llm/kernels/ops/gemm/linear.py:17-40).
+  are ``F.linear`` (rapid_llm/kernels/ops/gemm/linear.py:17-40).  In between (17 to 64 rows) a
+  narrow matrix whose result a norm adds to the residual may hand that norm float32 runs of
+  K instead (``partial_sums``).
 """
 
 from __future__ import annotations
