@@ -65,14 +65,15 @@ def test_graph_replays_match_eager(tmp_path, which, dtype):
         r.cache.check_invariants()
 
 
-@pytest.mark.parametrize("batch", [17, 40])
-def test_graph_of_a_batch_beyond_the_skinny_product(tmp_path, batch):
-    """More than 16 rows: the bfloat16 products are the library's.  Their graph replays are
+@pytest.mark.parametrize("which,batch", [("B", 17), ("B", 40), ("E", 23), ("E", 64)])
+def test_graph_of_a_batch_beyond_the_skinny_product(tmp_path, which, batch):
+    """More than 16 rows: the bfloat16 products are the library's, and in configuration E the
+    output and down projections run as runs of K that the norms add.  The graph replays are
     checked one by one against eager steps of a second engine, with eager work between."""
     from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
 
-    cfg, page, seed = TINY["B"]
-    model_dir = make_model_dir(tmp_path, "B", "bfloat16")
+    cfg, page, seed = TINY[which]
+    model_dir = make_model_dir(tmp_path, which, "bfloat16")
     make = lambda graph: ModelRunner(
         model_dir,
         EngineConfig(dtype="bfloat16", max_seq_len=64, page_size=page, num_pages=batch * 4 + 8,

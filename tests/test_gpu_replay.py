@@ -23,6 +23,7 @@ LENGTHS = {
     "B": [22, 37, 51, 84, 110, 170],         # prompts 2/17/31/64/90/150 + 20 decoded
     "C": [9, 33, 48, 77, 130, 201],
     "D": [12, 40, 66, 150, 333, 600],
+    "E": [20, 35, 49, 64, 90, 200],          # portions of 17 to 64 tokens take the mid-size product
 }
 
 
@@ -70,7 +71,7 @@ def _check(got, want, dtype, label):
             raise AssertionError(f"{label}: request {rid}, first wrong position {first}: {exc}") from None
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_every_cut_matches_plain(tmp_path, which, dtype):
     cfg, page, seed = TINY[which]

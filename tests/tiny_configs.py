@@ -47,8 +47,19 @@ TINY_D = dict(
 )
 PAGE_D = 8
 
+# E: widths that are multiples of 128, which the product for 17 to 64 rows needs (the output
+# projection in one run of K, the down projection in two), group 2, head 32, page 8
+TINY_E = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=128, num_attention_heads=4, num_key_value_heads=2,
+    head_dim=32, intermediate_size=1024, vocab_size=277, rope_theta=30000.0,
+    rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=256,
+    hidden_act="silu", attention_bias=False,
+)
+PAGE_E = 8
+
 TINY = {"A": (TINY_A, PAGE_A, 11), "B": (TINY_B, PAGE_B, 22), "C": (TINY_C, PAGE_C, 33),
-        "D": (TINY_D, PAGE_D, 44)}
+        "D": (TINY_D, PAGE_D, 44), "E": (TINY_E, PAGE_E, 55)}
 
 
 def make_model_dir(tmp_path: Path, which: str, dtype: str = "float32") -> Path:
