@@ -1,5 +1,6 @@
 // Bandwidth-bound bfloat16 product for few rows (decode): out[M,N] = X[M,K] * W[N,K]^T with
-// M <= 16, float32 accumulation on the matrix cores, optionally fused with SwiGLU.
+// M <= 16, float32 accumulation on the matrix cores, optionally fused with SwiGLU.  (The last
+// section of the file holds the product for 17 to 64 rows of the narrow matrices.)
 //
 // Every weight byte is read once, in long contiguous runs: a workgroup owns NT tiles of 16
 // weight rows and its 8 waves interleave over K in steps of 128 elements, so that at any
