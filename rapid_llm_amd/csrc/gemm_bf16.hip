@@ -74,7 +74,8 @@ __device__ inline void store_out<bf16_t>(bf16_t* p, float v) {
 // the same bytes 10 / 6.5 / 16 / 34.  Non-temporal loads, more waves, K split over workgroups
 // and staggered K offsets did not help.  Two chunks in flight per wave, in two sets of
 // registers (see the main loop), then gave 14.0 / 9.4 / 21.9 / 38.4 where one chunk at a time
-// gave 14.9 / 9.7 / 22.2 / 42.6 in the same run.
+// gave 14.9 / 9.7 / 22.2 / 42.6 in the same run; four chunks in flight (where a compute unit holds
+// one workgroup anyway) were no faster than two (9.8 against 9.3, 22.1 against 21.9).
 // sum over the four lanes l, l + 16, l + 32, l + 48 (two lane swaps of gfx950), left in all four
 __device__ inline float sum_rows_of_16(float v) {
     const unsigned u = __float_as_uint(v);
