@@ -172,6 +172,30 @@ def test_bfloat16_generation_stays_near_the_plain_choice(tmp_path, which):
             assert len(out.token_ids) == 16
 
 
+def test_bfloat16_generation_of_forty_requests_at_once(tmp_path):
+    """Decode batches between 17 and 64 rows (configuration E: the output and down projections
+    then run as runs of K added by the norms), with and without graphs."""
+    from rapid_llm_amd import SamplingParams
+
+    cfg, page, seed = TINY["E"]
+    model_dir = make_model_dir(tmp_path, "E", "bfloat16")
+    pcfg, pw = plain_load(model_dir)
+    prompts = [random_tokens(2 + (7 * i) % 23, cfg["vocab_size"], seed + i) for i in range(40)]
+    for graph in (False, True):
+        llm = _llm(model_dir, "bfloat16", page, max_seq_len=64, max_num_seqs=48, num_pages=48 * 8 + 8,
+                   use_cuda_graph=graph)
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_gen_len=6))
+        for prompt, out in zip(prompts, outs):
+            ids = list(prompt)
+            for tok in out.token_ids:
+                logits = plain_forward(pcfg, pw, ids)[-1]
+                assert float(logits.max() - logits[tok]) < 0.05, graph
+                ids.append(tok)
+            assert len(out.token_ids) == 6
+        if graph:
+            assert any(17 <= key[0] <= 64 for key in llm.scheduler.runner._graphs)
+
+
 def test_stop_tokens_and_stream(tmp_path):
     from rapid_llm_amd import LLM, SamplingParams
 
