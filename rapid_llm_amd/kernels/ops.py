@@ -495,7 +495,10 @@ def gemm_bf16_residual(
     m, k = x.shape
     n = w.shape[0]
     if k != w.shape[1] or m > SKINNY_MAX_ROWS or k % 8:
-        raise KernelError(f"gemm_bf16_residual takes up to {SKINNY_MAX_ROWS} rows over a multiple of 8: x {tuple(x.shape)}, w {tuple(w.shape)}")
+        raise KernelError(
+            f"gemm_bf16_residual takes up to {SKINNY_MAX_ROWS} rows over a multiple of 8: "
+            f"x {tuple(x.shape)}, w {tuple(w.shape)}"
+        )
     _need(residual, "residual", torch.float32, (m, n))
     _need(norm_weight, "norm weight", torch.float32, (n,))
     lib = core()
@@ -546,7 +549,9 @@ def gemm_bf16_parts(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return parts
 
 
-def add_rmsnorm_parts(residual: torch.Tensor, parts: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float) -> None:
+def add_rmsnorm_parts(
+    residual: torch.Tensor, parts: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float
+) -> None:
     """``residual += bfloat16(sum of parts)`` in place, ``out = norm(residual) * weight``."""
     runs, tokens, hidden = parts.shape
     _need(residual, "residual", torch.float32, (tokens, hidden))

@@ -56,11 +56,14 @@ class Linear:
 
     def deferred(self, x: torch.Tensor, ctx):
         """The product, or a :class:`DeferredProduct` of it where the step allows it."""
-        if getattr(ctx, "defer_products", False) and isinstance(x, torch.Tensor) and (self.skinny(x) or self.midsize(x)):
+        allowed = getattr(ctx, "defer_products", False) and isinstance(x, torch.Tensor)
+        if allowed and (self.skinny(x) or self.midsize(x)):
             return DeferredProduct(self, x)
         return self(x)
 
-    def add_to_residual(self, x: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> ScaledRows:
+    def add_to_residual(
+        self, x: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float
+    ) -> ScaledRows:
         """``residual += x W^T`` in place; returns the new rows times ``norm_weight`` and the
         pieces of their sums of squares."""
         rows, partial = ops.gemm_bf16_residual(x, self.weight, residual, norm_weight)
