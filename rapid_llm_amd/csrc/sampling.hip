@@ -165,10 +165,19 @@ extern "C" int rl_argmax(const float* logits, const int* row_index, int* out, fl
 //
 // Per-row parameters, 8 int32 words: temperature, top_p, penalty (float bits), seed low,
 // seed high, counter, first and one-past-last index of its generated tokens in `history`.
+// A negative entry -(r + 1) of the history stands for a token the host has not read yet:
+// what sampling row r of the step before chose, kept in `fed` [fed_rows].  `fed` must not
+// be the buffer this launch writes its own choices to.
 // --------------------------------------------------------------------------- //
 #define SMP_THREADS 1024
 #define SMP_WAVES (SMP_THREADS / RL_WAVE)
 #define SMP_POOL 1024  // candidates of nucleus sampling (rapid_llm/engine/sampler.py:186)
+
+__device__ inline int history_token(int tok, const int* __restrict__ fed, int fed_rows) {
+    if (tok >= 0) return tok;
+    const int r = -tok - 1;
+    return (fed && r < fed_rows) ? fed[r] : -1;
+}
 
 __device__ inline uint32_t float_key(float v) {
     // order-preserving map float -> uint32 (NaN sorts lowest)
@@ -204,7 +213,8 @@ __device__ inline float wave_inclusive_scan(float v) {
 
 __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float* __restrict__ logits, const int* __restrict__ row_index,
-    const int* __restrict__ row_params, const int* __restrict__ history, int* __restrict__ out,
+    const int* __restrict__ row_params, const int* __restrict__ history,
+    const int* __restrict__ fed, int fed_rows, int* __restrict__ out,
     float* __restrict__ out_logprob, int vocab, int bitmap_words) {
     extern __shared__ uint32_t seen[];  // one bit per token id, when the row has a penalty
     __shared__ unsigned long long cand[SMP_POOL];
@@ -232,7 +242,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
         for (int i = tid; i < bitmap_words; i += SMP_THREADS) seen[i] = 0u;
         __syncthreads();
         for (int i = rp[6] + tid; i < rp[7]; i += SMP_THREADS) {
-            const int tok = history[i];
+            const int tok = history_token(history[i], fed, fed_rows);
             if (tok >= 0 && tok < vocab) atomicOr(&seen[tok >> 5], 1u << (tok & 31));
         }
         __syncthreads();
@@ -475,11 +485,13 @@ extern "C" float rl_sample_uniform(unsigned int seed_lo, unsigned int seed_hi,
 
 extern "C" int rl_sample_pool() { return SMP_POOL; }
 
-// history may be null when no row has a penalty.  out_logprob (optional): log-probability
-// of the chosen token under the penalised, temperature-scaled distribution.
+// history may be null when no row has a penalty, fed when the history names no row of the
+// step before.  out_logprob (optional): log-probability of the chosen token under the
+// penalised, temperature-scaled distribution.
 extern "C" int rl_sample(const float* logits, const int* row_index, const int* row_params,
-                         const int* history, int* out, float* out_logprob, int rows, int vocab,
-                         int any_penalty, hipStream_t stream) {
+                         const int* history, const int* fed, int fed_rows, int* out,
+                         float* out_logprob, int rows, int vocab, int any_penalty,
+                         hipStream_t stream) {
     if (rows <= 0) return RL_OK;
     if (vocab < 1) return RL_ERR_ARG;
     int words = 0;
@@ -488,8 +500,10 @@ extern "C" int rl_sample(const float* logits, const int* row_index, const int* r
         if ((size_t)words * 4 > 40 * 1024) return RL_ERR_ARG;  // the bitmap lives in LDS
         if (!history) return RL_ERR_ARG;
     }
+    if (fed && (fed == out || fed_rows < 0)) return RL_ERR_ARG;
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), (size_t)words * 4, stream,
-                       logits, row_index, row_params, history, out, out_logprob, vocab, words);
+                       logits, row_index, row_params, history, fed, fed_rows, out, out_logprob, vocab,
+                       words);
     return rl_launch_status();
 }
 
@@ -509,6 +523,7 @@ extern "C" int rl_sample(const float* logits, const int* row_index, const int* r
 __global__ __launch_bounds__(SMP_THREADS) void logprobs_kernel(
     const float* __restrict__ logits, const int* __restrict__ row_index,
     const int* __restrict__ row_params, const int* __restrict__ history,
+    const int* __restrict__ fed, int fed_rows,
     const int* __restrict__ targets, float* __restrict__ out_target, int* __restrict__ out_top_ids,
     float* __restrict__ out_top_lp, int vocab, int k, int bitmap_words) {
     extern __shared__ uint32_t seen[];
@@ -529,7 +544,7 @@ __global__ __launch_bounds__(SMP_THREADS) void logprobs_kernel(
         for (int i = tid; i < bitmap_words; i += SMP_THREADS) seen[i] = 0u;
         __syncthreads();
         for (int i = rp[6] + tid; i < rp[7]; i += SMP_THREADS) {
-            const int tok = history[i];
+            const int tok = history_token(history[i], fed, fed_rows);
             if (tok >= 0 && tok < vocab) atomicOr(&seen[tok >> 5], 1u << (tok & 31));
         }
         __syncthreads();
@@ -614,9 +629,10 @@ __global__ __launch_bounds__(SMP_THREADS) void logprobs_kernel(
 
 // targets [rows]: the token whose log-probability goes to out_target [rows] (NaN for an id
 // outside the vocabulary).  out_top_ids / out_top_lp [rows, k]; k may be 0.  row_params and
-// history as for rl_sample, or null for the raw distribution.
+// history and fed as for rl_sample, or null for the raw distribution.
 extern "C" int rl_logprobs(const float* logits, const int* row_index, const int* row_params,
-                           const int* history, const int* targets, float* out_target,
+                           const int* history, const int* fed, int fed_rows,
+                           const int* targets, float* out_target,
                            int* out_top_ids, float* out_top_lp, int rows, int vocab, int k,
                            int any_penalty, hipStream_t stream) {
     if (rows <= 0) return RL_OK;
@@ -628,8 +644,10 @@ extern "C" int rl_logprobs(const float* logits, const int* row_index, const int*
         if ((size_t)words * 4 > 40 * 1024) return RL_ERR_ARG;
         if (!history || !row_params) return RL_ERR_ARG;
     }
+    if (fed && fed_rows < 0) return RL_ERR_ARG;
     hipLaunchKernelGGL(logprobs_kernel, dim3(rows), dim3(SMP_THREADS), (size_t)words * 4, stream,
-                       logits, row_index, row_params, history, targets, out_target, out_top_ids,
+                       logits, row_index, row_params, history, fed, fed_rows, targets, out_target,
+                       out_top_ids,
                        out_top_lp, vocab, k, words);
     return rl_launch_status();
 }

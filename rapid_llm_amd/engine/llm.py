@@ -83,8 +83,15 @@ class GpuExecutor:
         runner = self.runner
         logits = runner.step(entries)
         in_order = sampling.logits_rows == list(range(logits.shape[0]))
+        fed = None
+        if any(r.repetition_penalty != 1.0 and any(t < 0 for t in r.generated[-1:]) for r in sampling.rows):
+            # a penalised row's newest token is still on the device, among the choices that
+            # this step's sampling is about to overwrite
+            fed = runner.sampled_before
+            fed.copy_(runner.sampled)
         ids, _ = self.sampler.sample(
-            logits, sampling.rows, row_index=None if in_order else sampling.logits_rows, out=runner.sampled
+            logits, sampling.rows, row_index=None if in_order else sampling.logits_rows, out=runner.sampled,
+            fed=fed,
         )
         host = {"ids": self._to_host(ids)}
         asked = [b for b, k in enumerate(sampling.logprob_ks) if k is not None]
@@ -96,6 +103,7 @@ class GpuExecutor:
                 max(sampling.logprob_ks[b] for b in asked),
                 rows=[sampling.rows[b] for b in asked],
                 row_index=[sampling.logits_rows[b] for b in asked],
+                fed=fed,
             )
             host.update(lp=self._to_host(lp), top_ids=self._to_host(top_ids), top_lp=self._to_host(top_lp))
         if sampling.prompt_rows:

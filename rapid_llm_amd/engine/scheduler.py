@@ -38,9 +38,9 @@ harvest: it counts in the request's length, and step N + 1 feeds it from the dev
 one more step, whose token is discarded, and its slot and pages are given back after that
 step.  Nobody is evicted or ended for want of pages on a guess: when pages are short, the
 step in flight is read first and the decision made on what is then known.  The tokens are
-those of the synchronous loop.  A step is run synchronously (harvest
-before planning) while a live request has a repetition penalty, whose history must hold the
-newest token.
+those of the synchronous loop, with a repetition penalty too: the history of a request whose
+newest token is pending names that token by its sampling row, and the sampling kernels read
+it on the device.
 """
 
 from __future__ import annotations
@@ -56,6 +56,7 @@ from ..config.engine_config import EngineConfig
 from ..sampling.logprobs import PositionLogprobs
 from ..sampling.params import SamplingParams
 from ..sampling.rng import derive_seed
+from .feed import fed_token
 from .request import Request, RequestStatus
 
 # Output tokens of a request between checks of the repetition breaker.  The reference polls
@@ -424,7 +425,7 @@ class Scheduler:
         """Plan one batch, run it, harvest chosen tokens.  Returns the requests that advanced
         or finished (rapid_llm/engine/scheduler.py:1405-1460).  Pipelined, the tokens harvested
         are those of the step queued by the previous call (:818-933)."""
-        if self.pipeline and self._can_pipeline():
+        if self.pipeline:
             try:
                 launched, advanced = self._launch()
             except _ReadFirst:
@@ -449,11 +450,15 @@ class Scheduler:
             advanced += self._harvest(launched)
         return advanced
 
-    def _can_pipeline(self) -> bool:
-        # the penalty reads the request's newest token from the host's list
-        return all(
-            r.params.repetition_penalty == 1.0 for r in itertools.chain(self.running, self.waiting)
-        )
+    @staticmethod
+    def _penalised_tokens(request: Request) -> Sequence[int]:
+        """The generated tokens a repetition penalty applies to; the one still on the device is
+        named by the sampling row that chose it."""
+        if request.params.repetition_penalty == 1.0:
+            return ()
+        if request.pending:
+            return [*request.output_token_ids, fed_token(request.pending_row)]
+        return request.output_token_ids
 
     def _launch(self) -> tuple["_Inflight | None", list[Request]]:
         """Plan a step and queue it; returns what is in flight and the requests the planner
@@ -496,7 +501,7 @@ class Scheduler:
                         repetition_penalty=p.repetition_penalty,
                         seed=r.seed,
                         counter=len(r.output_token_ids) + r.pending,
-                        generated=r.output_token_ids if p.repetition_penalty != 1.0 else (),
+                        generated=self._penalised_tokens(r),
                     )
                 )
                 sampling.logits_rows.append(num_rows + len(want))

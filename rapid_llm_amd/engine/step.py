@@ -157,6 +157,9 @@ class ModelRunner:
         # where the sampling kernels leave their choices, one row per sampled request of a
         # step; the next step's embedding reads fed tokens from here
         self.sampled = torch.zeros(max(1, self.engine.max_num_seqs), dtype=torch.int32, device=self.device)
+        # the choices of the step before, kept aside while a step's sampling kernels overwrite
+        # ``sampled``: a penalised row reads its own newest token from here
+        self.sampled_before = torch.zeros_like(self.sampled)
 
     # ------------------------------------------------------------------ sizing
     def _decide_num_pages(self, groups) -> int:

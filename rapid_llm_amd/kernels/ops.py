@@ -335,6 +335,21 @@ def _penalty_fits(vocab: int) -> None:
         )
 
 
+def _fed_tokens(fed: Optional[torch.Tensor], out: Optional[torch.Tensor]) -> None:
+    if fed is None:
+        return
+    _need(fed, "fed", torch.int32)
+    if fed.dim() != 1:
+        raise KernelError(f"fed tokens must be one-dimensional, are {tuple(fed.shape)}")
+    if out is not None and _overlap(fed, out):
+        raise KernelError("the fed tokens share memory with the tokens this call chooses")
+
+
+def _overlap(a: torch.Tensor, b: torch.Tensor) -> bool:
+    a0, b0 = a.data_ptr(), b.data_ptr()
+    return a0 < b0 + b.numel() * b.element_size() and b0 < a0 + a.numel() * a.element_size()
+
+
 def sample(
     logits: torch.Tensor,
     row_params: torch.Tensor,
@@ -343,10 +358,13 @@ def sample(
     out_logprob: Optional[torch.Tensor],
     any_penalty: bool,
     row_index: Optional[torch.Tensor] = None,
+    fed: Optional[torch.Tensor] = None,
 ) -> None:
     """General token selection (penalty, temperature, nucleus, seeded draw), one row per
     workgroup.  ``row_params [rows * 8]`` int32 as the kernel documents them; output row
-    ``b`` reads row ``row_index[b]`` of ``logits`` (row ``b`` without an index)."""
+    ``b`` reads row ``row_index[b]`` of ``logits`` (row ``b`` without an index).  A negative
+    entry ``-(r + 1)`` of ``history`` is read as ``fed[r]``; ``fed`` must not share memory
+    with ``out``."""
     vocab = logits.shape[1]
     rows = out.shape[0]
     _need(logits, "logits", torch.float32)
@@ -361,10 +379,12 @@ def sample(
         _need(history, "history", torch.int32)
     if any_penalty:
         _penalty_fits(vocab)
+    _fed_tokens(fed, out)
     _ok(
         core().rl_sample(
-            _p(logits), _p(row_index), _p(row_params), _p(history), _p(out), _p(out_logprob), rows,
-            vocab, int(bool(any_penalty)), _stream(),
+            _p(logits), _p(row_index), _p(row_params), _p(history), _p(fed),
+            0 if fed is None else fed.shape[0], _p(out), _p(out_logprob), rows, vocab,
+            int(bool(any_penalty)), _stream(),
         ),
         "rl_sample",
     )
@@ -378,12 +398,13 @@ def logprobs(
     history: Optional[torch.Tensor] = None,
     any_penalty: bool = False,
     row_index: Optional[torch.Tensor] = None,
+    fed: Optional[torch.Tensor] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Log-probability of ``targets[b]`` and the ``k`` most likely tokens of every row:
     ``(target [rows] float32, top ids [rows, k] int32, top log-probabilities [rows, k]
     float32)``, descending, equal values by ascending id.  With ``row_params`` the
     distribution is the one ``sample`` draws from (penalty, temperature; greedy rows count
-    as temperature 1); without, log_softmax of the raw logits."""
+    as temperature 1); without, log_softmax of the raw logits.  ``fed`` as for ``sample``."""
     vocab = logits.shape[1]
     rows = targets.shape[0]
     _need(logits, "logits", torch.float32)
@@ -401,12 +422,14 @@ def logprobs(
         _penalty_fits(vocab)
         if row_params is None or history is None:
             raise KernelError("a penalty needs row_params and history")
+    _fed_tokens(fed, None)
     target_lp = torch.empty(rows, dtype=torch.float32, device=logits.device)
     top_ids = torch.empty((rows, k), dtype=torch.int32, device=logits.device)
     top_lp = torch.empty((rows, k), dtype=torch.float32, device=logits.device)
     _ok(
         core().rl_logprobs(
-            _p(logits), _p(row_index), _p(row_params), _p(history), _p(targets), _p(target_lp),
+            _p(logits), _p(row_index), _p(row_params), _p(history), _p(fed),
+            0 if fed is None else fed.shape[0], _p(targets), _p(target_lp),
             _p(top_ids if k else None), _p(top_lp if k else None), rows, vocab, k,
             int(bool(any_penalty)), _stream(),
         ),

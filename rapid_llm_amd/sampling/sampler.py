@@ -29,12 +29,15 @@ class RowSampling:
     repetition_penalty: float = 1.0
     seed: int = 0
     counter: int = 0  # tokens the request has generated so far
-    generated: Sequence[int] = field(default_factory=tuple)  # read when the penalty is on
+    # read when the penalty is on; -(r + 1) names what sampling row r of the step before
+    # chose, for a token the host has not read back yet
+    generated: Sequence[int] = field(default_factory=tuple)
 
 
-def _pack_rows(rows: Sequence[RowSampling]) -> tuple[np.ndarray, int, bool]:
+def _pack_rows(rows: Sequence[RowSampling], fed_rows: int = 0) -> tuple[np.ndarray, int, bool, bool]:
     """The kernels' per-row parameter words followed by the rows' generated tokens:
-    ``(packed int32, words of parameters, whether any row is penalised)``."""
+    ``(packed int32, words of parameters, whether any row is penalised, whether a history
+    names a row of the step before)``; ``fed_rows`` is how many such rows there are."""
     n = len(rows)
     params = np.zeros((n, 8), dtype=np.int32)
     fl = params.view(np.float32)
@@ -54,8 +57,13 @@ def _pack_rows(rows: Sequence[RowSampling]) -> tuple[np.ndarray, int, bool]:
             history.extend(int(t) for t in r.generated)
             any_penalty = True
         params[i, 7] = len(history)
-    packed = np.concatenate([params.reshape(-1), np.asarray(history, dtype=np.int32)])
-    return packed, 8 * n, any_penalty
+    tokens = np.asarray(history, dtype=np.int32)
+    names_rows = bool(tokens.size) and int(tokens.min()) < 0
+    if names_rows and int(tokens.min()) < -fed_rows:
+        raise ValueError(
+            f"a history names sampling row {-int(tokens.min()) - 1} of the step before, which left {fed_rows}"
+        )
+    return np.concatenate([params.reshape(-1), tokens]), 8 * n, any_penalty, names_rows
 
 
 class Sampler:
@@ -74,12 +82,15 @@ class Sampler:
         want_logprobs: bool = False,
         row_index: Sequence[int] | None = None,
         out: torch.Tensor | None = None,
+        fed: torch.Tensor | None = None,
     ) -> tuple[torch.Tensor, torch.Tensor | None]:
         """``logits [R, vocab]`` float32 -> chosen ids ``[n]`` int32 (on the device) and,
         if asked, the chosen tokens' log-probabilities ``[n]`` float32.  Sampling row ``b``
         reads row ``row_index[b]`` of the logits; without an index there is one sampling
         row per row of logits, in order.  ``out`` (int32, at least ``n`` long) receives the
-        ids in place of a new tensor.  Nothing here waits for the device."""
+        ids in place of a new tensor.  ``fed`` (int32) holds the choices of the step before,
+        for the histories that name its rows; it is not ``out``.  Nothing here waits for the
+        device."""
         n = len(rows)
         reads = len(row_index) if row_index is not None else logits.shape[0]
         if n != reads:
@@ -97,11 +108,12 @@ class Sampler:
         if plain and not want_logprobs:
             ops.argmax(logits, out, index)
             return out, None
-        packed, words, any_penalty = _pack_rows(rows)
+        packed, words, any_penalty, names_rows = _pack_rows(rows, 0 if fed is None else fed.numel())
         dev = upload(packed, self.device)
         logprob = torch.empty(n, dtype=torch.float32, device=self.device) if want_logprobs else None
         ops.sample(
-            logits, dev[:words], dev[words:] if any_penalty else None, out, logprob, any_penalty, index
+            logits, dev[:words], dev[words:] if any_penalty else None, out, logprob, any_penalty, index,
+            fed if names_rows else None,
         )
         return out, logprob
 
@@ -112,6 +124,7 @@ class Sampler:
         k: int,
         rows: Sequence[RowSampling] | None = None,
         row_index: Sequence[int] | None = None,
+        fed: torch.Tensor | None = None,
     ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         """Log-probability of ``targets[b]`` and the ``k`` most likely tokens, on the device:
         ``(target [n], top ids [n, k], top log-probabilities [n, k])``.
@@ -130,10 +143,11 @@ class Sampler:
         index = self._index(row_index)
         if rows is None:
             return ops.logprobs(logits, targets, k, row_index=index)
-        packed, words, any_penalty = _pack_rows(rows)
+        packed, words, any_penalty, names_rows = _pack_rows(rows, 0 if fed is None else fed.numel())
         dev = upload(packed, self.device)
         return ops.logprobs(
-            logits, targets, k, dev[:words], dev[words:] if any_penalty else None, any_penalty, index
+            logits, targets, k, dev[:words], dev[words:] if any_penalty else None, any_penalty, index,
+            fed if names_rows else None,
         )
 
 

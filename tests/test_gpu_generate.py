@@ -259,6 +259,47 @@ def test_pipeline_gives_the_tokens_of_the_synchronous_loop(tmp_path, dtype, grap
                 assert [r.token_id for r in a.outputs[0].logprobs] == [r.token_id for r in b.outputs[0].logprobs]
 
 
+def test_a_repetition_penalty_rides_the_pipeline(tmp_path):
+    """With a penalty the newest token of a request is part of what the next choice depends
+    on; pipelined, that token is still on the device.  Tokens and records are those of the
+    synchronous loop and of the plain model and sampler, with ample pages and with few."""
+    from rapid_llm_amd import SamplingParams
+
+    cfg, page, seed = TINY["A"]
+    model_dir = make_model_dir(tmp_path, "A", "float32")
+    cfg, w = plain_load(model_dir)
+    prompts = [random_tokens(n, cfg["vocab_size"], seed + 3 * n) for n in (5, 21, 2, 13, 30)]
+    params = [SamplingParams(temperature=0.0 if i % 2 == 0 else 0.9, top_p=0.95, max_gen_len=10 + 3 * i, seed=i,
+                             repetition_penalty=1.0 if i == 3 else 6.0 + 0.5 * i, stop_on_repeat=False,
+                             logprobs=2 if i == 0 else None)
+              for i in range(len(prompts))]
+    common = dict(max_seq_len=128, max_chunk_size=16, max_num_batched_tokens=40, max_num_seqs=4,
+                  use_cuda_graph=False)
+    outs = {}
+    for pipeline in (False, True):
+        for pages in (200, 18):  # 17 pages of 4: the longest request alone fits, four together do not
+            llm = _llm(model_dir, "float32", page, pipeline=pipeline, num_pages=pages, **common)
+            outs[pipeline, pages] = llm.generate(prompts, params)
+            assert not llm.scheduler.cache.live_requests() and not llm.scheduler._held
+            if pages == 18:
+                assert llm.scheduler.num_preemptions > 0
+    base = outs[False, 200]
+    for prompt, p, o in zip(prompts, params, base):
+        if p.temperature == 0.0:  # a sampled row may sit within rounding of another token
+            want = _plain_generate(cfg, w, prompt, p.max_gen_len, penalty=p.repetition_penalty)
+            assert o.token_ids == want
+            if p.repetition_penalty > 1.0:
+                assert len(set(want)) > len(want) // 2, "the penalty changed nothing to see"
+    greedy_free = _plain_generate(cfg, w, prompts[0], params[0].max_gen_len)
+    assert greedy_free != base[0].token_ids, "the penalty made no difference to the tokens"
+    for key, got in outs.items():
+        for a, b in zip(base, got):
+            assert a.token_ids == b.token_ids, key
+            if a.outputs[0].logprobs is not None:
+                assert [(r.token_id, r.top_token_ids) for r in a.outputs[0].logprobs] == \
+                       [(r.token_id, r.top_token_ids) for r in b.outputs[0].logprobs], key
+
+
 def test_command_line_batch(tmp_path, capsys):
     from rapid_llm_amd.cli import main
 

@@ -203,3 +203,42 @@ def test_sampling_through_a_row_index():
     picked, _ = sampler.sample(logits, rows, row_index=index)
     direct, _ = sampler.sample(logits[index].contiguous(), rows)
     assert picked.tolist() == direct.tolist()
+
+
+def test_a_history_may_name_tokens_still_on_the_device():
+    """A history entry -(r + 1) is read as row r of the choices of the step before: the chosen
+    tokens and the records are those of the history written out; a row beyond that buffer and
+    a buffer that this call overwrites are refused."""
+    from rapid_llm_amd.kernels.ops import KernelError
+
+    sampler, Row = _sampler()
+    gen = torch.Generator().manual_seed(11)
+    vocab = 5003
+    logits = (torch.randn(4, vocab, generator=gen) * 0.05)
+    before = [17, 4000, 2, 911, 77]  # what five rows of the step before chose
+    for i, tok in enumerate(before[:4]):
+        logits[i, tok] = 6.0  # without the penalty each row would choose its own newest token
+        logits[i, 100 + i] = 5.0  # with it, the runner-up
+    logits = logits.cuda()
+    fed = torch.tensor(before, dtype=torch.int32, device="cuda")
+    named = [[30, 31, -3], [-2], [5, 6, 7, 8, -1], [-4]]
+    written = [[30, 31, before[2]], [before[1]], [5, 6, 7, 8, before[0]], [before[3]]]
+    index = [2, 1, 0, 3]  # sampling row b reads the logits row whose favourite its history names
+    kinds = [dict(temperature=0.0), dict(temperature=0.7, top_p=0.9, seed=5, counter=3),
+             dict(temperature=0.0), dict(temperature=1.3, seed=9, counter=1)]
+    rows_named = [Row(repetition_penalty=4.0, generated=g, **k) for g, k in zip(named, kinds)]
+    rows_written = [Row(repetition_penalty=4.0, generated=g, **k) for g, k in zip(written, kinds)]
+    got, got_lp = sampler.sample(logits, rows_named, want_logprobs=True, row_index=index, fed=fed)
+    want, want_lp = sampler.sample(logits, rows_written, want_logprobs=True, row_index=index)
+    assert got.tolist() == want.tolist()
+    assert got.tolist()[0] == 102 and got.tolist()[2] == 100  # the greedy rows: the runner-up
+    assert torch.equal(got_lp, want_lp)
+    a = sampler.logprobs(logits, got, 3, rows=rows_named, row_index=index, fed=fed)
+    b = sampler.logprobs(logits, want, 3, rows=rows_written, row_index=index)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    with pytest.raises(ValueError, match="names sampling row 5"):
+        sampler.sample(logits, [Row(repetition_penalty=2.0, generated=[-6])] * 4, fed=fed)
+    with pytest.raises(ValueError, match="names sampling row 0"):
+        sampler.sample(logits, [Row(repetition_penalty=2.0, generated=[-1])] * 4)
+    with pytest.raises(KernelError, match="share memory"):
+        sampler.sample(logits, rows_named, row_index=index, out=fed, fed=fed)

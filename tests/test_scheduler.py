@@ -3,6 +3,8 @@
 The pattern is the reference's ``_ScriptedExecutor`` (tests/engine/test_scheduler.py:46-74,
 tests/engine/test_batch_planner.py:156-610)."""
 
+import dataclasses
+
 import pytest
 
 from rapid_llm_amd.cache import CacheManager, GroupSpec
@@ -17,7 +19,9 @@ EOS = 99
 
 class ScriptedExecutor:
     """Checks that every step is runnable from what the plan reserved, records its shape,
-    and "samples" token ``f(request, index of the output token)``."""
+    and "samples" token ``f(request, index of the output token)``; a row with a repetition
+    penalty takes the next id that its history does not hold, so its tokens depend on all
+    the tokens before."""
 
     def __init__(self, num_pages, page, seqs, max_len, window=0, token=None):
         self.cache = CacheManager([GroupSpec(0, window, (0,))], num_pages, page, seqs, max_len)
@@ -42,7 +46,13 @@ class ScriptedExecutor:
             self.wants.append((e.request_id, start, len(e.tokens), list(e.want)))
             if e.want and k < len(rows) and sampling.logits_rows[k] == num_rows + len(e.want) - 1:
                 assert e.want[-1] == len(e.tokens) - 1
-                out.append(self.token(e.request_id, rows[k].counter))
+                token = self.token(e.request_id, rows[k].counter)
+                if rows[k].repetition_penalty != 1.0:
+                    assert len(rows[k].generated) == rows[k].counter, "the history misses a token"
+                    assert min(rows[k].generated, default=0) >= 0, "a history token nobody resolved"
+                    while token != EOS and token in rows[k].generated:
+                        token = (token + 1) % 50
+                out.append(token)
                 k += 1
             num_rows += len(e.want)
         assert k == len(rows)
@@ -94,9 +104,7 @@ class PipelinedExecutor(ScriptedExecutor):
             for i, t in enumerate(tokens):
                 assert self.history.setdefault((e.request_id, start + i), t) == t, "a position changed its token"
             resolved.append(type(e)(e.request_id, tokens, e.want))
-        result = self.execute(resolved, sampling)
-        rids = [e.request_id for e, n in zip(entries, [len(e.want) for e in entries])
-                if e.want and e.want[-1] == len(e.tokens) - 1]
+        # a penalised row's history may name its newest token the same way
         sampled_rids = []
         num_rows, k = 0, 0
         for e in entries:
@@ -104,6 +112,17 @@ class PipelinedExecutor(ScriptedExecutor):
                 sampled_rids.append(e.request_id)
                 k += 1
             num_rows += len(e.want)
+        rows = []
+        for rid, row in zip(sampled_rids, sampling.rows):
+            history = list(row.generated)
+            assert all(t >= 0 for t in history[:-1]), "only the newest token can be pending"
+            if history and history[-1] < 0:
+                owner, token = self.previous[fed_row(history[-1])]
+                assert owner == rid, "a history names another request's row"
+                history[-1] = token
+            rows.append(dataclasses.replace(row, generated=history))
+        sampling = dataclasses.replace(sampling, rows=rows)
+        result = self.execute(resolved, sampling)
         self.previous = list(zip(sampled_rids, result.token_ids))
         self.unread += 1
         self.max_unread = max(self.max_unread, self.unread)
@@ -504,16 +523,23 @@ def test_pipeline_ends_by_count_cost_no_extra_step():
     assert r.seq_len == 8 and r.finish_reason == "length" and len(ex.steps) == 3
 
 
-def test_a_penalty_falls_back_to_the_synchronous_loop():
+@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("pool", [200, 17])
+def test_a_penalty_rides_the_pipeline(seed, pool):
+    """A penalised request's history names the token still on the device by its sampling row;
+    the tokens, which depend on the whole history, are those of the synchronous loop."""
     outcomes = []
     for pipeline in (False, True):
-        s, ex = _make_pipelined(pipeline=pipeline, seqs=3, token=_token_with_stops)
-        requests = _workload(s, 3, penalty=True)
+        s, ex = _make_pipelined(num_pages=pool, pipeline=pipeline, seqs=3, max_len=64, token=_token_with_stops,
+                                max_num_batched_tokens=24, max_chunk_size=8)
+        requests = _workload(s, seed, penalty=True)
         while s.has_unfinished_requests():
             s.step()
+        assert ex.max_unread == (2 if pipeline else 1)
         outcomes.append([(r.output_token_ids, r.finish_reason) for r in requests])
         assert not ex.cache.live_requests()
     assert outcomes[0] == outcomes[1]
+    assert any(len(set(out)) == len(out) > 8 for out, _ in outcomes[0]), "no penalised request ran long"
 
 
 def test_abort_while_a_step_is_in_flight():
