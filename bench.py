@@ -1,6 +1,7 @@
 """Decode and prefill speed of the engine on one MI355X, random weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16]
+                    [--shape NAME] [--batch B] [--prompt-len T] [--context C]
 
 A "step" is one decode step of the whole batch through the engine's step function and the
 greedy sampling kernel, tokens fed back.  The default run has the layer sizes of
@@ -8,7 +9,9 @@ Qwen3-8B (BASELINE.json ``configs[2]``), a batch of 8, every request with a 2,04
 prompt, context 4,096.  One JSON line is printed: decoded tokens a second (``value``), the
 2,048-token prefill (``prefill``), the decode step against the HBM roofline (``roofline``)
 and decoding at batch 1 and 64 (``points``, which also holds the true 32-bit path's decode
-and prefill speed, measured in a second process).
+and prefill speed, measured in a second process).  ``--shape``, ``--prompt-len`` and
+``--context`` measure the same at other sizes of the model family and other lengths; the
+line then names them in ``metric`` and ``config``.
 
 Metric definitions follow rapid_llm's docs/benchmark_models.md:141-149: decode tok/s is
 batch / mean step time; prefill tok/s is prompt tokens / prefill latency; both timed
@@ -64,6 +67,22 @@ def load_shape() -> dict:
         context=num(r"context (\d+)"),
         prompt_len=num(r"one ([\d,]+)-token prompt"),
     )
+
+
+# Other members of the model family (layer sizes as their model cards give them), for
+# measurements beside the default run's.
+FAMILY = {
+    "qwen3-0.6b": dict(num_hidden_layers=28, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8,
+                       intermediate_size=3072, tie_word_embeddings=True),
+    "qwen3-1.7b": dict(num_hidden_layers=28, hidden_size=2048, num_attention_heads=16, num_key_value_heads=8,
+                       intermediate_size=6144, tie_word_embeddings=True),
+    "qwen3-4b": dict(num_hidden_layers=36, hidden_size=2560, num_attention_heads=32, num_key_value_heads=8,
+                     intermediate_size=9728, tie_word_embeddings=True),
+    "qwen3-14b": dict(num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                      intermediate_size=17408, tie_word_embeddings=False),
+    "qwen3-32b": dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
+                      intermediate_size=25600, tie_word_embeddings=False),
+}
 
 
 def weight_bytes(cfg, elem: int) -> int:
@@ -133,6 +152,11 @@ def float32_points(args) -> dict:
     ]
     if args.layers is not None:
         cmd += ["--layers", str(args.layers)]
+    cmd += ["--shape", args.shape]
+    if args.prompt_len is not None:
+        cmd += ["--prompt-len", str(args.prompt_len)]
+    if args.context is not None:
+        cmd += ["--context", str(args.context)]
     try:
         done = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
         line = json.loads(done.stdout.strip().splitlines()[-1])
@@ -153,6 +177,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--shape", default="qwen3-8b", choices=["qwen3-8b", *FAMILY],
+                    help="layer sizes: qwen3-8b is BASELINE.json configs[2], the others its family's")
+    ap.add_argument("--prompt-len", type=int, default=None, help="tokens of every prompt (default 2,048)")
+    ap.add_argument("--context", type=int, default=None, help="longest sequence the engine is sized for")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to measure ('' for none)")
     ap.add_argument("--point-steps", type=int, default=32)
@@ -179,6 +207,17 @@ def main() -> int:
 
     shape = load_shape()
     context, prompt_len = shape.pop("context"), shape.pop("prompt_len")
+    if args.shape != "qwen3-8b":
+        shape.update(FAMILY[args.shape])
+    if args.prompt_len is not None:
+        prompt_len = args.prompt_len
+        context = max(context, prompt_len + 2048)
+    if args.context is not None:
+        context = args.context
+    room = max(args.steps + args.warmup, args.point_steps + max(2, args.warmup // 2)) + 2
+    if prompt_len < 1 or prompt_len + room > context:
+        print(f"a prompt of {prompt_len} tokens and {room} decoded ones do not fit a context of {context}")
+        return 2
     full_layers = shape["num_hidden_layers"]
     if args.layers is not None:
         shape["num_hidden_layers"] = args.layers
@@ -190,9 +229,9 @@ def main() -> int:
         dtype=args.dtype,
         max_seq_len=context,
         page_size=16,
-        num_pages=max_batch * (context // 16) + 1,
+        num_pages=max_batch * (-(-(prompt_len + room) // 16)) + 1,
         max_num_seqs=max_batch,
-        max_num_batched_tokens=max(8192, prompt_len),
+        max_num_batched_tokens=8192,
         use_graph=not args.no_graph,
         seed=1234,
     )
@@ -207,15 +246,23 @@ def main() -> int:
     def prompt() -> list[int]:
         return torch.randint(0, vocab, (prompt_len,), generator=gen).tolist()
 
-    # ---- prefill of one 2,048-token prompt ------------------------------------
+    def portions(rid: str, toks: list[int]) -> list[StepEntry]:
+        """The prompt as the steps that run it: whole if the step's token budget holds it, else
+        in portions of that budget; the last one asks for the logits of its last token."""
+        budget = engine.max_num_batched_tokens
+        cuts = [toks[lo : lo + budget] for lo in range(0, len(toks), budget)]
+        return [StepEntry(rid, part, [len(part) - 1] if i == len(cuts) - 1 else []) for i, part in enumerate(cuts)]
+
+    # ---- prefill of one prompt (2,048 tokens unless asked otherwise) ----------
     prefill = None
     if not args.no_prefill:
         times = []
         for i in range(4):
-            toks = prompt()
+            cuts = portions("p", prompt())
             torch.cuda.synchronize()
             t = time.perf_counter()
-            runner.step([StepEntry("p", toks, [prompt_len - 1])])
+            for entry in cuts:
+                runner.step([entry])
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t)
             runner.finish("p")
@@ -246,7 +293,10 @@ def main() -> int:
         ids = [f"d{i}" for i in range(batch)]
         tokens = []
         for rid in ids:  # prompts, one request a step
-            tokens += executor.execute([StepEntry(rid, prompt(), [prompt_len - 1])], greedy(1)).token_ids
+            cuts = portions(rid, prompt())
+            for entry in cuts[:-1]:
+                executor.execute([entry], greedy(0))
+            tokens += executor.execute([cuts[-1]], greedy(1)).token_ids
         plan = greedy(batch)
         fed = [StepEntry(rid, [fed_token(i)], [0]) for i, rid in enumerate(ids)]
         inflight = executor.launch([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)], plan)
@@ -277,11 +327,13 @@ def main() -> int:
             runner.finish(rid)
         return sec, mean_ctx
 
+    model_name = "Qwen3-" + args.shape.split("-")[1].upper()
     sec, mean_ctx = decode(args.batch, args.steps, args.warmup)
     step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
     achieved = step_bytes / sec / 1e9
     result = {
-        "metric": "Qwen3-8B bf16 decode tok/s (batch 8, 2048-token prompts); prefill tok/s at 2048 tokens",
+        "metric": f"{model_name} {'bf16' if args.dtype == 'bfloat16' else 'fp32'} decode tok/s (batch {args.batch}, "
+                  f"{prompt_len}-token prompts); prefill tok/s at {prompt_len} tokens",
         "value": round(args.batch / sec, 2),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -294,7 +346,7 @@ def main() -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic (uniform random token ids, random N(0,0.02) weights, norm weights 1)",
         "config": {
-            "model": "Qwen3-8B shape",
+            "model": f"{model_name} shape",
             "layers": cfg.num_hidden_layers,
             "layers_full": full_layers,
             "hidden": cfg.hidden_size,
