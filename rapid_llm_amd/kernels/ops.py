@@ -52,7 +52,9 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
 
 
 def _stream() -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the raw handle of the current stream of the current device, without the stream object
+    # that ``torch.cuda.current_stream()`` builds (2.8 against 0.2 us a call, on every launch)
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
 
 
 def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
@@ -74,8 +76,12 @@ def _need(t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape=No
     if dtype is not None and t.dtype != dtype:
         raise KernelError(f"{name} must be {dtype}, is {t.dtype}")
     if shape is not None:
-        if len(shape) != t.dim() or any(s is not None and s != a for s, a in zip(shape, t.shape)):
-            raise KernelError(f"{name} must have shape {tuple(shape)}, has {tuple(t.shape)}")
+        have = t.shape
+        if len(shape) != len(have):
+            raise KernelError(f"{name} must have shape {tuple(shape)}, has {tuple(have)}")
+        for want, size in zip(shape, have):
+            if want is not None and want != size:
+                raise KernelError(f"{name} must have shape {tuple(shape)}, has {tuple(have)}")
 
 
 def _ok(code: int, what: str) -> None:
