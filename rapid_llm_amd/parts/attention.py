@@ -97,7 +97,7 @@ class GQAAttention(Mixer):
     # ---- step ------------------------------------------------------------------
     @property
     def accepts_scaled_rows(self) -> bool:
-        return self.qkv.weight.dtype == torch.bfloat16
+        return self.qkv.takes_scaled_rows()
 
     def forward(self, x, ctx, cache):
         tokens = x.shape[0]

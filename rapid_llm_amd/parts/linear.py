@@ -41,6 +41,11 @@ class Linear:
             and x.shape[0] <= ops.SKINNY_MAX_ROWS and self.in_features % 8 == 0
         )
 
+    def takes_scaled_rows(self) -> bool:
+        """Whether this product can finish a norm whose rows arrive unscaled (whatever the
+        few rows of a step are): only the few-row kernel has that epilogue."""
+        return self.weight is not None and self.weight.dtype == torch.bfloat16 and self.in_features % 8 == 0
+
     def midsize(self, x) -> bool:
         """Whether ``x`` (more rows than the few-row kernel takes) may run as float32 runs of K
         that a norm adds (narrow matrices only: the wide ones are faster in the library)."""

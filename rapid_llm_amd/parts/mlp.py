@@ -50,7 +50,7 @@ class SwiGLU(FeedForward):
 
     @property
     def accepts_scaled_rows(self) -> bool:
-        return self.gate_up.weight.dtype == torch.bfloat16
+        return self.gate_up.takes_scaled_rows()
 
     def forward(self, x, ctx):
         w = self.gate_up.weight

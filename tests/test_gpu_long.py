@@ -25,7 +25,7 @@ def _runner(model_dir, dtype, page, max_seq_len, graph=False, num_pages=None, se
     )
 
 
-@pytest.mark.parametrize("which", ["B", "C", "D"])
+@pytest.mark.parametrize("which", ["B", "C", "D", "F"])
 @pytest.mark.parametrize("dtype,graph", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
 def test_long_decoding(tmp_path, which, dtype, graph):
     from rapid_llm_amd import StepEntry
@@ -61,7 +61,7 @@ def test_long_decoding(tmp_path, which, dtype, graph):
     runner.cache.check_invariants()
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "F"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens(tmp_path, which, dtype):
     """Positions 0, 1, 2: a one-token prompt, its first decoded tokens, a two-token prompt cut

@@ -24,6 +24,7 @@ LENGTHS = {
     "C": [9, 33, 48, 77, 130, 201],
     "D": [12, 40, 66, 150, 333, 600],
     "E": [20, 35, 49, 64, 90, 200],          # portions of 17 to 64 tokens take the mid-size product
+    "F": [3, 31, 33, 64, 97, 180],           # page of 32: requests within one page, at its edge, across several
 }
 
 
@@ -71,7 +72,7 @@ def _check(got, want, dtype, label):
             raise AssertionError(f"{label}: request {rid}, first wrong position {first}: {exc}") from None
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_every_cut_matches_plain(tmp_path, which, dtype):
     cfg, page, seed = TINY[which]

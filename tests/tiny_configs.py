@@ -57,9 +57,20 @@ TINY_E = dict(
     hidden_act="silu", attention_bias=False,
 )
 PAGE_E = 8
+# F: widths that no vector access divides (70 = 2 * 35, 99 odd, vocabulary 211 prime): every
+# kernel takes its element-by-element path and the bfloat16 products go to the library;
+# heads * head_dim = 96 beside a width of 70; a page larger than most requests
+TINY_F = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=70, num_attention_heads=6, num_key_value_heads=3,
+    head_dim=16, intermediate_size=99, vocab_size=211, rope_theta=7777.0,
+    rms_norm_eps=4e-6, tie_word_embeddings=False, max_position_embeddings=256,
+    hidden_act="silu", attention_bias=False,
+)
+PAGE_F = 32
 
 TINY = {"A": (TINY_A, PAGE_A, 11), "B": (TINY_B, PAGE_B, 22), "C": (TINY_C, PAGE_C, 33),
-        "D": (TINY_D, PAGE_D, 44), "E": (TINY_E, PAGE_E, 55)}
+        "D": (TINY_D, PAGE_D, 44), "E": (TINY_E, PAGE_E, 55), "F": (TINY_F, PAGE_F, 66)}
 
 
 def make_model_dir(tmp_path: Path, which: str, dtype: str = "float32") -> Path:
