@@ -38,3 +38,39 @@ def test_whole_prompts(tmp_path, which, dtype):
         tol = F32_TOL if dtype == "float32" else BF16_TOL
         torch.testing.assert_close(got, want, **tol)
     runner.cache.check_invariants()
+
+
+def test_matrices_stored_in_32_bit_stay_so_in_a_bfloat16_engine(tmp_path):
+    """A checkpoint may store some tensors in 32-bit: they are held and multiplied in 32-bit
+    beside bfloat16 neighbours (a fused matrix with one 32-bit source is 32-bit whole), in whole
+    prompts and in single decoded tokens, where the bfloat16 products around them fold norms
+    into their kernels and these cannot."""
+    from safetensors.torch import load_file, save_file
+
+    from rapid_llm_amd import StepEntry
+
+    cfg, page, seed = TINY["D"]
+    model_dir = make_model_dir(tmp_path, "D", "bfloat16")
+    path = str(model_dir / "model.safetensors")
+    tensors = load_file(path)
+    gen = torch.Generator().manual_seed(5)
+    wide = ["model.layers.0.mlp.gate_proj.weight", "model.layers.0.mlp.up_proj.weight",
+            "model.layers.1.self_attn.o_proj.weight", "model.layers.0.self_attn.k_proj.weight",
+            "model.layers.1.mlp.down_proj.weight", "model.embed_tokens.weight"]
+    for name in wide:  # values that bfloat16 cannot hold
+        t = tensors[name].float()
+        tensors[name] = t + 1e-4 * torch.randn(t.shape, generator=gen)
+    save_file(tensors, path)
+    pcfg, pw = plain_load(model_dir)
+    runner = _runner(model_dir, "bfloat16", page)
+    matrices = {name: p.dtype for name, p in runner.params.items() if p.dim() == 2}
+    assert set(matrices.values()) == {torch.float32, torch.bfloat16}
+    assert matrices["layers.0.ff.gate_up"] == torch.float32 and matrices["layers.1.ff.gate_up"] == torch.bfloat16
+    assert matrices["layers.0.mixer.qkv"] == torch.float32  # one of its three sources is 32-bit
+    toks = random_tokens(60, cfg["vocab_size"], seed)
+    want = plain_forward(pcfg, pw, toks)
+    got = [runner.step([StepEntry("r", toks[:40], list(range(40)))]).cpu()]
+    for t in toks[40:]:
+        got.append(runner.step([StepEntry("r", [t], [0])]).cpu())
+    torch.testing.assert_close(torch.cat(got), want, **BF16_TOL)
+    runner.finish("r")
