@@ -317,6 +317,50 @@ def test_command_line_batch(tmp_path, capsys):
     assert str(_plain_generate(pcfg, pw, [1, 2, 3, 4], 6)) in text
 
 
+def _word_tokenizer(model_dir, vocab):
+    """A tokenizer.json in which the word ``w<i>`` is token ``i``."""
+    from tokenizers import Tokenizer, models, pre_tokenizers
+
+    tok = Tokenizer(models.WordLevel({f"w{i}": i for i in range(vocab)}, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+    tok.save(str(model_dir / "tokenizer.json"))
+
+
+def test_text_prompts_with_a_tokenizer(tmp_path, capsys, monkeypatch):
+    """A model folder with a tokenizer.json takes text and gives text back: through
+    ``generate``, through ``stream`` (whose deltas add up to the text), and through the
+    ``batch`` and ``chat`` commands."""
+    from rapid_llm_amd import SamplingParams
+    from rapid_llm_amd.cli import main
+
+    cfg, page, seed = TINY["A"]
+    model_dir = make_model_dir(tmp_path, "A", "float32")
+    _word_tokenizer(model_dir, cfg["vocab_size"])
+    llm = _llm(model_dir, "float32", page, max_seq_len=64)
+    params = SamplingParams(temperature=0.0, max_gen_len=6)
+    by_text = llm.generate(["w5 w17 w3", "w9"], params)
+    by_ids = llm.generate([[5, 17, 3], [9]], params)
+    for a, b in zip(by_text, by_ids):
+        assert a.prompt_token_ids == b.prompt_token_ids and a.token_ids == b.token_ids
+        assert a.text == " ".join(f"w{t}" for t in a.token_ids)
+    assert by_text[0].prompt == "w5 w17 w3"
+    texts = [batch[0].text for batch in llm.stream("w5 w17 w3", params)]
+    assert texts[-1] == by_text[0].text and len(texts) >= 6
+    assert all(later.startswith(earlier) for earlier, later in zip(texts, texts[1:]))
+    prompts = tmp_path / "prompts.txt"
+    prompts.write_text("w5 w17 w3\nw9\n")
+    common = ["--model-dir", str(model_dir), "--dtype", "float32", "--max-seq-len", "64", "--temperature", "0",
+              "--max-gen-len", "6", "--repetition-penalty", "1.0", "--no-cuda-graph"]
+    assert main(["batch", *common, "--prompts-file", str(prompts), "--no-chat-template"]) == 0
+    text = capsys.readouterr().out
+    assert by_text[0].text in text and by_text[1].text in text
+    lines = iter(["w5 w17 w3", "/clear", "", "w9", "exit"])
+    monkeypatch.setattr("builtins.input", lambda prompt="": next(lines))
+    assert main(["chat", *common]) == 0
+    text = capsys.readouterr().out
+    assert text.count("w") > 10  # two streamed answers of six words each
+
+
 def test_command_line_bench(tmp_path, capsys):
     import json
 

@@ -20,3 +20,34 @@ def test_a_product_takes_unscaled_rows_only_if_its_few_row_kernel_runs():
     assert not _bound(70, 198, torch.bfloat16).takes_scaled_rows()
     assert not _bound(96, 70, torch.float32).takes_scaled_rows()  # a matrix the checkpoint stores in 32-bit
     assert not Linear(96, 70).takes_scaled_rows()  # nothing bound yet
+
+
+class _ByteTokenizer:
+    """Token id = one byte: a character of several bytes spans tokens."""
+
+    def decode(self, ids, skip_special_tokens=True):
+        return bytes(ids).decode("utf-8", errors="replace")
+
+
+def test_text_is_released_only_with_whole_characters():
+    from rapid_llm_amd.engine.tokenizer import Detokenizer
+
+    text = "a é 漢字 ok"
+    detok = Detokenizer(_ByteTokenizer())
+    pieces = [detok.append(b) for b in text.encode("utf-8")]
+    assert "".join(pieces) == text
+    assert all("�" not in p for p in pieces)
+    assert pieces[2] == "" and pieces[3] == "é"  # the first byte of a two-byte character releases nothing
+
+
+def test_stop_ids_come_from_generation_config_and_config(tmp_path):
+    from rapid_llm_amd.engine.tokenizer import load_stop_token_ids, load_tokenizer
+
+    assert load_stop_token_ids(tmp_path, config_eos=[7]) == {7}
+    (tmp_path / "generation_config.json").write_text('{"eos_token_id": [3, 9]}')
+    assert load_stop_token_ids(tmp_path, config_eos=[7]) == {3, 7, 9}
+    (tmp_path / "generation_config.json").write_text('{"eos_token_id": 4}')
+    assert load_stop_token_ids(tmp_path) == {4}
+    (tmp_path / "generation_config.json").write_text("{not json")
+    assert load_stop_token_ids(tmp_path, config_eos=[1]) == {1}
+    assert load_tokenizer(tmp_path) is None  # no tokenizer.json: prompts are token ids
