@@ -317,6 +317,36 @@ def test_command_line_batch(tmp_path, capsys):
     assert str(_plain_generate(pcfg, pw, [1, 2, 3, 4], 6)) in text
 
 
+def test_entry_point_options(tmp_path):
+    """What ``LLM(...)`` takes beside the model folder: options of the reference that this
+    engine has no use for are refused by name; the cache pool comes from the reference's knob
+    (in tokens), or from the memory that is free, capped at what every slot at full length can
+    use; ``hf_overrides`` changes configuration keys; ``load_format="random"`` needs no
+    weights file and is fixed by the seed."""
+    from rapid_llm_amd import LLM, SamplingParams
+
+    cfg, page, seed = TINY["B"]
+    model_dir = make_model_dir(tmp_path, "B", "float32")
+    for kw, message in ((dict(quantization="int8"), "quantization"), (dict(tensor_parallel_size=2), "one GPU"),
+                        (dict(data_parallel_size=4), "one GPU"), (dict(kv_cache_dtype="fp8"), "kv_cache_dtype")):
+        with pytest.raises(ValueError, match=message):
+            LLM(str(model_dir), **kw)
+    common = dict(dtype="float32", max_seq_len=64, page_size=8, max_num_seqs=4, use_cuda_graph=False)
+    assert LLM(str(model_dir), max_gpu_num_blocks=200, **common).scheduler.cache.pools[0].num_usable == 25
+    assert LLM(str(model_dir), **common).scheduler.cache.pools[0].num_usable == 4 * 8
+    # two of the three layers: the plain model with the same key changed
+    prompt = random_tokens(9, cfg["vocab_size"], 3)
+    params = SamplingParams(temperature=0.0, max_gen_len=8)
+    pcfg, pw = plain_load(model_dir)
+    short = LLM(str(model_dir), hf_overrides={"num_hidden_layers": 2}, **common).generate(prompt, params)[0]
+    assert short.token_ids == _plain_generate(dict(pcfg, num_hidden_layers=2), pw, prompt, 8)
+    assert short.token_ids != _plain_generate(pcfg, pw, prompt, 8)
+    # random weights from a configuration alone
+    outs = [LLM(dict(cfg), load_format="random", seed=s, **common).generate(prompt, params)[0].token_ids
+            for s in (3, 3, 4)]
+    assert outs[0] == outs[1] and outs[0] != outs[2]
+
+
 def _word_tokenizer(model_dir, vocab):
     """A tokenizer.json in which the word ``w<i>`` is token ``i``."""
     from tokenizers import Tokenizer, models, pre_tokenizers
