@@ -391,6 +391,37 @@ def test_text_prompts_with_a_tokenizer(tmp_path, capsys, monkeypatch):
     assert text.count("w") > 10  # two streamed answers of six words each
 
 
+def test_command_line_defaults_and_replay(tmp_path, capsys, monkeypatch):
+    """``batch`` with the command line's own defaults (temperature 0.6, nucleus 0.9, penalty
+    1.1, graphs, the folder from the environment) ends every request; ``replay`` writes the
+    logits ``bin/trace_run`` would."""
+    import json
+
+    import numpy as np
+
+    from rapid_llm_amd.cli import main
+
+    cfg, page, seed = TINY["D"]
+    model_dir = make_model_dir(tmp_path, "D", "bfloat16")
+    monkeypatch.setenv("RAPID_LLM_MODEL_DIR", str(model_dir))
+    assert main(["batch", "--max-seq-len", "96", "--max-gen-len", "40", "--show-stats"]) == 0
+    text = capsys.readouterr().out
+    assert text.count("--- [") == 4 and "4 requests" in text
+    trace = tmp_path / "trace.jsonl"
+    toks = random_tokens(20, cfg["vocab_size"], 1)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:17], "want": [16]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[17:], "want": [0, 2]}], "end": ["a"]}]
+    trace.write_text("".join(json.dumps(s) + "\n" for s in steps))
+    out = tmp_path / "logits"
+    assert main(["replay", "--model", str(model_dir), "--dtype", "float32", "--out", str(out), "--max-tokens", "64",
+                 "--trace", str(trace)]) == 0
+    assert capsys.readouterr().out.split() == ["done", "0", "done", "1"]
+    pcfg, pw = plain_load(model_dir)
+    want = plain_forward(pcfg, pw, toks)
+    got = np.fromfile(out / "1.f32", dtype="<f4").reshape(2, cfg["vocab_size"])
+    assert np.allclose(got, want[[17, 19]].numpy(), rtol=2e-5, atol=3e-6)
+
+
 def test_command_line_bench(tmp_path, capsys):
     import json
 

@@ -51,3 +51,32 @@ def test_stop_ids_come_from_generation_config_and_config(tmp_path):
     (tmp_path / "generation_config.json").write_text("{not json")
     assert load_stop_token_ids(tmp_path, config_eos=[1]) == {1}
     assert load_tokenizer(tmp_path) is None  # no tokenizer.json: prompts are token ids
+
+
+def test_command_line_init_writes_a_model_folder_and_names_a_missing_one(tmp_path, capsys, monkeypatch):
+    import json
+
+    import pytest
+    from safetensors.torch import load_file
+
+    from rapid_llm_amd.cli import main
+    from tiny_configs import TINY_B
+
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(TINY_B))
+    for seed in (4, 4, 5):
+        assert main(["init", "--config", str(config), "--out", str(tmp_path / f"m{seed}"), "--seed", str(seed),
+                     "--dtype", "bfloat16"]) == 0
+    a = load_file(str(tmp_path / "m4" / "model.safetensors"))
+    assert json.loads((tmp_path / "m4" / "config.json").read_text())["torch_dtype"] == "bfloat16"
+    assert a["model.layers.2.mlp.down_proj.weight"].shape == (96, 320)
+    assert a["model.embed_tokens.weight"].dtype == __import__("torch").bfloat16
+    b = load_file(str(tmp_path / "m5" / "model.safetensors"))
+    assert not (a["lm_head.weight"] == b["lm_head.weight"]).all()
+    # generation commands name the folder they lack, or take it from the environment
+    monkeypatch.delenv("RAPID_LLM_MODEL_DIR", raising=False)
+    with pytest.raises(SystemExit, match="Model directory not provided"):
+        main(["batch"])
+    monkeypatch.setenv("RAPID_LLM_MODEL_DIR", str(tmp_path / "nowhere"))
+    with pytest.raises(SystemExit, match="does not exist"):
+        main(["batch"])
