@@ -172,18 +172,20 @@ def test_bfloat16_generation_stays_near_the_plain_choice(tmp_path, which):
             assert len(out.token_ids) == 16
 
 
-def test_bfloat16_generation_of_forty_requests_at_once(tmp_path):
+@pytest.mark.parametrize("which,count,rows", [("E", 40, (17, 64)), ("D", 100, (65, 128))])
+def test_bfloat16_generation_of_many_requests_at_once(tmp_path, which, count, rows):
     """Decode batches between 17 and 64 rows (configuration E: the output and down projections
-    then run as runs of K added by the norms), with and without graphs."""
+    then run as runs of K added by the norms) and beyond 64 (every product from the library),
+    with and without graphs."""
     from rapid_llm_amd import SamplingParams
 
-    cfg, page, seed = TINY["E"]
-    model_dir = make_model_dir(tmp_path, "E", "bfloat16")
+    cfg, page, seed = TINY[which]
+    model_dir = make_model_dir(tmp_path, which, "bfloat16")
     pcfg, pw = plain_load(model_dir)
-    prompts = [random_tokens(2 + (7 * i) % 23, cfg["vocab_size"], seed + i) for i in range(40)]
+    prompts = [random_tokens(2 + (7 * i) % 23, cfg["vocab_size"], seed + i) for i in range(count)]
     for graph in (False, True):
-        llm = _llm(model_dir, "bfloat16", page, max_seq_len=64, max_num_seqs=48, num_pages=48 * 8 + 8,
-                   use_cuda_graph=graph)
+        llm = _llm(model_dir, "bfloat16", page, max_seq_len=64, max_num_seqs=count + 8,
+                   num_pages=(count + 8) * (64 // page) + 8, use_cuda_graph=graph)
         outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_gen_len=6))
         for prompt, out in zip(prompts, outs):
             ids = list(prompt)
@@ -193,7 +195,7 @@ def test_bfloat16_generation_of_forty_requests_at_once(tmp_path):
                 ids.append(tok)
             assert len(out.token_ids) == 6
         if graph:
-            assert any(17 <= key[0] <= 64 for key in llm.scheduler.runner._graphs)
+            assert any(rows[0] <= key[0] <= rows[1] for key in llm.scheduler.runner._graphs)
 
 
 def test_stop_tokens_and_stream(tmp_path):
