@@ -74,3 +74,18 @@ def test_matrices_stored_in_32_bit_stay_so_in_a_bfloat16_engine(tmp_path):
         got.append(runner.step([StepEntry("r", [t], [0])]).cpu())
     torch.testing.assert_close(torch.cat(got), want, **BF16_TOL)
     runner.finish("r")
+
+
+def test_a_bfloat16_checkpoint_in_a_float32_engine(tmp_path):
+    """The engine's type, not the file's, decides the arithmetic: weights stored in bfloat16
+    are widened once and everything runs in true 32-bit."""
+    from rapid_llm_amd import StepEntry
+
+    cfg, page, seed = TINY["B"]
+    model_dir = make_model_dir(tmp_path, "B", "bfloat16")
+    pcfg, pw = plain_load(model_dir)
+    runner = _runner(model_dir, "float32", page)
+    assert {p.dtype for p in runner.params.values()} == {torch.float32}
+    toks = random_tokens(50, cfg["vocab_size"], seed)
+    got = runner.step([StepEntry("r", toks, list(range(50)))]).cpu()
+    torch.testing.assert_close(got, plain_forward(pcfg, pw, toks), **F32_TOL)
