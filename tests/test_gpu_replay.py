@@ -124,3 +124,42 @@ def test_trace_run_program(tmp_path, dtype):
     steps = ru.mixed(requests, seed + 5, max_tokens=max_tokens)
     got = ru.run_trace_program(model_dir, dtype, steps, tmp_path / "out", max_tokens, cfg["vocab_size"])
     _check(got, want, dtype, f"trace_run/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_request_id_is_used_again_after_it_ended(tmp_path, dtype):
+    """An id that ended names a new request the next time it appears: nothing of the old one
+    (its length, its pages, its place in the block table) is left, also when the new one
+    starts in the very step after and beside other requests."""
+    which = "B"
+    cfg, page, seed = TINY[which]
+    model_dir = make_model_dir(tmp_path, which, dtype)
+    pcfg, pw = plain_load(model_dir)
+    vocab = cfg["vocab_size"]
+    first, second, other = (random_tokens(n, vocab, seed + n) for n in (45, 30, 38))
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": first[:40], "want": list(range(40))},
+                                {"id": "o", "tokens": other[:20], "want": list(range(20))}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": first[40:], "want": list(range(5))},
+                                {"id": "o", "tokens": other[20:21], "want": [0]}], "end": ["a"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": second[:7], "want": list(range(7))},
+                                {"id": "o", "tokens": other[21:], "want": list(range(17))}], "end": ["o"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": second[7:], "want": list(range(23))}], "end": ["a"]},
+    ]
+    runner = _runner(model_dir, dtype, page, 7, cfg["max_position_embeddings"])  # 6 pages of 16: reuse
+    rows = {"a1": [], "a2": [], "o": []}
+    from rapid_llm_amd import StepEntry
+
+    for step in steps:
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in step["entries"]]).cpu()
+        at = 0
+        for e in step["entries"]:
+            key = "o" if e["id"] == "o" else ("a1" if step["step"] < 2 else "a2")
+            rows[key].append(logits[at : at + len(e["want"])])
+            at += len(e["want"])
+        for rid in step["end"]:
+            runner.finish(rid)
+    want = {"a1": plain_forward(pcfg, pw, first), "a2": plain_forward(pcfg, pw, second), "o": plain_forward(pcfg, pw, other)}
+    _check({k: torch.cat(v) for k, v in rows.items()}, want, dtype, f"id reuse/{dtype}")
+    assert not runner.cache.live_requests()
+    runner.cache.check_invariants()
