@@ -77,23 +77,27 @@ def test_sampled_generation_tiny_b_chunked_and_mixed(tmp_path):
         assert solo.generate(prompt, p)[0].token_ids == out.token_ids
 
 
-def test_eviction_changes_nothing(tmp_path):
+@pytest.mark.parametrize("which,pages", [("A", 24), ("C", 13)])
+def test_eviction_changes_nothing(tmp_path, which, pages):
     """So few pages that running requests are evicted and recomputed: the tokens are the ones
-    an ample pool gives, greedy and sampled."""
+    an ample pool gives, greedy and sampled.  Configuration C has windowed layers beside a
+    full one: two pools, of which the windowed one gives pages back while requests run."""
     from rapid_llm_amd import SamplingParams
 
-    cfg, page, seed = TINY["A"]
-    model_dir = make_model_dir(tmp_path, "A", "float32")
+    cfg, page, seed = TINY[which]
+    model_dir = make_model_dir(tmp_path, which, "float32")
     prompts = [random_tokens(n, cfg["vocab_size"], seed + n) for n in (9, 14, 6, 11)]
     params = [SamplingParams(temperature=0.0 if i % 2 else 0.7, top_p=0.95, max_gen_len=30, seed=i,
                              repetition_penalty=1.15) for i in range(4)]
     ample = _llm(model_dir, "float32", page, max_seq_len=128).generate(prompts, params)
-    tight = _llm(model_dir, "float32", page, max_seq_len=128, num_pages=24)  # 23 pages of 4: ~2 requests
+    tight = _llm(model_dir, "float32", page, max_seq_len=128, num_pages=pages)  # room for about two requests
     outs = tight.generate(prompts, params)
     assert tight.scheduler.num_preemptions > 0
     assert [o.token_ids for o in outs] == [o.token_ids for o in ample]
-    tight.scheduler.cache.check_invariants()
-    assert tight.scheduler.cache.num_free_pages() == 23
+    cache = tight.scheduler.cache
+    cache.check_invariants()
+    assert all(pool.num_free == pages - 1 for pool in cache.pools.values())
+    assert len(cache.pools) == (2 if which == "C" else 1)
 
 
 def test_logprob_records_of_prompt_and_output(tmp_path):
