@@ -1,6 +1,9 @@
 // Token selection from float32 logits.  Greedy rows take the arg-max (the lowest index
 // among equal maxima, as torch.argmax does on one device).
 #include "common.h"
+#include "static_entry.h"
+
+#include <mutex>
 
 // row_index (optional, in every kernel of this file): the row of `logits` that output row b
 // reads; without it output row b reads row b.
@@ -144,6 +147,58 @@ extern "C" int rl_argmax(const float* logits, const int* row_index, int* out, fl
     }
     hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, stream, logits, row_index,
                        out, vocab);
+    return rl_launch_status();
+}
+
+// The two-stage arg-max for callers that cannot allocate (static_entry.h): stage one's results
+// live in this array, of which every GPU holds its own copy at its own address.  In host code
+// the array's name is only a handle for hipGetSymbolAddress; kernels and every other host use
+// take the address that call returned for the current device.
+static __device__ __align__(256) unsigned char argmax_static_scratch[RL_ARGMAX_STATIC_ENTRIES * 8];
+
+#define RL_MAX_DEVICES 64
+static void* argmax_static_ptr[RL_MAX_DEVICES];
+static std::mutex argmax_static_mutex;
+
+// The address of the current device's copy of the array; looked up once per device.
+static int argmax_static_address(void** ptr) {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= RL_MAX_DEVICES)
+        return RL_ERR_SETUP;
+    std::lock_guard<std::mutex> guard(argmax_static_mutex);
+    if (!argmax_static_ptr[device]) {
+        void* found = nullptr;
+        if (hipGetSymbolAddress(&found, HIP_SYMBOL(argmax_static_scratch)) != hipSuccess || !found)
+            return RL_ERR_SETUP;
+        argmax_static_ptr[device] = found;
+    }
+    *ptr = argmax_static_ptr[device];
+    return RL_OK;
+}
+
+extern "C" int rl_argmax_static_prepare() {
+    void* ptr = nullptr;
+    return argmax_static_address(&ptr);
+}
+
+extern "C" int rl_argmax_static_limit() { return RL_ARGMAX_STATIC_ENTRIES; }
+
+extern "C" int rl_argmax_static(const float* logits, const int* row_index, int* out, int rows,
+                                int vocab, hipStream_t stream) {
+    if (rows <= 0) return RL_OK;
+    if (vocab < 1 || rows > 65535) return RL_ERR_ARG;
+    const int slices = (vocab + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
+    if ((long)rows * slices > RL_ARGMAX_STATIC_ENTRIES) return RL_ERR_ARG;
+    void* base = nullptr;
+    const int rc = argmax_static_address(&base);
+    if (rc != RL_OK) return rc;
+    float* part_v = reinterpret_cast<float*>(base);
+    int* part_i = reinterpret_cast<int*>(static_cast<unsigned char*>(base) + RL_ARGMAX_STATIC_ENTRIES * 4);
+    hipLaunchKernelGGL(argmax_slices_kernel, dim3(slices, rows), dim3(256), 0, stream, logits,
+                       row_index, part_v, part_i, vocab, slices);
+    if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
+    hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(RL_WAVE), 0, stream, part_v, part_i,
+                       out, slices);
     return rl_launch_status();
 }
 

@@ -41,7 +41,7 @@ CORE_SOURCES = (
     "gemm_bf16.hip",
 )
 ATTENTION_SOURCES = ("attention_mfma.hip", "attention_f32.hip")
-HEADERS = ("common.h",)
+HEADERS = ("common.h", "static_entry.h")
 
 # head sizes built ahead of time by build_all(): every one the kernels take.  A fresh
 # checkout compiles only the head size of the model it is asked to run.
