@@ -229,7 +229,7 @@ class Scheduler:
         number = next(self._ids)
         if request_id is None:
             request_id = f"req-{number}"
-        if request_id in self._requests and not self._requests[request_id].is_finished:
+        if request_id in self._requests:  # finished requests are not kept: the id is free again
             raise ValueError(f"request id {request_id!r} is already in use")
         if isinstance(prompt, str):
             if self.tokenizer is None:
@@ -293,6 +293,8 @@ class Scheduler:
         request.finish_reason = reason
         request.finish_time = time.monotonic()
         self._detok.pop(request.request_id, None)
+        # the caller holds the request object; the engine keeps nothing of a finished request
+        self._requests.pop(request.request_id, None)
 
     def _preempt(self, request: Request, plan: StepPlan) -> None:
         """Eviction by recomputation (rapid_llm/engine/batch_planner.py:987-1023)."""
@@ -374,6 +376,10 @@ class Scheduler:
             request = self.waiting[0]
             count = self._portion(request, budget)
             if count < 1:
+                break
+            if cache.has(request.request_id):
+                # the id's previous request has ended, but a step in flight still rides on its
+                # slot and pages: the new one waits the one step until they are given back
                 break
             if cache.admit(request.request_id) is None:
                 break

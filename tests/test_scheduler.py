@@ -185,19 +185,20 @@ def test_prompt_is_cut_into_portions_and_sampled_with_the_last():
 
 def test_decodes_run_beside_portions_under_one_budget():
     s, ex = _make(max_num_batched_tokens=20, max_chunk_size=16)
-    s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=8))
+    rs = [s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=8))]
     s.step()  # a: whole prompt, sampled
-    s.add_request(list(range(40)), GREEDY)
+    rs.append(s.add_request(list(range(40)), GREEDY))
     s.step()
     assert ex.steps[1] == [("req-0", 1, True), ("req-1", 16, False)]  # decode first, then the portion
-    s.add_request(list(range(30)), GREEDY)
+    rs.append(s.add_request(list(range(30)), GREEDY))
     s.step()
     # budget 20: 1 decode + 16 of req-1 + 3 left for the newcomer's first portion
     assert ex.steps[2] == [("req-0", 1, True), ("req-1", 16, False), ("req-2", 3, False)]
     for shape in ex.steps:
         assert sum(n for _, n, _ in shape) <= 20
     s.run_to_completion()
-    assert all(r.finish_reason == "length" for r in s._requests.values())
+    assert all(r.finish_reason == "length" for r in rs)
+    assert not s._requests  # the engine keeps nothing of a finished request
 
 
 def test_first_come_first_served_and_slot_limit():
@@ -556,6 +557,36 @@ def test_abort_while_a_step_is_in_flight():
         s.step()
     assert r.output_token_ids == kept and not ex.cache.live_requests()
     assert len(q.output_token_ids) == 3
+
+
+@pytest.mark.parametrize("pipeline", [True, False])
+def test_an_id_is_used_again_while_its_last_step_is_still_in_flight(pipeline):
+    """A request that a stop token ended rides one more step, on whose slot and pages it is
+    still held; the same id submitted at that moment names a new request, which waits that one
+    step and then runs as any other."""
+    s, ex = _make_pipelined(token=lambda rid, i: EOS if i == 1 else 40 + i, pipeline=pipeline)
+    first = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=10), request_id="x")
+    while not first.is_finished:
+        s.step()
+    assert first.finish_reason == "eos" and first.output_token_ids == [40]
+    if pipeline:
+        assert [r.request_id for r in s._held] == ["x"] and ex.cache.has("x")
+    second = s.add_request([1, 2, 3], SamplingParams(temperature=0.0, max_gen_len=10), request_id="x")
+    assert second is not first
+    other = s.add_request([5, 6], SamplingParams(temperature=0.0, max_gen_len=3))
+    steps = 0
+    while s.has_unfinished_requests():
+        s.step()
+        steps += 1
+        assert steps < 50
+    assert second.finish_reason == "eos" and second.output_token_ids == [40]
+    assert first.output_token_ids == [40] and first.pending == 0 and first.discard == 0
+    assert len(other.output_token_ids) == 1 and other.finish_reason == "eos"
+    assert not ex.cache.live_requests() and not s._held and not s._requests
+    ex.cache.check_invariants()
+    with pytest.raises(ValueError, match="already in use"):
+        s.add_request([1], GREEDY, request_id="y")
+        s.add_request([1], GREEDY, request_id="y")
 
 
 def test_request_tokens_name_the_pending_row():
