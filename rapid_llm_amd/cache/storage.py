@@ -96,8 +96,9 @@ class DeviceCache:
             owns = False
             if need.kind == "kv" and need.share_with is None:
                 pages = manager.pools[gid].num_pages
-                # zero-filled once: page 0 is never written, and nothing is ever read from a
-                # page beyond what the masks allow
+                # zero-filled once.  Page 0, the null page, is written by rows that only pad a
+                # batch (their keys and values land in its first slot) and never read unmasked;
+                # nothing is ever read from a page beyond what the masks allow
                 k = torch.zeros((pages, need.num_kv_heads, P, need.head_dim), dtype=dtype, device=device)
                 v = torch.zeros((pages, need.num_kv_heads, need.head_dim, P), dtype=dtype, device=device)
                 owns = True

@@ -74,10 +74,19 @@ def _engine(args, max_num_seqs: int = 32):
     )
 
 
-_CHATML_USER = "<|im_start|>user\n{}<|im_end|>\n<|im_start|>assistant\n"
+def _prompter(args, use_template: bool = True):
+    """The model folder's chat template (rapid_llm/cli.py:650-652), or ``None``: a folder
+    without one, or a base checkpoint, takes its prompts as they are."""
+    from .engine.prompting import build_prompter, is_instruct
+
+    model_dir = _model_dir(args)
+    prompter = build_prompter(model_dir, use_template)
+    if prompter is None and use_template and is_instruct(model_dir) and (Path(model_dir) / "tokenizer.json").is_file():
+        print("the model folder has no chat template: prompts go in as they are", file=sys.stderr)
+    return prompter
 
 
-def _parse_prompt(line: str, engine, template: bool):
+def _parse_prompt(line: str, engine, prompter=None):
     """A line of text, or a list of token ids written as ``[1, 2, 3]`` (models without a
     tokenizer)."""
     line = line.strip()
@@ -85,7 +94,7 @@ def _parse_prompt(line: str, engine, template: bool):
         return [int(t) for t in json.loads(line)]
     if engine.tokenizer is None:
         raise SystemExit("the model folder has no tokenizer.json: give prompts as lists of token ids")
-    return _CHATML_USER.format(line) if template else line
+    return prompter.insert_prompt(line) if prompter is not None else line
 
 
 def cmd_batch(args) -> int:
@@ -105,10 +114,9 @@ def cmd_batch(args) -> int:
         if not lines:
             raise SystemExit(f"{args.prompts_file!r} contains no prompts")
     params = _sampling(args)
+    prompter = _prompter(args, not args.no_chat_template)
     started = time.perf_counter()
-    requests = [
-        engine.add_request(_parse_prompt(ln, engine, not args.no_chat_template), params) for ln in lines
-    ]
+    requests = [engine.add_request(_parse_prompt(ln, engine, prompter), params) for ln in lines]
     engine.run_to_completion()
     elapsed = time.perf_counter() - started
     for index, request in enumerate(requests):
@@ -129,7 +137,9 @@ def cmd_batch(args) -> int:
 def cmd_chat(args) -> int:
     engine = _engine(args, 1)
     params = _sampling(args)
-    history = ""
+    prompter = _prompter(args)
+    messages: list[dict[str, str]] = []  # the conversation so far, formatted anew every turn
+    history = ""  # without a template: the plain text so far
     print("Type a message; '/clear' forgets the conversation, 'exit' leaves.")
     while True:
         try:
@@ -140,12 +150,17 @@ def cmd_chat(args) -> int:
             break
         if line == "/clear":
             history = ""
+            messages = []
             continue
         if not line:
             continue
-        prompt = _parse_prompt(line, engine, True)
+        prompt = _parse_prompt(line, engine)
         if isinstance(prompt, str):
-            prompt = history + prompt
+            if prompter is not None:
+                messages.append({"role": "user", "content": prompt})
+                prompt = prompter.apply(messages)
+            else:
+                prompt = history + prompt
         request = engine.add_request(prompt, params)
         while engine.has_unfinished_requests():
             for r in engine.step():
@@ -155,7 +170,10 @@ def cmd_chat(args) -> int:
             print(request.output_token_ids)
         else:
             print()
-            history = prompt + request.text + "<|im_end|>\n"
+            if prompter is not None:
+                messages.append({"role": "assistant", "content": request.text})
+            else:
+                history = prompt + request.text + "\n"
     return 0
 
 

@@ -153,8 +153,8 @@ struct DecodeFrags {
 };
 
 template <bool V16>
-__device__ inline void decode_load(DecodeFrags& f, const bf16_t* __restrict__ k_cache,
-                                   const bf16_t* __restrict__ v_cache, const int* pages,
+__device__ inline void decode_load(DecodeFrags& f, const bf16_t* k_cache, const bf16_t* v_cache,
+                                   const int* pages,
                                    int page0, int page_size, int nkv, int hk, int base,
                                    int last_key, int col, int g) {
 #pragma unroll
@@ -207,6 +207,9 @@ struct DecodeExtra {
     int qkv_stride;  // elements between the rows of `q` (fused: the packed q|k|v row)
 };
 
+// k_cache and v_cache carry no promise of being the only way to their memory: in the fused
+// form the token's own key and value are stored through ex.k_write / ex.v_write, which point
+// into the same tensors, and read back through them after a fence and a barrier.
 // FUSED: `q` holds raw packed [q | k | v] rows.  The workgroup norms and rotates the query
 // heads of its kv head itself (rapid_llm/models/base.py:134-140), and the workgroup whose
 // split holds the token's own position norms, rotates and writes the new key and value
@@ -215,8 +218,8 @@ struct DecodeExtra {
 // every rotation pair.
 template <bool V16, bool FUSED>
 __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
-    const bf16_t* __restrict__ v_cache, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    const bf16_t* __restrict__ q, const bf16_t* k_cache, const bf16_t* v_cache,
+    bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const int* __restrict__ seq_token,
     const int* __restrict__ positions, const int* __restrict__ token_slot,
     const int* __restrict__ block_table, int table_stride, int page_size, int nq, int nkv,

@@ -30,10 +30,35 @@ def load_tokenizer(model_dir: str | Path) -> TextTokenizer | None:
     return TextTokenizer(path) if path.is_file() else None
 
 
+def tokenizer_eos_token_id(model_dir: str | Path | None, tokenizer: Any = None) -> int | None:
+    """The tokenizer's own end-of-sequence id: ``eos_token_id`` of the tokenizer object if it
+    has one, else ``eos_token`` of ``tokenizer_config.json`` (a string or a record with
+    ``content``) looked up in the vocabulary."""
+    eos_id = getattr(tokenizer, "eos_token_id", None)
+    if isinstance(eos_id, int):
+        return eos_id
+    from .prompting import _special_token, read_tokenizer_config
+
+    cfg = read_tokenizer_config(model_dir)
+    if isinstance(cfg.get("eos_token_id"), int):
+        return int(cfg["eos_token_id"])
+    token = _special_token(cfg.get("eos_token"))
+    if token is not None and tokenizer is not None and hasattr(tokenizer, "token_to_id"):
+        found = tokenizer.token_to_id(token)
+        if found is not None:
+            return int(found)
+    return None
+
+
 def load_stop_token_ids(model_dir: str | Path | None, config_eos=(), tokenizer: Any = None) -> set[int]:
-    """``eos_token_id`` of ``generation_config.json`` (an int or a list) and of
-    ``config.json`` (rapid_llm/engine/stop_criteria.py:29-54)."""
+    """The tokenizer's end-of-sequence id *and* ``eos_token_id`` of ``generation_config.json``
+    (an int or a list) and of ``config.json`` (rapid_llm/engine/stop_criteria.py:29-54: an
+    instruction-tuned model usually ends on another token than the tokenizer's default, so
+    both count)."""
     stop = {int(t) for t in config_eos}
+    own = tokenizer_eos_token_id(model_dir, tokenizer)
+    if own is not None:
+        stop.add(own)
     if model_dir is not None:
         path = Path(model_dir) / "generation_config.json"
         if path.is_file():

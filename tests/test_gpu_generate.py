@@ -397,6 +397,37 @@ def test_text_prompts_with_a_tokenizer(tmp_path, capsys, monkeypatch):
     assert text.count("w") > 10  # two streamed answers of six words each
 
 
+def test_template_and_stop_token_of_the_model_folder(tmp_path, capsys):
+    """``batch`` formats prompts with the folder's chat template, and a token that only
+    ``tokenizer_config.json`` names as the end of a sequence ends one."""
+    import json
+
+    from rapid_llm_amd import SamplingParams
+    from rapid_llm_amd.cli import main
+
+    cfg, page, seed = TINY["A"]
+    model_dir = make_model_dir(tmp_path, "A", "float32")
+    _word_tokenizer(model_dir, cfg["vocab_size"])
+    params = SamplingParams(temperature=0.0, max_gen_len=6)
+    free = _llm(model_dir, "float32", page, max_seq_len=64).generate(["w7 w5 w17 w3 w8"], params)[0]
+    assert free.finish_reason == "length"
+    third = free.token_ids[2]
+    (model_dir / "tokenizer_config.json").write_text(json.dumps({
+        "eos_token": f"w{third}",
+        "chat_template": "w7 {{ messages[0]['content'] }}{% if add_generation_prompt %} w8{% endif %}",
+    }))
+    stopped = _llm(model_dir, "float32", page, max_seq_len=64).generate(["w7 w5 w17 w3 w8"], params)[0]
+    assert stopped.finish_reason == "eos" and stopped.token_ids == free.token_ids[:2]
+    prompts = tmp_path / "prompts.txt"
+    prompts.write_text("w5 w17 w3\n")
+    common = ["--model-dir", str(model_dir), "--dtype", "float32", "--max-seq-len", "64", "--temperature", "0",
+              "--max-gen-len", "6", "--repetition-penalty", "1.0", "--no-cuda-graph", "--prompts-file", str(prompts)]
+    assert main(["batch", *common]) == 0
+    text = capsys.readouterr().out
+    assert "[0] eos" in text and stopped.text in text  # the template wrapped the line as the text prompt above
+    assert main(["batch", *common, "--no-chat-template"]) == 0
+
+
 def test_command_line_defaults_and_replay(tmp_path, capsys, monkeypatch):
     """``batch`` with the command line's own defaults (temperature 0.6, nucleus 0.9, penalty
     1.1, graphs, the folder from the environment) ends every request; ``replay`` writes the
