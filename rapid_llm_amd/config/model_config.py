@@ -245,10 +245,12 @@ class Qwen3Config:
                 f"num_attention_heads {self.num_attention_heads} is not divisible by "
                 f"num_key_value_heads {self.num_key_value_heads}"
             )
-        if self.head_dim % 16 or self.head_dim > 256:
+        if self.head_dim % 8 or self.head_dim > 256:
+            # the reference's rule (rapid_llm/models/config.py:357-388); multiples of 16 run on
+            # the matrix cores, the sizes between on the slower kernel that takes any size
             raise ConfigError(
                 f"head_dim {self.head_dim} is not supported: the attention kernels take "
-                "multiples of 16 up to 256"
+                "multiples of 8 up to 256"
             )
         if not self.rms_norm_eps > 0:
             raise ConfigError(f"rms_norm_eps must be positive, got {self.rms_norm_eps}")

@@ -814,13 +814,13 @@ def paged_attention(
 ) -> None:
     """Attention of every token of the step over its request's cached keys.
 
-    float32 runs the float32 matrix-core kernel (head sizes in steps of 16; the FMA kernel
-    otherwise).  bfloat16 runs the bfloat16 matrix-core kernels: single tokens go
-    to the split-key decode kernel, portions to the tiled prefill kernel."""
+    Head sizes in steps of 16 run on the matrix cores: float32 on the float32 kernel,
+    bfloat16 on the bfloat16 kernels (single tokens go to the split-key decode kernel, portions
+    to the tiled prefill kernel).  Other head sizes run the FMA kernel in either type."""
     if q.dtype == torch.float32 and d % 16 == 0:
         attention_f32(q, k_cache, v_cache, out, ctx, block_table, page_size, nq, nkv, d, window, scale)
         return
-    if q.dtype != torch.bfloat16:
+    if q.dtype != torch.bfloat16 or d % 16:
         attention_generic(
             q, k_cache, v_cache, out, ctx.positions, ctx.token_slot, block_table, page_size,
             nq, nkv, d, window, scale, ctx.max_position,

@@ -47,8 +47,8 @@ class GQAAttention(Mixer):
     ) -> None:
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not divisible by {num_kv_heads} kv heads")
-        if head_dim % 16 or not 16 <= head_dim <= 256:
-            raise ValueError(f"attention kernels take head sizes in steps of 16 up to 256, got {head_dim}")
+        if head_dim % 8 or not 8 <= head_dim <= 256:
+            raise ValueError(f"attention kernels take head sizes in steps of 8 up to 256, got {head_dim}")
         self.hidden_size = hidden_size
         self.nq, self.nkv, self.d = num_heads, num_kv_heads, head_dim
         self.prefix = checkpoint_prefix

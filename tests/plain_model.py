@@ -78,6 +78,7 @@ def plain_attention(
     window: int | None = None,
     q_positions: torch.Tensor | None = None,
     k_positions: torch.Tensor | None = None,
+    hidden: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Causal grouped-query attention of one whole sequence, dense mask.
 
@@ -89,6 +90,8 @@ def plain_attention(
     "itself included" (rapid_llm/engine/kv_cache_spec.py:203-205,222), ``p - j < w``.
     Scores are ``(q . k) * scale`` with ``scale = 1/sqrt(d)``
     (rapid_llm/modules/attention.py:62), softmax over the visible keys, then ``P @ V``.
+    ``hidden [Tq, Tk]`` (tests of the tests only) marks keys to lose on purpose: what a kernel
+    that skips them would compute.
     """
     tq, nq, d = q.shape
     tk, nkv, _ = k.shape
@@ -100,6 +103,8 @@ def plain_attention(
     visible = k_positions[None, :] <= q_positions[:, None]
     if window is not None:
         visible &= (q_positions[:, None] - k_positions[None, :]) < window
+    if hidden is not None:
+        visible = visible & ~hidden
     out = torch.empty_like(q)
     for h in range(nq):
         kh = h // group
@@ -174,8 +179,13 @@ def plain_load(model_dir: str | Path, dtype: torch.dtype = torch.float32) -> tup
     return cfg, weights
 
 
+def _same(x: torch.Tensor) -> torch.Tensor:
+    return x
+
+
 def plain_block(
-    h: torch.Tensor, cfg: dict, w: dict, layer: int, positions: torch.Tensor, window: int | None
+    h: torch.Tensor, cfg: dict, w: dict, layer: int, positions: torch.Tensor, window: int | None,
+    cast=_same, hide=None,
 ) -> torch.Tensor:
     """One pre-norm block: ``h += Attn(rms(h)); h += MLP(rms(h))``.
 
@@ -184,6 +194,11 @@ def plain_block(
     Inside attention: QKV projection (base.py:121-132), per-head q/k RMSNorm over head_dim
     *before* the rotation (base.py:134-137), rotation (base.py:139-140), attention, output
     projection (base.py:164-165).
+
+    ``cast`` is applied wherever the reference stores an activation in the model's type (the
+    residual stream stays as it is); the identity gives exact arithmetic, a round trip through
+    bfloat16 shows how far a bfloat16 engine may drift by rounding alone.  ``hide(layer,
+    q_positions, k_positions)`` returns keys to lose on purpose (see ``plain_attention``).
     """
     p = f"model.layers.{layer}."
     eps = cfg["rms_norm_eps"]
@@ -192,30 +207,36 @@ def plain_block(
     d = cfg.get("head_dim") or cfg["hidden_size"] // nq
     t = h.shape[0]
 
-    x = plain_rmsnorm(h, w[p + "input_layernorm.weight"], eps)
-    q = (x @ w[p + "self_attn.q_proj.weight"].T).view(t, nq, d)
-    k = (x @ w[p + "self_attn.k_proj.weight"].T).view(t, nkv, d)
-    v = (x @ w[p + "self_attn.v_proj.weight"].T).view(t, nkv, d)
+    x = cast(plain_rmsnorm(h, w[p + "input_layernorm.weight"], eps))
+    q = cast(x @ w[p + "self_attn.q_proj.weight"].T).view(t, nq, d)
+    k = cast(x @ w[p + "self_attn.k_proj.weight"].T).view(t, nkv, d)
+    v = cast(x @ w[p + "self_attn.v_proj.weight"].T).view(t, nkv, d)
     q = plain_rmsnorm(q, w[p + "self_attn.q_norm.weight"], eps)
     k = plain_rmsnorm(k, w[p + "self_attn.k_norm.weight"], eps)
     cos, sin = plain_rope_tables(positions, d, plain_rope_theta(cfg), h.dtype)
-    q = plain_rope_apply(q, cos, sin)
-    k = plain_rope_apply(k, cos, sin)
-    a = plain_attention(q, k, v, 1.0 / math.sqrt(d), window, positions, positions)
-    h = h + a.reshape(t, nq * d) @ w[p + "self_attn.o_proj.weight"].T
+    q = cast(plain_rope_apply(q, cos, sin))
+    k = cast(plain_rope_apply(k, cos, sin))
+    hidden = hide(layer, positions, positions) if hide is not None else None
+    a = cast(plain_attention(q, k, v, 1.0 / math.sqrt(d), window, positions, positions, hidden))
+    h = h + cast(a.reshape(t, nq * d) @ w[p + "self_attn.o_proj.weight"].T)
 
-    x = plain_rmsnorm(h, w[p + "post_attention_layernorm.weight"], eps)
-    h = h + plain_swiglu_mlp(
-        x,
-        w[p + "mlp.gate_proj.weight"],
-        w[p + "mlp.up_proj.weight"],
-        w[p + "mlp.down_proj.weight"],
-    )
-    return h
+    x = cast(plain_rmsnorm(h, w[p + "post_attention_layernorm.weight"], eps))
+    if cast is _same:
+        return h + plain_swiglu_mlp(
+            x,
+            w[p + "mlp.gate_proj.weight"],
+            w[p + "mlp.up_proj.weight"],
+            w[p + "mlp.down_proj.weight"],
+        )
+    g = cast(x @ w[p + "mlp.gate_proj.weight"].T)
+    u = cast(x @ w[p + "mlp.up_proj.weight"].T)
+    act = cast((g * torch.sigmoid(g)) * u)
+    return h + cast(act @ w[p + "mlp.down_proj.weight"].T)
 
 
 def plain_forward(
-    cfg: dict, w: dict, token_ids: list[int] | torch.Tensor, position_offset: int = 0
+    cfg: dict, w: dict, token_ids: list[int] | torch.Tensor, position_offset: int = 0,
+    cast=_same, hide=None, rows=None,
 ) -> torch.Tensor:
     """Logits ``[T, V]`` of one whole sequence.
 
@@ -223,15 +244,20 @@ def plain_forward(
     blocks, the final norm (rapid_llm/models/base.py:619-621) and the output projection,
     which reuses the embedding table when ``tie_word_embeddings`` is set and the checkpoint
     ships no ``lm_head.weight`` (rapid_llm/models/weights.py:197-214).
-    ``position_offset`` shifts every position; it exists for the invariance test.
+    ``position_offset`` shifts every position; it exists for the invariance test.  ``cast`` and
+    ``hide`` as in ``plain_block``; ``rows`` (a list of positions) limits the final norm and the
+    output projection to those rows, for vocabularies and lengths whose whole product is too
+    large to hold.
     """
     ids = torch.as_tensor(token_ids, dtype=torch.long)
     positions = torch.arange(ids.numel()) + position_offset
     h = w["model.embed_tokens.weight"][ids]
     windows = plain_layer_windows(cfg)
     for layer in range(cfg["num_hidden_layers"]):
-        h = plain_block(h, cfg, w, layer, positions, windows[layer])
-    h = plain_rmsnorm(h, w["model.norm.weight"], cfg["rms_norm_eps"])
+        h = plain_block(h, cfg, w, layer, positions, windows[layer], cast, hide)
+    if rows is not None:
+        h = h[torch.as_tensor(rows, dtype=torch.long)]
+    h = cast(plain_rmsnorm(h, w["model.norm.weight"], cfg["rms_norm_eps"]))
     head = w.get("lm_head.weight")
     if head is None:
         if not cfg.get("tie_word_embeddings", False):

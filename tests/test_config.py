@@ -71,7 +71,7 @@ def test_window_keys():
         ({"hidden_size": None}, "hidden_size"),
         ({"rms_norm_eps": None}, "rms_norm_eps"),
         ({"num_attention_heads": 3}, "not divisible"),
-        ({"head_dim": 24}, "head_dim 24"),
+        ({"head_dim": 20}, "head_dim 20"),
         ({"head_dim": 272}, "head_dim 272"),
         ({"attention_bias": True}, "attention_bias"),
         ({"hidden_act": "gelu"}, "hidden_act"),

@@ -7,6 +7,7 @@ cannot pass."""
 import pytest
 import torch
 
+import parity
 import replay_util as ru
 from plain_model import plain_forward, plain_load
 from tiny_configs import TINY, make_model_dir, random_tokens
@@ -15,8 +16,7 @@ pytestmark = pytest.mark.gpu
 
 # float32: the engine and the plain implementation differ only in summation order
 F32_TOL = dict(rtol=2e-5, atol=3e-6)
-# bfloat16: activations, cache and weights carry 8 bits of mantissa
-BF16_TOL = dict(rtol=5e-2, atol=3e-2)
+# bfloat16: bounds relative to the spread of the logits, see parity.py
 
 LENGTHS = {
     "A": [13, 17, 25, 41, 70, 100],          # prompts 1/5/13/29 + 12 decoded, and two longer
@@ -25,6 +25,7 @@ LENGTHS = {
     "D": [12, 40, 66, 150, 333, 600],
     "E": [20, 35, 49, 64, 90, 200],          # portions of 17 to 64 tokens take the mid-size product
     "F": [3, 31, 33, 64, 97, 180],           # page of 32: requests within one page, at its edge, across several
+    "G": [6, 21, 38, 75, 120, 190],          # head size 24; the window of 37 passes whole pages of 4
 }
 
 
@@ -36,11 +37,14 @@ def _requests(which):
 _PLAIN = {}
 
 
-def _plain(which, model_dir):
-    key = (which, model_dir.name)
+def _plain(which, model_dir, rounded=False):
+    """The plain implementation's logits of every request (``rounded``: with activations
+    rounded to bfloat16 where an engine stores them)."""
+    key = (which, model_dir.name, rounded)
     if key not in _PLAIN:
         cfg, w = plain_load(model_dir)
-        _PLAIN[key] = {rid: plain_forward(cfg, w, toks) for rid, toks in _requests(which).items()}
+        cast = dict(cast=parity.to_bf16) if rounded else {}
+        _PLAIN[key] = {rid: plain_forward(cfg, w, toks, **cast) for rid, toks in _requests(which).items()}
     return _PLAIN[key]
 
 
@@ -59,8 +63,16 @@ def _runner(model_dir, dtype, page, num_pages, max_seq_len):
     return runner
 
 
-def _check(got, want, dtype, label):
-    tol = F32_TOL if dtype == "float32" else BF16_TOL
+def _check(got, want, dtype, label, rounded=None):
+    if dtype != "float32":
+        # all requests as one block: one spread, the worst row of any of them
+        order = sorted(want)
+        parity.assert_bf16_close(
+            torch.cat([got[r] for r in order]), torch.cat([want[r] for r in order]), label,
+            None if rounded is None else torch.cat([rounded[r] for r in order]),
+        )
+        return
+    tol = F32_TOL
     for rid in want:
         assert got[rid].shape == want[rid].shape, (label, rid)
         assert torch.isfinite(got[rid]).all(), (label, rid)
@@ -72,13 +84,14 @@ def _check(got, want, dtype, label):
             raise AssertionError(f"{label}: request {rid}, first wrong position {first}: {exc}") from None
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F", "G"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_every_cut_matches_plain(tmp_path, which, dtype):
     cfg, page, seed = TINY[which]
     model_dir = make_model_dir(tmp_path, which, dtype)
     requests = _requests(which)
     want = _plain(which, model_dir)
+    rounded = _plain(which, model_dir, rounded=True) if dtype == "bfloat16" else None
     max_len = cfg["max_position_embeddings"]
 
     schedules = {
@@ -95,7 +108,7 @@ def test_every_cut_matches_plain(tmp_path, which, dtype):
             pages += 3
         runner = _runner(model_dir, dtype, page, pages + 1, max_len)
         got = ru.run_in_process(runner, steps)
-        _check(got, want, dtype, f"{which}/{dtype}/{label}")
+        _check(got, want, dtype, f"{which}/{dtype}/{label}", rounded)
         runner.cache.check_invariants()
         assert not runner.cache.live_requests()
         for g in runner.cache.groups:

@@ -69,8 +69,21 @@ TINY_F = dict(
 )
 PAGE_F = 32
 
+# G: a head size between the matrix cores' steps of 16 (24: the kernel that takes any size runs
+# the attention, in both types), group 3, a window on the first layer, vocabulary 257, page 4
+TINY_G = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=88, num_attention_heads=3, num_key_value_heads=1,
+    head_dim=24, intermediate_size=136, vocab_size=257, rope_theta=40000.0,
+    rms_norm_eps=5e-6, tie_word_embeddings=True, max_position_embeddings=192,
+    hidden_act="silu", attention_bias=False,
+    sliding_window=37, layer_types=["sliding_attention", "full_attention"],
+)
+PAGE_G = 4
+
 TINY = {"A": (TINY_A, PAGE_A, 11), "B": (TINY_B, PAGE_B, 22), "C": (TINY_C, PAGE_C, 33),
-        "D": (TINY_D, PAGE_D, 44), "E": (TINY_E, PAGE_E, 55), "F": (TINY_F, PAGE_F, 66)}
+        "D": (TINY_D, PAGE_D, 44), "E": (TINY_E, PAGE_E, 55), "F": (TINY_F, PAGE_F, 66),
+        "G": (TINY_G, PAGE_G, 77)}
 
 
 def make_model_dir(tmp_path: Path, which: str, dtype: str = "float32") -> Path:
