@@ -423,13 +423,14 @@ def test_template_and_stop_token_of_the_model_folder(tmp_path, capsys):
     params = SamplingParams(temperature=0.0, max_gen_len=6)
     free = _llm(model_dir, "float32", page, max_seq_len=64).generate(["w7 w5 w17 w3 w8"], params)[0]
     assert free.outputs[0].finish_reason == "length"
-    third = free.token_ids[2]
+    stop = free.token_ids[-1]
+    first = free.token_ids.index(stop)
     (model_dir / "tokenizer_config.json").write_text(json.dumps({
-        "eos_token": f"w{third}",
+        "eos_token": f"w{stop}",
         "chat_template": "w7 {{ messages[0]['content'] }}{% if add_generation_prompt %} w8{% endif %}",
     }))
     stopped = _llm(model_dir, "float32", page, max_seq_len=64).generate(["w7 w5 w17 w3 w8"], params)[0]
-    assert stopped.outputs[0].finish_reason == "eos" and stopped.token_ids == free.token_ids[:2]
+    assert stopped.outputs[0].finish_reason == "eos" and stopped.token_ids == free.token_ids[:first]
     prompts = tmp_path / "prompts.txt"
     prompts.write_text("w5 w17 w3\n")
     common = ["--model-dir", str(model_dir), "--dtype", "float32", "--max-seq-len", "64", "--temperature", "0",

@@ -37,14 +37,11 @@ def _requests(which):
 _PLAIN = {}
 
 
-def _plain(which, model_dir, rounded=False):
-    """The plain implementation's logits of every request (``rounded``: with activations
-    rounded to bfloat16 where an engine stores them)."""
-    key = (which, model_dir.name, rounded)
+def _plain(which, model_dir):
+    key = (which, model_dir.name)
     if key not in _PLAIN:
         cfg, w = plain_load(model_dir)
-        cast = dict(cast=parity.to_bf16) if rounded else {}
-        _PLAIN[key] = {rid: plain_forward(cfg, w, toks, **cast) for rid, toks in _requests(which).items()}
+        _PLAIN[key] = {rid: plain_forward(cfg, w, toks) for rid, toks in _requests(which).items()}
     return _PLAIN[key]
 
 
@@ -63,14 +60,11 @@ def _runner(model_dir, dtype, page, num_pages, max_seq_len):
     return runner
 
 
-def _check(got, want, dtype, label, rounded=None):
+def _check(got, want, dtype, label):
     if dtype != "float32":
         # all requests as one block: one spread, the worst row of any of them
         order = sorted(want)
-        parity.assert_bf16_close(
-            torch.cat([got[r] for r in order]), torch.cat([want[r] for r in order]), label,
-            None if rounded is None else torch.cat([rounded[r] for r in order]),
-        )
+        parity.assert_bf16_close(torch.cat([got[r] for r in order]), torch.cat([want[r] for r in order]), label)
         return
     tol = F32_TOL
     for rid in want:
@@ -91,7 +85,6 @@ def test_every_cut_matches_plain(tmp_path, which, dtype):
     model_dir = make_model_dir(tmp_path, which, dtype)
     requests = _requests(which)
     want = _plain(which, model_dir)
-    rounded = _plain(which, model_dir, rounded=True) if dtype == "bfloat16" else None
     max_len = cfg["max_position_embeddings"]
 
     schedules = {
@@ -108,7 +101,7 @@ def test_every_cut_matches_plain(tmp_path, which, dtype):
             pages += 3
         runner = _runner(model_dir, dtype, page, pages + 1, max_len)
         got = ru.run_in_process(runner, steps)
-        _check(got, want, dtype, f"{which}/{dtype}/{label}", rounded)
+        _check(got, want, dtype, f"{which}/{dtype}/{label}")
         runner.cache.check_invariants()
         assert not runner.cache.live_requests()
         for g in runner.cache.groups:

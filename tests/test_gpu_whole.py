@@ -30,7 +30,7 @@ def test_whole_prompts(tmp_path, which, dtype):
     model_dir = make_model_dir(tmp_path, which, dtype)
     pcfg, pw = plain_load(model_dir)
     runner = _runner(model_dir, dtype, page)
-    gots, wants, roundeds = [], [], []
+    gots, wants = [], []
     for i, n in enumerate([1, 5, 13, 29, 64, 100]):
         toks = random_tokens(n, cfg["vocab_size"], seed + i)
         want = plain_forward(pcfg, pw, toks)
@@ -41,9 +41,8 @@ def test_whole_prompts(tmp_path, which, dtype):
         else:
             gots.append(got)
             wants.append(want)
-            roundeds.append(plain_forward(pcfg, pw, toks, cast=parity.to_bf16))
     if gots:
-        parity.assert_bf16_close(torch.cat(gots), torch.cat(wants), f"whole/{which}", torch.cat(roundeds))
+        parity.assert_bf16_close(torch.cat(gots), torch.cat(wants), f"whole/{which}")
     runner.cache.check_invariants()
 
 
@@ -79,7 +78,6 @@ def test_matrices_stored_in_32_bit_stay_so_in_a_bfloat16_engine(tmp_path):
     got = [runner.step([StepEntry("r", toks[:40], list(range(40)))]).cpu()]
     for t in toks[40:]:
         got.append(runner.step([StepEntry("r", [t], [0])]).cpu())
-    # the 32-bit matrices are multiplied in 32-bit: no rounded plain result models this mix
     parity.assert_bf16_close(torch.cat(got), want, "whole/32-bit matrices beside bfloat16")
     runner.finish("r")
 
