@@ -1,0 +1,143 @@
+"""Two layers at the widths the benchmark runs (hidden 4,096, 32 query and 8 kv heads of 128,
+intermediate 12,288, an untied vocabulary of 151,936), float32 and bfloat16, against the plain
+implementation on the CPU: one 2,048-token step, portions of 512 behind a growing prefix, then
+single tokens at batch 1, 8 and 64 replayed from graphs whose context bucket is 4,096.
+
+At these widths run kernels and launch shapes that no tiny configuration reaches: the few-row
+product with two tiles of weight rows a workgroup, the output projection over 151,936 rows,
+the product for 17 to 64 rows inside a model, the fused decode kernel at head size 128 with
+keys split for a bucket of 4,096, the prefill kernel with two wave groups on a tile and with
+tiles cut into key runs.  The pattern is the reference's whole-model comparison
+(tests/cpu/test_inference.py:108-126) at the benchmark's sizes."""
+
+import pytest
+import torch
+
+import parity
+from plain_model import plain_forward, plain_load
+from tiny_configs import random_tokens
+
+pytestmark = pytest.mark.gpu
+
+CONFIG = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+    head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=4096,
+    hidden_act="silu", attention_bias=False,
+)
+PAGE = 16
+DECODE_STEPS = 2  # single-token steps at each batch size
+# float32: sums of 4,096 to 12,288 terms in another order than the plain product's
+F32_TOL = dict(rtol=1e-4, atol=5e-5)
+
+
+class _Sequences:
+    """The requests of the test: their tokens, and which positions' logits are compared."""
+
+    def __init__(self):
+        vocab = CONFIG["vocab_size"]
+        tail = 3 * DECODE_STEPS  # the longest-lived request decodes at batch 1, 8 and 64
+        self.prompt = {"a": 2048, "b": 2560, "c": 700}
+        for i in range(61):
+            self.prompt[f"s{i}"] = 3 + (i * 7) % 90
+        self.tokens = {rid: random_tokens(n + tail, vocab, 1000 + k) for k, (rid, n) in enumerate(self.prompt.items())}
+        self.rows: dict[str, list[int]] = {rid: [] for rid in self.prompt}
+
+    def want(self, rid, positions):
+        self.rows[rid].extend(positions)
+        return list(positions)
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    from rapid_llm_amd import write_random_model
+
+    folder = tmp_path_factory.mktemp("real_widths") / "two_layers"
+    write_random_model(dict(CONFIG), 7, folder, dtype="bfloat16", norm_std=0.1)
+    return folder
+
+
+def _plan(seqs):
+    """The steps of the test as (label, entries, graph) with entries (request, first position,
+    count, wanted places); positions are filled in as the plan is laid out."""
+    done = {rid: 0 for rid in seqs.prompt}
+    steps = []
+
+    def entry(rid, count, want):
+        e = (rid, done[rid], count, want)
+        seqs.want(rid, [done[rid] + w for w in want])
+        done[rid] += count
+        return e
+
+    # one 2,048-token step: the prefill kernel's two-wave-group shape; every 64th row and the end
+    steps.append(("a whole", [entry("a", 2048, list(range(0, 2048, 64)) + list(range(2040, 2048)))], False))
+    for i in range(DECODE_STEPS):
+        steps.append((f"batch 1 step {i}", [entry("a", 1, [0])], True))
+    # portions of 512: from the second on, few long tiles whose keys are cut into runs
+    for p in range(5):
+        steps.append((f"b portion {p}", [entry("b", 512, [0, 1, 255, 256, 510, 511])], False))
+    # six prompts in one step beside nothing else, then batch 8
+    firsts = ["c"] + [f"s{i}" for i in range(5)]
+    steps.append(("six prompts", [entry(r, seqs.prompt[r], [seqs.prompt[r] - 1]) for r in firsts], False))
+    eight = ["a", "b"] + firsts
+    for i in range(DECODE_STEPS):
+        steps.append((f"batch 8 step {i}", [entry(r, 1, [0]) for r in eight], True))
+    # 56 more prompts beside the eight's next tokens (portions beside decoded tokens), then batch 64
+    rest = [f"s{i}" for i in range(5, 61)]
+    steps.append(("mixed", [entry(r, 1, [0]) for r in eight] + [entry(r, seqs.prompt[r], [seqs.prompt[r] - 1]) for r in rest], False))
+    everyone = eight + rest
+    for i in range(DECODE_STEPS - 1):
+        steps.append((f"batch 64 step {i}", [entry(r, 1, [0]) for r in everyone], True))
+    return steps
+
+
+@pytest.fixture(scope="module")
+def reference(model):
+    """The plan and the plain implementation's logits at every compared position (the weights as
+    the bfloat16 checkpoint stores them, arithmetic in float32: the oracle of both engines)."""
+    seqs = _Sequences()
+    steps = _plan(seqs)
+    pcfg, pw = plain_load(model)
+    plain = {}
+    for rid, rows in seqs.rows.items():
+        length = max(rows) + 1
+        logits = plain_forward(pcfg, pw, seqs.tokens[rid][:length], rows=rows)
+        plain[rid] = {pos: logits[i] for i, pos in enumerate(rows)}
+    del pw
+    return seqs, steps, plain
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_benchmark_widths_match_plain(model, reference, dtype):
+    from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
+
+    seqs, steps, plain = reference
+    runner = ModelRunner(
+        model,
+        EngineConfig(dtype=dtype, max_seq_len=4096, page_size=PAGE, num_pages=1200, max_num_seqs=64, use_graph=True),
+    )
+    for label, entries, graph in steps:
+        before = set(runner._graphs)
+        logits = runner.step(
+            [StepEntry(rid, seqs.tokens[rid][start : start + count], want) for rid, start, count, want in entries]
+        ).cpu()
+        want = torch.stack([plain[rid][start + w] for rid, start, count, ws in entries for w in ws])
+        assert logits.shape == want.shape, label
+        if graph:
+            keys = set(runner._graphs)
+            assert keys, f"{label}: the step was not replayed from a graph"
+            bucket = {k for k in keys if k[0] >= len(entries) and k[1] == 4096}
+            assert bucket, f"{label}: no graph for {len(entries)} rows in the bucket of 4,096 ({sorted(keys)})"
+        else:
+            assert set(runner._graphs) == before, f"{label}: a step with a portion was recorded"
+        if dtype == "float32":
+            err = float((logits - want).abs().max())
+            print(f"real widths float32 {label}: worst error {err:.3e} (logits spread {float(want.std()):.3f})")
+            torch.testing.assert_close(logits, want, **F32_TOL)
+        else:
+            parity.assert_bf16_close(logits, want, f"real widths/{label}")
+    for rid in seqs.prompt:
+        runner.finish(rid)
+    runner.cache.check_invariants()
+    assert not runner.cache.live_requests()
