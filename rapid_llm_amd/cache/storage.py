@@ -33,7 +33,14 @@ class LayerCache:
     k: torch.Tensor | None  # [pages, kv_heads, page_size, head_dim]
     v: torch.Tensor | None  # [pages, kv_heads, head_dim, page_size]
     owns_pages: bool  # False: reads another layer's pages and must not write them
-    state: torch.Tensor | None  # [max_seqs + 1, *state_shape], zeroed when a slot is taken
+    # fixed-size per-request tensors by name, each [max_seqs + 1, *shape], zeroed when a slot
+    # is taken (the last row belongs to the filler slot of padded batches)
+    states: dict[str, torch.Tensor]
+
+    @property
+    def state(self) -> torch.Tensor | None:
+        """The mixer's one state tensor (the one it asked for as ``state_shape``)."""
+        return self.states.get("state")
 
 
 def plan_groups(needs: list[CacheNeed]) -> tuple[list[GroupSpec], list[int | None]]:
@@ -64,6 +71,16 @@ def plan_groups(needs: list[CacheNeed]) -> tuple[list[GroupSpec], list[int | Non
     windows = {gid: w for w, gid in keys.items()}
     groups = [GroupSpec(gid, windows[gid], tuple(layers_of[gid])) for gid in sorted(windows)]
     return groups, group_of
+
+
+def state_bytes(needs: list[CacheNeed], slots: int, elem: int) -> int:
+    """Bytes the per-request state tensors of every layer take for ``slots`` slots."""
+    total = 0
+    for need in needs:
+        for spec in need.state_specs():
+            size = getattr(torch, spec.dtype).itemsize if spec.dtype else elem
+            total += slots * int(np.prod(spec.shape, dtype=np.int64)) * size
+    return total
 
 
 def page_bytes(needs: list[CacheNeed], group_of: list[int | None], page_size: int, elem: int) -> dict[int, int]:
@@ -102,11 +119,14 @@ class DeviceCache:
                 k = torch.zeros((pages, need.num_kv_heads, P, need.head_dim), dtype=dtype, device=device)
                 v = torch.zeros((pages, need.num_kv_heads, need.head_dim, P), dtype=dtype, device=device)
                 owns = True
-            state = None
-            if need.state_shape is not None:
-                sdt = getattr(torch, need.state_dtype) if need.state_dtype else dtype
-                state = torch.zeros((manager.max_seqs + 1, *need.state_shape), dtype=sdt, device=device)
-            self.layers.append(LayerCache(i, gid, P, k, v, owns, state))
+            states = {
+                spec.name: torch.zeros(
+                    (manager.max_seqs + 1, *spec.shape),
+                    dtype=getattr(torch, spec.dtype) if spec.dtype else dtype, device=device,
+                )
+                for spec in need.state_specs()
+            }
+            self.layers.append(LayerCache(i, gid, P, k, v, owns, states))
         for i, need in enumerate(needs):
             if need.kind == "kv" and need.share_with is not None:
                 src = self.layers[need.share_with]
@@ -135,8 +155,8 @@ class DeviceCache:
         if m.fresh_slots:
             index = None
             for layer in self.layers:
-                if layer.state is not None:
+                for state in layer.states.values():
                     if index is None:
                         index = upload_ints(sorted(m.fresh_slots), self.device, np.int64)
-                    layer.state.index_fill_(0, index, 0)
+                    state.index_fill_(0, index, 0)
             m.fresh_slots.clear()

@@ -22,7 +22,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheError, CacheManager
-from ..cache.storage import DeviceCache, page_bytes, plan_groups
+from ..cache.storage import DeviceCache, page_bytes, plan_groups, state_bytes
 from ..config.engine_config import EngineConfig
 from ..config.model_config import read_config_json
 from ..config.registry import config_from_dict
@@ -79,10 +79,14 @@ class StepContext:
     max_position: int = 0
     max_seq_tokens: int = 0  # longest portion in the batch
     fed_tokens: torch.Tensor | None = None  # [rows] what the latest sampling chose (see fed_token)
-    # a step of few rows in bfloat16: parts may hand their last product on unfinished, so that
-    # the norm that follows is folded into the products around it (parts/lazy.py)
-    defer_products: bool = False
-    extra: dict[str, Any] = field(default_factory=dict)  # per-step device metadata of kernels
+    # Launch data of the parts' kernels, made on first use and shared by the layers of the step.
+    # ``static`` holds what depends only on what a recorded step fixes (the number of rows, one
+    # token a request, ``static["context_bound"]``, and in a recorded step
+    # ``static["decode_only_tokens"]``): it is kept from the eager run before a recording into the
+    # recording itself and lives as long as the graph.  ``extra`` holds anything else of one
+    # forward pass and is emptied between the two.
+    static: dict[Any, Any] = field(default_factory=dict)
+    extra: dict[Any, Any] = field(default_factory=dict)
 
 
 class ModelRunner:
@@ -144,6 +148,7 @@ class ModelRunner:
         groups, group_of = plan_groups(needs)
         elem = 4 if self.dtype == torch.float32 else 2
         self.page_bytes = page_bytes(needs, group_of, self.engine.page_size, elem)
+        self.state_bytes = state_bytes(needs, self.engine.max_num_seqs + 1, elem)
         num_pages = self._decide_num_pages(groups)
         self.cache = CacheManager(
             groups, num_pages, self.engine.page_size, self.engine.max_num_seqs, self.engine.max_seq_len
@@ -168,15 +173,43 @@ class ModelRunner:
             return e.num_pages
         if e.max_gpu_num_blocks is not None:  # the reference's knob counts tokens (README.md:121)
             return -(-e.max_gpu_num_blocks // e.page_size) + 1
-        # what is left of the device after the weights, times the utilisation, shared by
-        # the groups (rapid_llm/executor/kv_cache_manager.py:91-130)
+        # what is left of the device after the weights, times the utilisation, less what else the
+        # engine will allocate (the per-request state tensors, the recorded steps' private
+        # buffers, a step's activations), shared by the groups
+        # (rapid_llm/executor/kv_cache_manager.py:91-130)
         free, total = torch.cuda.mem_get_info(self.device)
-        budget = free - int(total * (1.0 - e.gpu_memory_utilization)) - (2 << 30)
+        reserve = self.state_bytes + self._graph_pool_estimate() + (1 << 30)
+        budget = free - int(total * (1.0 - e.gpu_memory_utilization)) - reserve
         per_page = sum(self.page_bytes.values()) or 1
-        pages = max(2, budget // per_page)
+        if budget < 2 * per_page:
+            raise ValueError(
+                f"no memory is left for the cache: {free >> 20} MiB are free, gpu_memory_utilization "
+                f"{e.gpu_memory_utilization} keeps {int(total * (1.0 - e.gpu_memory_utilization)) >> 20} MiB back, "
+                f"state tensors, recorded steps and activations take {reserve >> 20} MiB, and a page costs "
+                f"{per_page >> 10} KiB; lower max_num_seqs or max_seq_len, or give num_pages"
+            )
+        pages = budget // per_page
         # never more than every slot at full length can use
         cap = e.max_num_seqs * (-(-e.max_seq_len // e.page_size)) + 1
         return int(min(pages, cap))
+
+    def _graph_pool_estimate(self) -> int:
+        """Bytes the recorded decode steps may come to hold: every batch size of the ladder up
+        to ``max_num_seqs``, in every context bucket, keeps its float32 logits and a few rows of
+        activations."""
+        e = self.engine
+        if not (e.use_graph and self.model.replayable()):
+            return 0
+        rows = sum(b for b in GRAPH_BATCHES if b <= max(1, e.max_num_seqs)) or 1
+        buckets, bound = 1, 512
+        while bound < e.max_seq_len:
+            bound *= 2
+            buckets += 1
+        widest = max(
+            [self.spec.hidden_size]
+            + [p.shape[0] for p in self.params.values() if p.dim() == 2 and p.shape[0] != self.spec.vocab_size]
+        )
+        return rows * buckets * 4 * (self.spec.vocab_size + 8 * widest)
 
     # ------------------------------------------------------------------ requests
     def tokens_cached(self, request_id: str) -> int:
@@ -306,7 +339,6 @@ class ModelRunner:
             logit_rows=part[7],
             block_tables=self.device_cache.tables,
             fed_tokens=self.sampled,
-            defer_products=self.dtype == torch.bfloat16 and meta["num_tokens"] <= ops.MID_MAX_ROWS,
             **meta,
         )
 
@@ -354,12 +386,19 @@ class ModelRunner:
         key = (rows, bound)
         entry = self._graphs.get(key)
         if entry is None:
+            # One eager run first, on a side stream: kernels get loaded, the allocator warm, and
+            # the parts make the launch data they keep in ctx.static.  It runs filler rows only
+            # (token 0 at position 0 of the filler slot): a mixer with state of its own must not
+            # see a real request's step twice, and what the attention writes goes to the null page.
+            blank, _, _ = self._padded_decode(dict(meta, num_seqs=0, h_seq_slots=[], h_seq_starts=[]), [], rows)
             static = torch.zeros(len(host), dtype=torch.int32, device=self.device)
-            upload(host, self.device, into=static)
-            ctx = self._context(static, offs, dict(meta, max_position=bound - 1))
-            ctx.extra["decode_only_tokens"] = torch.arange(rows, dtype=torch.int32, device=self.device)
-            ctx.extra["context_bound"] = bound
-            # one eager run on a side stream first: kernels get loaded, the allocator warm
+            upload(blank, self.device, into=static)
+            filler = [self.device_cache.filler_slot] * rows
+            ctx = self._context(
+                static, offs, dict(meta, max_position=bound - 1, h_seq_slots=filler, h_seq_starts=[0] * rows)
+            )
+            ctx.static["decode_only_tokens"] = torch.arange(rows, dtype=torch.int32, device=self.device)
+            ctx.static["context_bound"] = bound
             current = torch.cuda.current_stream()
             side = torch.cuda.Stream()
             side.wait_stream(current)
@@ -367,18 +406,16 @@ class ModelRunner:
                 self.model.forward(ctx, self.device_cache.layers)
             current.wait_stream(side)
             torch.cuda.synchronize()
-            # launch data that depends on the batch's shape only was uploaded by that run and is
-            # kept: nothing may be copied from the host while the graph is recorded
-            ctx.extra = {
-                k: v for k, v in ctx.extra.items()
-                if k in ("decode_only_tokens", "context_bound") or (isinstance(k, tuple) and k[0] == "f32_tiles")
-            }
+            # what the parts left in ctx.static (launch data that depends on the step's shape
+            # only) was uploaded by that run and is kept: nothing may be copied from the host
+            # while the graph is recorded.  Everything else of that run is dropped.
+            ctx.extra = {}
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, self.device_cache.layers)
             # the graph's kernel nodes hold raw pointers: everything they point at that was
-            # allocated outside the capture (the static inputs, the index list in ctx.extra)
-            # must live as long as the graph does, so the context is kept with it
+            # allocated outside the capture (the static inputs, what ctx.static holds) must
+            # live as long as the graph does, so the context is kept with it
             entry = (graph, static, logits, ctx)
             self._graphs[key] = entry
         graph, static, logits, _ctx = entry

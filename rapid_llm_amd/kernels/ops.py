@@ -626,7 +626,7 @@ class AttentionPlan:
                  "_prefill_tokens", "_prefill_list")
 
     def __init__(self, ctx, group: int, tile_rows: int) -> None:
-        fixed = ctx.extra.get("decode_only_tokens")
+        fixed = _static(ctx).get("decode_only_tokens")
         if fixed is not None:
             # a step of single tokens whose index list is already on the device (graphs)
             self.num_decode = fixed.numel()
@@ -736,11 +736,20 @@ def _prefill_shape(plan: "AttentionPlan", nkv: int, window: int, tile_rows: int)
     return (2 if paired < max(longest_steps, share) else 1), nsplit
 
 
+def _static(ctx) -> dict:
+    """Where launch data that depends on the step's shape alone is kept (``StepContext.static``:
+    it survives from the eager run before a recording into the recording)."""
+    static = getattr(ctx, "static", None)
+    return ctx.extra if static is None else static
+
+
 def _f32_tiles(ctx, group: int) -> tuple[torch.Tensor, int]:
     """Tiles of 16 (token, head of the group) rows, request by request: ``[tiles, 3]`` int32
-    (first token of the request in the step, its tokens, first row of the tile)."""
+    (first token of the request in the step, its tokens, first row of the tile).  A function of
+    the requests' token counts alone."""
     key = ("f32_tiles", group)
-    made = ctx.extra.get(key)
+    store = _static(ctx)
+    made = store.get(key)
     if made is None:
         tiles: list[int] = []
         at = 0
@@ -749,7 +758,7 @@ def _f32_tiles(ctx, group: int) -> tuple[torch.Tensor, int]:
                 tiles += [at, n, row0]
             at += n
         made = (upload_ints(tiles, ctx.token_ids.device), len(tiles) // 3)
-        ctx.extra[key] = made
+        store[key] = made
     return made
 
 
@@ -885,7 +894,7 @@ def _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_s
     ``q`` the packed [q | k | v] rows."""
     group = nq // nkv
     # under a graph the split is laid out for the longest context of the graph's bucket
-    span = ctx.extra.get("context_bound", plan.max_decode_ctx)
+    span = _static(ctx).get("context_bound", plan.max_decode_ctx)
     if window > 0:
         span = min(span, window + 31)
     chunks = (group + 15) // 16

@@ -10,16 +10,19 @@ from __future__ import annotations
 
 import torch
 
+from dataclasses import replace
+
 from ..parts.base import (
     BLOCKS,
+    EMBEDDINGS,
     FEED_FORWARDS,
     MIXERS,
     NORMS,
+    OUTPUT_PROJECTIONS,
     POSITION_ENCODINGS,
     CacheNeed,
     ParamSpec,
 )
-from ..parts.embedding import OutputProjection, TokenEmbedding
 from ..parts.lazy import plain, run_norm
 from .spec import ModelSpec
 
@@ -29,13 +32,8 @@ class CausalLM:
         import rapid_llm_amd.parts  # noqa: F401  registers the built-in part kinds
 
         self.spec = spec
-        self.embed = TokenEmbedding(spec.vocab_size, spec.hidden_size, spec.embedding_source)
-        self.output = OutputProjection(
-            spec.vocab_size,
-            spec.hidden_size,
-            spec.output_source,
-            tied_to="embed.weight" if spec.tie_output_to_embedding else None,
-        )
+        self.embed = EMBEDDINGS.create(spec.embedding.kind, **spec.embedding.params, name="embed")
+        self.output = OUTPUT_PROJECTIONS.create(spec.output.kind, **spec.output.params, name="output")
         self.final_norm = NORMS.create(spec.final_norm.kind, **spec.final_norm.params, name="final_norm")
         self.order = list(spec.order())
         for li in self.order:
@@ -111,10 +109,7 @@ class CausalLM:
                     raise ValueError(
                         f"layer {li} reads the cache of layer {share}, which has not run before it"
                     )
-                need = CacheNeed(
-                    need.kind, need.window, need.num_kv_heads, need.head_dim,
-                    need.state_shape, need.state_dtype, last_place[share],
-                )
+                need = replace(need, share_with=last_place[share])
             needs.append(need)
             last_place[li] = place
         return needs
@@ -123,7 +118,7 @@ class CausalLM:
     def forward(self, ctx, caches) -> torch.Tensor:
         """Run the tokens of ``ctx`` through every layer (which writes their keys and values)
         and return float32 logits ``[len(ctx.logit_rows), vocab]``."""
-        residual = self.embed.forward(ctx.token_ids, ctx.fed_tokens)
+        residual = self.embed.forward(ctx.token_ids, ctx)
         delta = None
         for place, li in enumerate(self.order):
             block = self.blocks[li]
@@ -133,7 +128,7 @@ class CausalLM:
         if ctx.num_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=residual.device)
         h = run_norm(self.final_norm, residual, delta, ctx, rows=ctx.logit_rows)
-        return self.output.forward(h)
+        return self.output.forward(h, ctx)
 
 
 def model_param_specs(spec: ModelSpec) -> list[ParamSpec]:

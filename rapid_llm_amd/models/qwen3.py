@@ -10,7 +10,7 @@ from __future__ import annotations
 
 from ..config.model_config import Qwen3Config
 from ..config.registry import register_architecture
-from .spec import IgnoreRule, LayerSpec, ModelSpec, PartSpec
+from .spec import IgnoreRule, LayerSpec, ModelSpec, PartSpec, linear_output, token_embedding
 
 
 def build_qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
@@ -72,9 +72,8 @@ def build_qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
             "rmsnorm",
             {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps, "checkpoint_name": "model.norm.weight"},
         ),
-        embedding_source="model.embed_tokens.weight",
-        output_source="lm_head.weight",
-        tie_output_to_embedding=cfg.tie_word_embeddings,
+        embedding=token_embedding(cfg.vocab_size, cfg.hidden_size, "model.embed_tokens.weight"),
+        output=linear_output(cfg.vocab_size, cfg.hidden_size, "lm_head.weight", cfg.tie_word_embeddings),
         # layers beyond num_hidden_layers are dropped unread (base.py:494-497), so a
         # layer-trimmed config.json still loads the full checkpoint
         ignore_tensors=(

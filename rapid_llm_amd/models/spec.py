@@ -2,9 +2,9 @@
 
 An architecture's builder turns its typed configuration into a :class:`ModelSpec`:
 which mixer, feed-forward, norms and block each layer has (chosen layer by layer, each
-with its own parameters), and the order in which layers run.  The order is data too:
-``run_order`` may name a layer twice, and a layer may read another layer's cache
-(``LayerSpec.share_cache_with``).
+with its own parameters), which embedding and output projection stand at its two ends,
+and the order in which layers run.  The order is data too: ``run_order`` may name a layer
+twice, and a layer may read another layer's cache (``LayerSpec.share_cache_with``).
 """
 
 from __future__ import annotations
@@ -42,15 +42,31 @@ class LayerSpec:
     share_cache_with: int | None = None  # index of the layer whose cache this one reads
 
 
+def token_embedding(vocab_size: int, hidden_size: int, checkpoint_name: str) -> PartSpec:
+    """The plain table lookup."""
+    return PartSpec(
+        "token_embedding", {"vocab_size": vocab_size, "hidden_size": hidden_size, "checkpoint_name": checkpoint_name}
+    )
+
+
+def linear_output(vocab_size: int, hidden_size: int, checkpoint_name: str, tied: bool) -> PartSpec:
+    """The plain product with a ``[vocab, hidden]`` matrix; ``tied``: the embedding's table
+    stands in when the checkpoint ships none (the embedding part's parameter is ``embed.weight``)."""
+    return PartSpec(
+        "linear_output",
+        {"vocab_size": vocab_size, "hidden_size": hidden_size, "checkpoint_name": checkpoint_name,
+         "tied_to": "embed.weight" if tied else None},
+    )
+
+
 @dataclass(frozen=True)
 class ModelSpec:
     hidden_size: int
     vocab_size: int
     layers: tuple[LayerSpec, ...]
     final_norm: PartSpec
-    embedding_source: str  # checkpoint name of the embedding table
-    output_source: str  # checkpoint name of the output projection
-    tie_output_to_embedding: bool
+    embedding: PartSpec  # built with name="embed"
+    output: PartSpec  # built with name="output"
     run_order: tuple[int, ...] | None = None  # None: 0..len(layers)-1
     ignore_tensors: tuple[IgnoreRule, ...] = ()
     max_position: int = 0  # largest position the architecture is defined for (0: unbounded)

@@ -10,6 +10,8 @@ model it sits in.  Five kinds exist:
 * ``Norm``: normalisation, fused with the residual add in front of it.
 * ``PositionEncoding``: what a mixer consults to encode positions (rotation tables here).
 * ``Block``: the arrangement of mixer, feed-forward and norms around the residual stream.
+* ``Embedding`` and ``OutputProjection``: the two ends of the model, token ids to the
+  residual stream and the last hidden rows to logits.
 
 Every part declares its tensors as :class:`ParamSpec` (``param_specs``), receives them
 loaded (``bind``), and runs on a flat batch of tokens described by a
@@ -70,13 +72,24 @@ class ParamSpec:
 
 
 @dataclass(frozen=True)
+class StateSpec:
+    """One fixed-size per-request tensor: ``[slots, *shape]`` on the device."""
+
+    name: str
+    shape: tuple[int, ...]
+    dtype: str | None = None  # torch dtype name; None: the engine's compute type
+
+
+@dataclass(frozen=True)
 class CacheNeed:
     """What a mixer asks of the cache manager.
 
     ``kind == "kv"``: paged keys and values; ``window`` 0 keeps every position, otherwise
     only the last ``window`` positions of a request are kept and older pages are given back.
-    ``kind == "state"``: nothing paged.  ``state_shape`` (may accompany either kind) is a
-    fixed-size per-request tensor the mixer owns, zeroed when a request takes the slot.
+    ``kind == "state"``: nothing paged.  Fixed-size per-request tensors the mixer owns, zeroed
+    when a request takes the slot, may accompany either kind: one as ``state_shape`` (and
+    ``state_dtype``), or several, each under a name, as ``states`` (a mixer with a short
+    convolution's tail beside a recurrent state names both).
     ``share_with`` names the place in the run order whose cache this one reads instead of
     writing its own.
     """
@@ -88,6 +101,16 @@ class CacheNeed:
     state_shape: tuple[int, ...] | None = None
     state_dtype: str | None = None  # torch dtype name; None: the engine's compute type
     share_with: int | None = None
+    states: tuple[StateSpec, ...] = ()
+
+    def state_specs(self) -> tuple[StateSpec, ...]:
+        """Every per-request tensor asked for; the one given as ``state_shape`` is named ``"state"``."""
+        single = (StateSpec("state", self.state_shape, self.state_dtype),) if self.state_shape is not None else ()
+        specs = single + tuple(self.states)
+        names = [s.name for s in specs]
+        if len(names) != len(set(names)):
+            raise ValueError(f"a mixer names two state tensors alike: {names}")
+        return specs
 
 
 class Part:
@@ -95,11 +118,16 @@ class Part:
 
     #: A part whose ``forward`` may be recorded once into a HIP graph and replayed for later
     #: steps declares ``replayable = True``.  It promises that everything ``forward`` does on
-    #: the host depends only on what is fixed for a recorded step (the number of rows, the
-    #: context bound in ``ctx.extra["context_bound"]``), that every per-step value (ids,
-    #: positions, slots, block tables, state) is read on the device from the tensors of
-    #: ``ctx`` and of the cache, and that nothing waits for the device or copies from the host.
-    #: A model with a part that does not declare it runs every step eagerly.
+    #: the host depends only on what is fixed for a recorded step (the number of rows, that
+    #: every request brings one token, the context bound in ``ctx.static["context_bound"]``),
+    #: that every per-step value (ids, positions, slots, block tables, state) is read on the
+    #: device from the tensors of ``ctx`` and of the cache, and that nothing waits for the
+    #: device or copies from the host while the step is recorded.  Launch data that depends
+    #: only on what a recorded step fixes (index lists, tile tables) is kept in ``ctx.static``:
+    #: the step runs once eagerly before it is recorded, what that run left in ``ctx.static`` is
+    #: there again during the recording and lives as long as the graph, whereas ``ctx.extra`` is
+    #: emptied between the two.  A model with a part that does not declare it runs every step
+    #: eagerly.
     replayable = False
 
     def param_specs(self) -> list[ParamSpec]:
@@ -152,6 +180,23 @@ class Block(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """Token ids to the float32 residual stream."""
+
+    def forward(self, token_ids: "torch.Tensor", ctx: "StepContext") -> "torch.Tensor":
+        """``token_ids [T]`` int32 -> ``[T, hidden]`` float32.  An id ``-(r + 1)`` stands for
+        ``ctx.fed_tokens[r]``, the token that row ``r`` of the latest sampling chose on the
+        device (:func:`~rapid_llm_amd.engine.feed.fed_token`)."""
+        raise NotImplementedError
+
+
+class OutputProjection(Part):
+    """The normalised hidden rows that were asked for to float32 logits ``[rows, vocab]``."""
+
+    def forward(self, h: "torch.Tensor", ctx: "StepContext") -> "torch.Tensor":
+        raise NotImplementedError
+
+
 # --------------------------------------------------------------------------- #
 # registries: kind name -> constructor
 # --------------------------------------------------------------------------- #
@@ -192,3 +237,5 @@ FEED_FORWARDS = PartRegistry("feed-forward")
 NORMS = PartRegistry("norm")
 POSITION_ENCODINGS = PartRegistry("position encoding")
 BLOCKS = PartRegistry("block")
+EMBEDDINGS = PartRegistry("embedding")
+OUTPUT_PROJECTIONS = PartRegistry("output projection")

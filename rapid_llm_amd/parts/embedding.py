@@ -10,11 +10,11 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import ParamSpec, Part, Source
+from .base import EMBEDDINGS, OUTPUT_PROJECTIONS, Embedding, OutputProjection, ParamSpec, Source
 from .linear import Linear
 
 
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     replayable = True
 
     def __init__(self, vocab_size: int, hidden_size: int, checkpoint_name: str, name: str = "embed") -> None:
@@ -36,15 +36,17 @@ class TokenEmbedding(Part):
     def bind(self, params, runtime) -> None:
         self.table = params[self.name + ".weight"]
 
-    def forward(self, token_ids: torch.Tensor, fed_tokens: torch.Tensor | None = None) -> torch.Tensor:
-        """Rows of the table for the ids; an id ``-(r + 1)`` takes ``fed_tokens[r]``."""
+    def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
+        """Rows of the table for the ids; an id ``-(r + 1)`` takes ``ctx.fed_tokens[r]``."""
         out = torch.empty((token_ids.numel(), self.hidden_size), dtype=torch.float32, device=token_ids.device)
-        ops.embed(token_ids, self.table, out, fed_tokens)
+        ops.embed(token_ids, self.table, out, getattr(ctx, "fed_tokens", None))
         return out
 
 
-class OutputProjection(Part):
-    """``logits = h W^T`` in float32, over the rows that were asked for only."""
+class LinearOutput(OutputProjection):
+    """``logits = h W^T`` in float32, over the rows that were asked for only.  ``tied_to``
+    names the parameter (the embedding's table) that stands in when the checkpoint ships no
+    tensor of this part's own."""
 
     replayable = True
 
@@ -76,5 +78,9 @@ class OutputProjection(Part):
     def bind(self, params, runtime) -> None:
         self.proj.bind(params[self.name + ".weight"])
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, ctx=None) -> torch.Tensor:
         return self.proj(h, out_dtype=torch.float32)
+
+
+EMBEDDINGS.register("token_embedding", TokenEmbedding)
+OUTPUT_PROJECTIONS.register("linear_output", LinearOutput)

@@ -5,8 +5,9 @@ the smallest: it only has to know every row's sum of squares.  Two lazy values l
 products on either side absorb it, without any part knowing its neighbours:
 
 * :class:`DeferredProduct`: what a mixer or a feed-forward returns in place of its last
-  product ``x W^T`` when the step allows it.  Whoever receives it may run the product with
-  an epilogue of its own, or simply ``materialize()`` it.
+  product ``x W^T`` when that product's own kernels could absorb a norm (``Linear.deferred``
+  decides: bfloat16 and few rows).  Whoever receives it may run the product with an epilogue
+  of its own, or simply ``materialize()`` it.
 * :class:`ScaledRows`: what a norm returns in place of normalised rows when its consumer
   says it accepts them: the rows times the norm's weight, and the pieces of every row's sum
   of squares; the factor ``rsqrt(mean + eps)`` is a scalar per row and commutes with the

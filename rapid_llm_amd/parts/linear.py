@@ -59,10 +59,11 @@ class Linear:
         """``[runs, M, out]`` float32 whose sum over the runs is ``x W^T``."""
         return ops.gemm_bf16_parts(x, self.weight)
 
-    def deferred(self, x: torch.Tensor, ctx):
-        """The product, or a :class:`DeferredProduct` of it where the step allows it."""
-        allowed = getattr(ctx, "defer_products", False) and isinstance(x, torch.Tensor)
-        if allowed and (self.skinny(x) or self.midsize(x)):
+    def deferred(self, x: torch.Tensor, ctx=None):
+        """The product, or a :class:`DeferredProduct` of it where one of this product's kernels
+        could fold a neighbouring norm into itself (bfloat16, up to 16 rows, or 17 to 64 rows of a
+        narrow matrix).  Whoever receives it and has no use for that simply materialises it."""
+        if isinstance(x, torch.Tensor) and (self.skinny(x) or self.midsize(x)):
             return DeferredProduct(self, x)
         return self(x)
 

@@ -9,6 +9,7 @@ from dataclasses import dataclass
 import pytest
 import torch
 
+import parity
 from plain_model import (
     plain_attention,
     plain_load,
@@ -62,7 +63,7 @@ def test_parts_alone(tmp_path, which, dtype):
     model = runner.model
 
     # ---- embedding: a row gather into the float32 stream --------------------------------
-    emb = model.embed.forward(ctx.token_ids).cpu()
+    emb = model.embed.forward(ctx.token_ids, ctx).cpu()
     ids = [t for e in entries for t in e.tokens]
     assert emb.dtype == torch.float32
     torch.testing.assert_close(emb, w["model.embed_tokens.weight"][torch.tensor(ids)], rtol=0, atol=0)
@@ -112,7 +113,7 @@ def test_parts_alone(tmp_path, which, dtype):
 
     # ---- output projection -------------------------------------------------------------------
     h = torch.randn(3, H, generator=gen).to(tdt)
-    logits = model.output.forward(h.cuda()).cpu()
+    logits = model.output.forward(h.cuda(), ctx).cpu()
     head = w.get("lm_head.weight", w["model.embed_tokens.weight"])
     assert logits.dtype == torch.float32
     torch.testing.assert_close(logits, h.float() @ head.T, **tol)
@@ -135,18 +136,24 @@ class ToyConfig:
     experts: int = 0  # > 0: layer 0's feed-forward routes every token to one of so many experts
     period: float = 0.0  # > 0: the toy mixer adds a phase of the position to its input
     toynorm: bool = False  # layer 1 uses a norm defined here, which knows nothing of unfinished products
+    ends: bool = False  # an embedding that scales its rows and an output projection that caps its logits
+    replay: bool = False  # the toy mixer runs on the device alone and declares itself replayable
 
     @classmethod
     def from_dict(cls, data, overrides=None):
         return cls(data["hidden"], data["vocab"], data["heads"], data["head_dim"], data["inter"],
                    data["decay"], data.get("twice", False), data.get("share", False),
-                   data.get("experts", 0), data.get("period", 0.0), data.get("toynorm", False))
+                   data.get("experts", 0), data.get("period", 0.0), data.get("toynorm", False),
+                   data.get("ends", False), data.get("replay", False))
 
     def to_dict(self):
         return dict(architectures=["ToyForCausalLM"], hidden=self.hidden, vocab=self.vocab, heads=self.heads,
                     head_dim=self.head_dim, inter=self.inter, decay=self.decay, twice=self.twice,
                     share=self.share, experts=self.experts, period=self.period, toynorm=self.toynorm,
-                    torch_dtype="float32")
+                    ends=self.ends, replay=self.replay, torch_dtype="float32")
+
+
+CAP = 0.3  # the toy output projection's cap: logits = CAP * tanh(h W^T / CAP)
 
 
 def _phase(positions, period, size):
@@ -156,11 +163,52 @@ def _phase(positions, period, size):
 
 
 def _toy_parts():
+    from rapid_llm_amd.kernels.upload import upload_ints
     from rapid_llm_amd.parts import (
-        FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheNeed, FeedForward, Mixer, Norm, ParamSpec,
-        PositionEncoding, Source,
+        EMBEDDINGS, FEED_FORWARDS, MIXERS, NORMS, OUTPUT_PROJECTIONS, POSITION_ENCODINGS, CacheNeed, Embedding,
+        FeedForward, Mixer, Norm, OutputProjection, ParamSpec, PositionEncoding, Source, StateSpec,
     )
     from rapid_llm_amd.parts.linear import Linear
+
+    class ScaledEmbedding(Embedding):
+        """Rows of the table times sqrt(hidden), with tensor operations; tokens still on the
+        device (negative ids) are looked up in the buffer the sampling kernels write."""
+
+        replayable = True
+
+        def __init__(self, vocab_size, hidden_size, checkpoint_name, name="embed"):
+            self.v, self.h, self.checkpoint_name, self.name = vocab_size, hidden_size, checkpoint_name, name
+
+        def param_specs(self):
+            return [ParamSpec(self.name + ".weight", (self.v, self.h), "matrix", (Source(self.checkpoint_name, self.v),))]
+
+        def bind(self, params, runtime):
+            self.table = params[self.name + ".weight"]
+
+        def forward(self, token_ids, ctx):
+            ids = token_ids.long()
+            fed = ctx.fed_tokens.long()
+            ids = torch.where(ids < 0, fed[(-ids - 1).clamp(min=0, max=fed.numel() - 1)], ids)
+            return self.table[ids].float() * math.sqrt(self.h)
+
+    class CappedOutput(OutputProjection):
+        replayable = True
+
+        def __init__(self, vocab_size, hidden_size, checkpoint_name, cap, name="output"):
+            self.v, self.h, self.checkpoint_name, self.cap, self.name = vocab_size, hidden_size, checkpoint_name, cap, name
+            self.proj = Linear(hidden_size, vocab_size)
+
+        def param_specs(self):
+            return [ParamSpec(self.name + ".weight", (self.v, self.h), "matrix", (Source(self.checkpoint_name, self.v),))]
+
+        def bind(self, params, runtime):
+            self.proj.bind(params[self.name + ".weight"])
+
+        def forward(self, h, ctx):
+            return self.cap * torch.tanh(self.proj(h, out_dtype=torch.float32) / self.cap)
+
+    EMBEDDINGS.register("toy_scaled_embedding", ScaledEmbedding, replace=True)
+    OUTPUT_PROJECTIONS.register("toy_capped_output", CappedOutput, replace=True)
 
     class PlainTorchNorm(Norm):
         """The same formula as the built-in norm, written with tensor operations: it declares
@@ -268,9 +316,61 @@ def _toy_parts():
 
     MIXERS.register("toy_decaying_sum", DecayingSum, replace=True)
 
+    class DeviceDecayingSum(Mixer):
+        """The same recurrence with two state tensors of its own (the sum, and how many tokens
+        went into it), run by device operations alone: a step of single tokens updates the slots of
+        all its requests at once and may be recorded.  The per-row decay it multiplies with is
+        launch data that depends on the number of rows only: it is uploaded once and kept in
+        ``ctx.static``, where the recording finds it again."""
+
+        replayable = True
+        uploads = 0  # how often the launch data was made (the test counts)
+
+        def __init__(self, hidden_size, decay, checkpoint_prefix, position=None, name="mixer"):
+            self.h, self.decay, self.prefix, self.name = hidden_size, decay, checkpoint_prefix, name
+            self.proj = Linear(hidden_size, hidden_size)
+
+        def param_specs(self):
+            return [ParamSpec(self.name + ".w", (self.h, self.h), "matrix", (Source(self.prefix + "w", self.h),))]
+
+        def bind(self, params, runtime):
+            self.proj.bind(params[self.name + ".w"])
+
+        def cache_need(self):
+            return CacheNeed("state", states=(StateSpec("sum", (self.h,), "float32"), StateSpec("count", (1,), "int32")))
+
+        def forward(self, x, ctx, cache):
+            total, count = cache.states["sum"], cache.states["count"]
+            slots = ctx.token_slot.long()
+            if ctx.max_seq_tokens == 1:  # fixed for a recorded step
+                key = ("toy_decay_rows", x.shape[0])
+                rows = ctx.static.get(key)
+                if rows is None:
+                    type(self).uploads += 1
+                    milli = upload_ints([int(round(self.decay * 1000))] * x.shape[0], x.device)
+                    rows = ctx.static[key] = (milli.float() / 1000.0)[:, None]
+                s = total[slots] * rows + x.float()
+                total.index_copy_(0, slots, s)
+                count.index_copy_(0, slots, count[slots] + 1)
+                return self.proj(s.to(x.dtype))
+            out = torch.empty_like(x, dtype=torch.float32)  # portions: never recorded, host lists are fine
+            at = 0
+            for slot, n in zip(ctx.h_seq_slots, ctx.h_seq_lens):
+                s = total[slot]
+                for t in range(at, at + n):
+                    s = self.decay * s + x[t].float()
+                    out[t] = s
+                total[slot] = s
+                count[slot] += n
+                at += n
+            return self.proj(out.to(x.dtype))
+
+    MIXERS.register("toy_device_decaying_sum", DeviceDecayingSum, replace=True)
+    return DeviceDecayingSum
+
 
 def _toy_spec(cfg: ToyConfig):
-    from rapid_llm_amd.models import LayerSpec, ModelSpec, PartSpec
+    from rapid_llm_amd.models import LayerSpec, ModelSpec, PartSpec, linear_output, token_embedding
 
     def norm(name):
         return PartSpec("rmsnorm", {"size": cfg.hidden, "eps": 1e-5, "checkpoint_name": name})
@@ -296,21 +396,29 @@ def _toy_spec(cfg: ToyConfig):
         return norm(name)
 
     layers = [
-        LayerSpec(PartSpec("toy_decaying_sum", {"hidden_size": cfg.hidden, "decay": cfg.decay,
-                                                "checkpoint_prefix": "l0.mix."}), ff0, norm("l0.n1"), norm("l0.n2"),
-                  position=pos0),
+        LayerSpec(PartSpec("toy_device_decaying_sum" if cfg.replay else "toy_decaying_sum",
+                           {"hidden_size": cfg.hidden, "decay": cfg.decay, "checkpoint_prefix": "l0.mix."}),
+                  ff0, norm("l0.n1"), norm("l0.n2"), position=pos0),
         LayerSpec(attn(1), ff(1), norm1("l1.n1"), norm1("l1.n2"), position=rope),
     ]
     if cfg.share:
         layers.append(LayerSpec(attn(2), ff(2), norm("l2.n1"), norm("l2.n2"), position=rope, share_cache_with=1))
     order = (0, 1, 0, 1) if cfg.twice else None
-    return ModelSpec(cfg.hidden, cfg.vocab, tuple(layers), norm("final"), "embed", "head", False, run_order=order)
+    embedding, output = token_embedding(cfg.vocab, cfg.hidden, "embed"), linear_output(cfg.vocab, cfg.hidden, "head", False)
+    if cfg.ends:
+        embedding = PartSpec("toy_scaled_embedding", {"vocab_size": cfg.vocab, "hidden_size": cfg.hidden,
+                                                      "checkpoint_name": "embed"})
+        output = PartSpec("toy_capped_output", {"vocab_size": cfg.vocab, "hidden_size": cfg.hidden,
+                                                "checkpoint_name": "head", "cap": CAP})
+    return ModelSpec(cfg.hidden, cfg.vocab, tuple(layers), norm("final"), embedding, output, run_order=order)
 
 
 def _toy_plain(w, cfg: ToyConfig, toks):
     """The toy model, whole sequence, in plain torch."""
     t = len(toks)
     h = w["embed"][torch.tensor(toks)]
+    if cfg.ends:
+        h = h * math.sqrt(cfg.hidden)
     pos = torch.arange(t)
 
     def ffn(i, h):
@@ -360,20 +468,36 @@ def _toy_plain(w, cfg: ToyConfig, toks):
         h = attn(1, h)
         if cfg.share:
             h = attn(2, h, kv)  # reads the keys and values layer 1 wrote
-    return plain_rmsnorm(h, w["final"], 1e-5) @ w["head"].T
+    logits = plain_rmsnorm(h, w["final"], 1e-5) @ w["head"].T
+    return CAP * torch.tanh(logits / CAP) if cfg.ends else logits
+
+
+def _unregister_toys():
+    from rapid_llm_amd.config import unregister_architecture
+    from rapid_llm_amd.parts import EMBEDDINGS, FEED_FORWARDS, MIXERS, NORMS, OUTPUT_PROJECTIONS, POSITION_ENCODINGS
+
+    unregister_architecture("ToyForCausalLM")
+    MIXERS.unregister("toy_decaying_sum")
+    MIXERS.unregister("toy_device_decaying_sum")
+    FEED_FORWARDS.unregister("toy_routed")
+    POSITION_ENCODINGS.unregister("toy_phase")
+    NORMS.unregister("toy_plain_norm")
+    EMBEDDINGS.unregister("toy_scaled_embedding")
+    OUTPUT_PROJECTIONS.unregister("toy_capped_output")
 
 
 @pytest.mark.parametrize("variant,dtype", [("plain", "float32"), ("twice", "float32"), ("share", "float32"),
-                                           ("routed", "float32"), ("toynorm", "float32"),
-                                           ("routed", "bfloat16"), ("toynorm", "bfloat16"), ("twice", "bfloat16")])
+                                           ("routed", "float32"), ("toynorm", "float32"), ("ends", "float32"),
+                                           ("replay", "float32"),
+                                           ("routed", "bfloat16"), ("toynorm", "bfloat16"), ("twice", "bfloat16"),
+                                           ("ends", "bfloat16")])
 def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
     """In bfloat16 the built-in parts hand unfinished products and unscaled rows to each other
     in steps of few tokens; the toy parts declare nothing and must only ever see tensors."""
     from safetensors.torch import load_file
 
     from rapid_llm_amd import StepEntry, write_random_model
-    from rapid_llm_amd.config import register_architecture, unregister_architecture
-    from rapid_llm_amd.parts import FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS
+    from rapid_llm_amd.config import register_architecture
 
     _toy_parts()
     register_architecture("ToyForCausalLM", ToyConfig, _toy_spec, replace=True)
@@ -381,7 +505,7 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
         cfg = ToyConfig(hidden=48, vocab=97, heads=3, head_dim=16, inter=80, decay=0.8,
                         twice=variant == "twice", share=variant == "share",
                         experts=3 if variant == "routed" else 0, period=9.0 if variant == "routed" else 0.0,
-                        toynorm=variant == "toynorm")
+                        toynorm=variant == "toynorm", ends=variant == "ends", replay=variant == "replay")
         folder = write_random_model(cfg.to_dict(), 3, tmp_path / "toy", dtype=dtype)
         weights = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
         if variant == "share":  # the sharing layer's own k/v projections exist but are never used
@@ -391,6 +515,14 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
         if variant == "toynorm":
             assert type(runner.model.blocks[1].mixer_norm).__name__ == "PlainTorchNorm"
         assert needs[0].kind == "state" and needs[1].kind == "kv"
+        if variant == "ends":
+            assert type(runner.model.embed).__name__ == "ScaledEmbedding"
+            assert type(runner.model.output).__name__ == "CappedOutput"
+        if variant == "replay":
+            states = runner.device_cache.layers[0].states
+            assert set(states) == {"sum", "count"} and states["count"].dtype == torch.int32
+            assert states["sum"].shape == (5, cfg.hidden) and runner.device_cache.layers[0].state is None
+            assert runner.state_bytes == 5 * (cfg.hidden * 4 + 4)
         if variant == "routed":
             assert type(runner.model.blocks[0].feed_forward).__name__ == "RoutedFF"
             assert type(runner.model.blocks[1].feed_forward).__name__ == "SwiGLU"
@@ -427,17 +559,19 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
                     for e in entries:
                         got[e.request_id].append(logits[at : at + len(e.tokens)])
                         at += len(e.tokens)
+            if variant == "replay":
+                counts = runner.device_cache.layers[0].states["count"].cpu()
+                for rid, toks in reqs.items():
+                    assert int(counts[runner.cache.slot_of(rid)]) == len(toks)
             for rid in reqs:
-                tol = dict(rtol=2e-5, atol=3e-6) if dtype == "float32" else dict(rtol=5e-2, atol=5e-2)
-                torch.testing.assert_close(torch.cat(got[rid]), want[rid], **tol)
+                if dtype == "float32":
+                    torch.testing.assert_close(torch.cat(got[rid]), want[rid], rtol=2e-5, atol=3e-6)
+                else:
+                    parity.assert_bf16_close(torch.cat(got[rid]), want[rid], f"toy/{variant}/{cut}/{rid}")
                 runner.finish(rid)  # the slot's state is cleared for whoever takes it next
         runner.cache.check_invariants()
     finally:
-        unregister_architecture("ToyForCausalLM")
-        MIXERS.unregister("toy_decaying_sum")
-        FEED_FORWARDS.unregister("toy_routed")
-        POSITION_ENCODINGS.unregister("toy_phase")
-        NORMS.unregister("toy_plain_norm")
+        _unregister_toys()
 
 
 def test_toy_architecture_generates_through_the_entry_point(tmp_path):
@@ -447,8 +581,7 @@ def test_toy_architecture_generates_through_the_entry_point(tmp_path):
     from safetensors.torch import load_file
 
     from rapid_llm_amd import LLM, SamplingParams, write_random_model
-    from rapid_llm_amd.config import register_architecture, unregister_architecture
-    from rapid_llm_amd.parts import FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS
+    from rapid_llm_amd.config import register_architecture
 
     _toy_parts()
     register_architecture("ToyForCausalLM", ToyConfig, _toy_spec, replace=True)
@@ -471,17 +604,56 @@ def test_toy_architecture_generates_through_the_entry_point(tmp_path):
             assert out.outputs[0].token_ids == toks[len(prompt):]
         runner.cache.check_invariants()
     finally:
-        unregister_architecture("ToyForCausalLM")
-        MIXERS.unregister("toy_decaying_sum")
-        FEED_FORWARDS.unregister("toy_routed")
-        POSITION_ENCODINGS.unregister("toy_phase")
-        NORMS.unregister("toy_plain_norm")
+        _unregister_toys()
+
+
+def test_toy_parts_that_declare_themselves_replayable_run_from_graphs(tmp_path):
+    """A toy mixer with two state tensors of its own that runs on the device alone, a toy
+    embedding and a toy output projection, all declared replayable in this file: the model's
+    decode steps are recorded and replayed under the scheduler and the pipeline, tokens fed from
+    the device, and the tokens are the plain toy model's.  The mixer's launch data, kept in
+    ``ctx.static``, is made once per recorded batch size and not again while recording."""
+    from safetensors.torch import load_file
+
+    from rapid_llm_amd import LLM, SamplingParams, write_random_model
+    from rapid_llm_amd.config import register_architecture
+
+    mixer_cls = _toy_parts()
+    register_architecture("ToyForCausalLM", ToyConfig, _toy_spec, replace=True)
+    try:
+        cfg = ToyConfig(hidden=48, vocab=97, heads=3, head_dim=16, inter=80, decay=0.8, ends=True, replay=True)
+        folder = write_random_model(cfg.to_dict(), 6, tmp_path / "toy", dtype="float32")
+        weights = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
+        llm = LLM(str(folder), dtype="float32", max_seq_len=64, page_size=8, num_pages=40, max_num_seqs=3,
+                  max_chunk_size=6, max_num_batched_tokens=64)  # portions of 6: none of a single token
+        runner = llm.scheduler.runner
+        assert runner.graphs_allowed and llm.scheduler.pipeline
+        prompts = [random_tokens(n, cfg.vocab, 90 + i) for i, n in enumerate((9, 14, 3, 11, 6))]
+        new = 9
+        mixer_cls.uploads = 0
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_gen_len=new))
+        sizes = sorted({key[0] for key in runner._graphs})
+        assert sizes and set(sizes) <= {1, 2, 4}, sizes
+        # one upload per recorded batch size (in the eager run before the recording) and one per
+        # eager decode step, of which there is none: every step of single tokens was replayed
+        assert mixer_cls.uploads == len(runner._graphs)
+        for prompt, out in zip(prompts, outs):
+            toks = list(prompt)
+            for _ in range(new):
+                toks.append(int(_toy_plain(weights, cfg, toks)[-1].argmax()))
+            assert out.outputs[0].token_ids == toks[len(prompt):]
+        runner.cache.check_invariants()
+    finally:
+        _unregister_toys()
 
 
 def test_unknown_part_kinds_are_named():
     from rapid_llm_amd.models import CausalLM, LayerSpec, ModelSpec, PartSpec
 
     norm = PartSpec("rmsnorm", {"size": 8, "eps": 1e-5, "checkpoint_name": "n"})
-    bad = ModelSpec(8, 10, (LayerSpec(PartSpec("no_such_mixer"), PartSpec("swiglu"), norm, norm),), norm, "e", "o", False)
+    from rapid_llm_amd.models import linear_output, token_embedding
+
+    bad = ModelSpec(8, 10, (LayerSpec(PartSpec("no_such_mixer"), PartSpec("swiglu"), norm, norm),), norm,
+                    token_embedding(10, 8, "e"), linear_output(10, 8, "o", False))
     with pytest.raises(ValueError, match="unknown mixer kind 'no_such_mixer'; known: .*gqa_attention"):
         CausalLM(bad)
