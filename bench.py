@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16]
                     [--shape NAME] [--batch B] [--prompt-len T] [--context C]
+    python bench.py --workload qwen3-0.6b-256 | qwen3-32b-32
 
 A "step" is one decode step of the whole batch through the engine's step function and the
 greedy sampling kernel, tokens fed back.  The default run has the layer sizes of
@@ -12,6 +13,14 @@ and decoding at batch 1 and 64 (``points``, which also holds the true 32-bit pat
 and prefill speed, measured in a second process).  ``--shape``, ``--prompt-len`` and
 ``--context`` measure the same at other sizes of the model family and other lengths; the
 line then names them in ``metric`` and ``config``.
+
+``points`` also holds the two scheduler workloads of BASELINE.json (``configs[3]``: the
+Qwen3-0.6B shape, 256 requests at once, prompts uniform in 64 to 1,024 tokens, 128 tokens each;
+``configs[4]``: the Qwen3-32B shape, 32 requests, prompts uniform in 4,096 to 16,384, context
+16,384, cache pages from the memory that is free, 128 tokens each): time per output token,
+generated tokens a second and the decode step's share of the HBM roofline, each measured in a
+process of its own through the continuous-batching scheduler (``--workload NAME`` runs one
+alone; ``--no-workloads`` leaves them out).
 
 Metric definitions follow rapid_llm's docs/benchmark_models.md:141-149: decode tok/s is
 batch / mean step time; prefill tok/s is prompt tokens / prefill latency; both timed
@@ -141,6 +150,80 @@ def measured_peaks() -> int:
     return 0
 
 
+# The scheduler workloads of BASELINE.json configs[3] and configs[4].
+WORKLOADS = {
+    "qwen3-0.6b-256": dict(shape="qwen3-0.6b", requests=256, low=64, high=1024, gen=128, context=2048, key="w06b",
+                           passes=2),
+    # one pass: its 300,000 prompt tokens take 25 s, and recording the decode graphs in the
+    # first steps changes the mean of 127 steps by under 1%
+    "qwen3-32b-32": dict(shape="qwen3-32b", requests=32, low=4096, high=16384, gen=128, context=16384 + 128, key="w32b",
+                         passes=1),
+}
+
+
+def run_workload(name: str, seed: int = 1234) -> int:
+    """One workload through the scheduler; prints one JSON line of its own."""
+    import torch
+
+    from rapid_llm_amd.cli import measure_offline, sample_prompt_lengths
+    from rapid_llm_amd.engine.llm import build_engine
+
+    w = WORKLOADS[name]
+    shape = load_shape()
+    shape.pop("context"), shape.pop("prompt_len")
+    shape.update(FAMILY[w["shape"]])
+    t0 = time.time()
+    engine = build_engine(
+        shape, load_format="random", dtype="bfloat16", max_seq_len=w["context"], max_num_seqs=w["requests"],
+        max_num_batched_tokens=8192, max_chunk_size=8192, page_size=16, seed=seed,
+    )
+    cfg = engine.runner.config
+    torch.cuda.synchronize()
+    print(f"[bench] {name}: model ready in {time.time() - t0:.1f} s, "
+          f"{engine.cache.capacity_tokens()} tokens of cache", file=sys.stderr, flush=True)
+    gen = torch.Generator().manual_seed(seed)
+    rows = []
+    for it in range(w["passes"]):  # with two, the first records the graphs and warms the allocator
+        lengths = sample_prompt_lengths(w["requests"], w["low"], w["high"], seed + it)
+        prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for n in lengths]
+        row = measure_offline(engine, prompts, w["gen"])
+        row["mean_prompt"] = sum(lengths) / len(lengths)
+        rows.append(row)
+        print(f"[bench] {name} pass {it}: {row}", file=sys.stderr, flush=True)
+    row = rows[-1]
+    tpot = row["tpot_s"]
+    mean_ctx = row["mean_prompt"] + w["gen"] / 2.0
+    step_bytes = weight_bytes(cfg, 2) + w["requests"] * mean_ctx * kv_bytes_per_token(cfg, 2)
+    k = w["key"]
+    print(json.dumps({
+        f"{k}_tpot_ms": round(tpot * 1e3, 3),
+        f"{k}_decode_tok_s": round(w["requests"] / tpot, 1),
+        f"{k}_tok_s": round(row["output_tokens"] / row["latency_s"], 1),
+        f"{k}_prefill_tok_s": round(row["prompt_tokens"] / row["ttft_s"], 1),
+        f"{k}_hbm_frac": round(step_bytes / tpot / 1e9 / HBM_GBPS, 4),
+        f"{k}_preemptions": row["preemptions"],
+    }), flush=True)
+    return 0
+
+
+def workload_points(names) -> dict:
+    """Each workload in a process of its own (the 32B shape needs the whole device)."""
+    import subprocess
+
+    out = {}
+    for name in names:
+        try:
+            done = subprocess.run(
+                [sys.executable, os.path.abspath(__file__), "--workload", name], capture_output=True, text=True, timeout=900
+            )
+            out.update(json.loads(done.stdout.strip().splitlines()[-1]))
+            print(f"[bench] workload {name}: {done.stdout.strip().splitlines()[-1]}", file=sys.stderr, flush=True)
+        except Exception as err:  # the main line must not be lost to a workload
+            tail = "" if "done" not in locals() else done.stderr[-800:]
+            print(f"[bench] workload {name} gave no result: {err!r} {tail}", file=sys.stderr, flush=True)
+    return out
+
+
 def float32_points(args) -> dict:
     """The same model through the true 32-bit path, in a process of its own (the float32
     weights need their own 33 GB): decode tok/s at the main batch size and prefill tok/s."""
@@ -173,7 +256,8 @@ def float32_points(args) -> dict:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=256,
+                    help="timed decode steps (BASELINE.json's decode workload: 256 tokens a request)")
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
@@ -183,11 +267,14 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=None, help="longest sequence the engine is sized for")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to measure ('' for none)")
-    ap.add_argument("--point-steps", type=int, default=32)
+    ap.add_argument("--point-steps", type=int, default=64)
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-pipeline", action="store_true", help="read every step's tokens before queueing the next")
     ap.add_argument("--no-fp32", action="store_true", help="skip the float32 points (a second process)")
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help="run one scheduler workload of BASELINE.json alone and print its own line")
+    ap.add_argument("--no-workloads", action="store_true", help="skip the scheduler workloads (processes of their own)")
     ap.add_argument("--peaks", action="store_true",
                     help="measure what the device reaches with library kernels (a large read, copy and square products) and exit")
     args = ap.parse_args()
@@ -196,6 +283,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
+    if args.workload is not None:
+        return run_workload(args.workload)
 
     import torch
 
@@ -382,6 +471,11 @@ def main() -> int:
         print(f"[bench] decode batch {b}: {pts[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
     if args.dtype == "bfloat16" and not args.no_fp32 and points:
         pts.update(float32_points(args))
+    default_run = args.shape == "qwen3-8b" and args.layers is None and args.prompt_len is None and args.context is None
+    if args.dtype == "bfloat16" and not args.no_workloads and points and default_run:
+        del runner, executor  # the workloads need the device's memory
+        torch.cuda.empty_cache()
+        pts.update(workload_points(sorted(WORKLOADS)))
     result["points"] = pts
     print(json.dumps(result), flush=True)
     return 0

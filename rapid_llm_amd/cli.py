@@ -177,49 +177,81 @@ def cmd_chat(args) -> int:
     return 0
 
 
-def cmd_bench(args) -> int:
-    """All prompts submitted at once, run to completion, timed between device
-    synchronisations: TTFT = time to the first token of the batch, TPOT = (latency - TTFT) /
-    (output_len - 1), TPS = 1000 / TPOT per request, TGS = all output tokens / latency.
-    Prompts are uniform random token ids of exactly ``--input-len`` tokens, as the
-    reference's RandomDataset makes them (rapid_llm/benchmark/datasets/random.py:70-110)."""
+def sample_prompt_lengths(count: int, low: int, high: int, seed: int) -> list[int]:
+    """``count`` prompt lengths, uniform in ``[low, high]``, fixed by the seed (the reference
+    draws ``[input_len * range_ratio, input_len]``, rapid_llm/benchmark/datasets/common.py:52-64)."""
     import random
-    import statistics
 
+    if not 1 <= low <= high:
+        raise ValueError(f"prompt lengths must satisfy 1 <= low <= high, got {low} and {high}")
+    rng = random.Random(seed)
+    return [rng.randint(low, high) for _ in range(count)]
+
+
+def measure_offline(engine, prompts, gen_len: int) -> dict:
+    """All prompts submitted at once and run to completion, timed between device
+    synchronisations (docs/benchmark_models.md:141-149): TTFT = time until every request has its
+    first token, TPOT = (latency - TTFT) / (gen_len - 1), TPS = 1000 / TPOT per request,
+    TGS = all output tokens / latency."""
     import torch
 
     from .sampling.params import SamplingParams
 
+    params = SamplingParams(temperature=0.0, max_gen_len=gen_len, ignore_eos=True)
+    before = engine.num_preemptions
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    requests = [engine.add_request(p, params) for p in prompts]
+    ttft = None
+    steps = decode_steps = 0
+    while engine.has_unfinished_requests():
+        engine.step()
+        steps += 1
+        if ttft is None:
+            if all(r.output_token_ids for r in requests):
+                torch.cuda.synchronize()
+                ttft = time.perf_counter() - start
+        else:
+            decode_steps += 1
+    torch.cuda.synchronize()
+    latency = time.perf_counter() - start
+    tokens = sum(len(r.output_token_ids) for r in requests)
+    return {
+        "ttft_s": ttft, "latency_s": latency, "output_tokens": tokens, "steps": steps,
+        "decode_steps": decode_steps, "prompt_tokens": sum(len(p) for p in prompts),
+        "tpot_s": (latency - ttft) / max(1, gen_len - 1), "preemptions": engine.num_preemptions - before,
+    }
+
+
+def cmd_bench(args) -> int:
+    """Offline generation speed with synthetic prompts: uniform random token ids of exactly
+    ``--input-len`` tokens, or of lengths uniform in ``[--input-len-min, --input-len-max]``
+    (equally ``[input_len * --range-ratio, input_len]``), as the reference's RandomDataset makes
+    them (rapid_llm/benchmark/datasets/random.py:70-110)."""
+    import random
+    import statistics
+
     engine = _engine(args, args.batch_size)
     vocab = engine.runner.vocab_size
     rng = random.Random(args.seed)
-    params = SamplingParams(temperature=0.0, max_gen_len=args.gen_len, ignore_eos=True)
+    high = args.input_len_max if args.input_len_max is not None else args.input_len
+    low = args.input_len_min if args.input_len_min is not None else max(1, int(high * args.range_ratio))
     rows = []
     for it in range(args.warmup + args.iterations):
-        prompts = [[rng.randrange(vocab) for _ in range(args.input_len)] for _ in range(args.batch_size)]
-        torch.cuda.synchronize()
-        start = time.perf_counter()
-        requests = [engine.add_request(p, params) for p in prompts]
-        ttft = None
-        while engine.has_unfinished_requests():
-            engine.step()
-            if ttft is None and all(r.output_token_ids for r in requests):
-                torch.cuda.synchronize()
-                ttft = time.perf_counter() - start
-        torch.cuda.synchronize()
-        latency = time.perf_counter() - start
+        lengths = sample_prompt_lengths(args.batch_size, low, high, args.seed + it)
+        prompts = [[rng.randrange(vocab) for _ in range(n)] for n in lengths]
+        row = measure_offline(engine, prompts, args.gen_len)
         if it >= args.warmup:
-            rows.append((ttft, latency, sum(len(r.output_token_ids) for r in requests)))
-    ttft = statistics.median(r[0] for r in rows)
-    latency = statistics.median(r[1] for r in rows)
-    tokens = rows[0][2]
-    tpot = (latency - ttft) / max(1, args.gen_len - 1)
+            rows.append(row)
+    ttft = statistics.median(r["ttft_s"] for r in rows)
+    latency = statistics.median(r["latency_s"] for r in rows)
+    tpot = statistics.median(r["tpot_s"] for r in rows)
     print(json.dumps({
-        "batch_size": args.batch_size, "input_len": args.input_len, "gen_len": args.gen_len,
+        "batch_size": args.batch_size, "input_len_min": low, "input_len_max": high, "gen_len": args.gen_len,
         "ttft_s": round(ttft, 4), "tpot_ms": round(tpot * 1e3, 3),
-        "tps": round(1.0 / tpot, 1) if tpot > 0 else None, "tgs": round(tokens / latency, 1),
-        "prefill_tok_s": round(args.batch_size * args.input_len / ttft, 1),
-        "preemptions": engine.num_preemptions,
+        "tps": round(1.0 / tpot, 1) if tpot > 0 else None, "tgs": round(rows[0]["output_tokens"] / latency, 1),
+        "prefill_tok_s": round(statistics.median(r["prompt_tokens"] / r["ttft_s"] for r in rows), 1),
+        "preemptions": sum(r["preemptions"] for r in rows),
     }))
     return 0
 
@@ -262,6 +294,10 @@ def main(argv=None) -> int:
     _common(bench, graph_default=True)
     bench.add_argument("--batch-size", type=int, default=8)
     bench.add_argument("--input-len", type=int, default=128)
+    bench.add_argument("--input-len-min", type=int, default=None, help="shortest prompt (default: input-len * range-ratio)")
+    bench.add_argument("--input-len-max", type=int, default=None, help="longest prompt (default: input-len)")
+    bench.add_argument("--range-ratio", type=float, default=1.0,
+                       help="prompt lengths are uniform in [input-len * ratio, input-len]; 1.0 pins them")
     bench.add_argument("--gen-len", type=int, default=128)
     bench.add_argument("--iterations", type=int, default=3)
     bench.add_argument("--warmup", type=int, default=1)

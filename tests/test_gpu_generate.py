@@ -482,6 +482,16 @@ def test_command_line_bench(tmp_path, capsys):
                  "--input-len", "40", "--gen-len", "12", "--iterations", "2", "--warmup", "1"])
     line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
     assert code == 0 and line["batch_size"] == 5 and line["tgs"] > 0 and line["ttft_s"] > 0 and line["tpot_ms"] > 0
+    assert line["input_len_min"] == line["input_len_max"] == 40
+    # prompt lengths drawn from a range, as the reference's random dataset draws them
+    code = main(["bench", "--model-dir", str(model_dir), "--max-seq-len", "128", "--batch-size", "6",
+                 "--input-len-min", "3", "--input-len-max", "70", "--gen-len", "9", "--iterations", "1", "--warmup", "0"])
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert code == 0 and (line["input_len_min"], line["input_len_max"]) == (3, 70) and line["tgs"] > 0
+    code = main(["bench", "--model-dir", str(model_dir), "--max-seq-len", "128", "--batch-size", "3",
+                 "--input-len", "64", "--range-ratio", "0.25", "--gen-len", "5", "--iterations", "1", "--warmup", "0"])
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert code == 0 and (line["input_len_min"], line["input_len_max"]) == (16, 64)
 
 
 def test_smoke_entry():
