@@ -275,7 +275,7 @@ def cmd_replay(args) -> int:
 
 
 def main(argv=None) -> int:
-    parser = argparse.ArgumentParser(prog="rapid-llm-amd", description=__doc__.split("\n\n")[0])
+    parser = argparse.ArgumentParser(prog="rapid-llm", description=__doc__.split("\n\n")[0])
     subs = parser.add_subparsers(dest="command", required=True)
 
     batch = subs.add_parser("batch", help="Run a prompt file through the continuous-batching engine")
