@@ -145,6 +145,27 @@ def measured_peaks() -> int:
         b = torch.randn(n, n, device="cuda", dtype=dtype)
         torch.backends.cuda.matmul.allow_tf32 = False
         out[f"gemm_{name}_tflops"] = round(2 * n**3 / timed(lambda: torch.matmul(a, b.t())) / 1e12, 1)
+    # What a kernel of a decode step can hope for: plain reads of the sizes of a layer's four
+    # weight matrices (Qwen3-8B: 34, 50, 100 and 201 MB) and of 400 MB, forty in a row replayed
+    # from a graph, every one over memory that no earlier one touched.  Microseconds a kernel;
+    # the rate is what a product of that size can reach at most, start and end included.
+    pool = torch.ones(1 << 30, dtype=torch.bfloat16, device="cuda")  # 2 GiB
+    chain = {}
+    for mb in (34, 50, 100, 201, 400):
+        n = int(mb * 1e6 / 2)
+        views = [pool[i * n : (i + 1) * n] for i in range(pool.numel() // n)]
+        best = None
+        for blocks in (256, 512, 2048):
+            graph = torch.cuda.CUDAGraph()
+            ops.read_buffer(views[0], blocks)
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph):
+                for i in range(40):
+                    ops.read_buffer(views[i % len(views)], blocks)
+            sec = timed(graph.replay, 5) / 40
+            best = sec if best is None else min(best, sec)
+        chain[f"{mb}MB"] = {"us": round(best * 1e6, 1), "gbps": round(mb * 1e6 / best / 1e9, 1)}
+    out["read_chain"] = chain
     out["published"] = {"hbm_gbps": HBM_GBPS, "bf16_tflops": PEAK_TFLOPS["bfloat16"], "fp32_tflops": PEAK_TFLOPS["float32"]}
     print(json.dumps(out), flush=True)
     return 0
