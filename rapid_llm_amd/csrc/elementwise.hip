@@ -378,6 +378,35 @@ extern "C" int rl_cast(const void* src, int src_type, void* dst, int dst_type, s
 }
 
 // --------------------------------------------------------------------------- //
+// bias of a product: y[r, c] += bias[c], the sum rounded once to y's type
+// (rapid_llm/modules/linear.py adds the bias inside F.linear; Qwen3 has none, other
+// architectures' projections do)
+// --------------------------------------------------------------------------- //
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, size_t total,
+                                int cols) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; idx < total; idx += step) y[idx] = from_float<T>(to_float(y[idx]) + bias[idx % cols]);
+}
+
+extern "C" int rl_add_bias(void* y, const float* bias, int rows, int cols, int act_type,
+                           hipStream_t stream) {
+    if (rows <= 0 || cols <= 0) return RL_OK;
+    const size_t total = (size_t)rows * cols;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    dim3 grid((unsigned)blocks), block(256);
+    if (act_type == RL_F32)
+        hipLaunchKernelGGL(add_bias_kernel<float>, grid, block, 0, stream, (float*)y, bias, total, cols);
+    else if (act_type == RL_BF16)
+        hipLaunchKernelGGL(add_bias_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, bias, total, cols);
+    else
+        return RL_ERR_ARG;
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
 // rotation tables: cos/sin[p, i] of the float32 product p * inv_freq[i]
 // rapid_llm/modules/rotary_embedding.py:194-202 (float32 outer product, then cos/sin)
 // --------------------------------------------------------------------------- //

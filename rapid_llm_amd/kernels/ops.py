@@ -174,6 +174,14 @@ def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
     )
 
 
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
+    """``y[r, :] += bias`` in place (``bias`` float32)."""
+    rows, cols = y.shape
+    _need(y, "y")
+    _need(bias, "bias", torch.float32, (cols,))
+    _ok(core().rl_add_bias(_p(y), _p(bias), rows, cols, _tag(y.dtype), _stream()), "rl_add_bias")
+
+
 def rope_table(inv_freq: torch.Tensor, positions: int) -> tuple[torch.Tensor, torch.Tensor]:
     _need(inv_freq, "inv_freq", torch.float32)
     half = inv_freq.numel()

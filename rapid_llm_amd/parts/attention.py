@@ -44,6 +44,8 @@ class GQAAttention(Mixer):
         o_name: str = "o_proj.weight",
         q_norm_name: str = "q_norm.weight",
         k_norm_name: str = "k_norm.weight",
+        qkv_bias: bool = False,
+        o_bias: bool = False,
     ) -> None:
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not divisible by {num_kv_heads} kv heads")
@@ -61,6 +63,10 @@ class GQAAttention(Mixer):
         self.qkv = Linear(hidden_size, (num_heads + 2 * num_kv_heads) * head_dim)
         self.o = Linear(num_heads * head_dim, hidden_size)
         self.q_norm_w = self.k_norm_w = None
+        # Qwen3 has neither (rapid_llm/models/qwen3.py:16-18: qkv_bias=False); architectures of the
+        # same skeleton do (rapid_llm/models/base.py:121-132 passes bias=qkv_bias), under the
+        # projections' names with ".bias" in place of ".weight"
+        self.qkv_bias, self.o_bias = bool(qkv_bias), bool(o_bias)
 
     # ---- tensors ---------------------------------------------------------------
     def param_specs(self) -> list[ParamSpec]:
@@ -80,11 +86,25 @@ class GQAAttention(Mixer):
                 ParamSpec(self.name + ".q_norm", (self.d,), "vector", (Source(p + n["qn"], self.d),), init="norm"),
                 ParamSpec(self.name + ".k_norm", (self.d,), "vector", (Source(p + n["kn"], self.d),), init="norm"),
             ]
+
+        def bias_of(weight_name: str) -> str:
+            return weight_name[: -len("weight")] + "bias" if weight_name.endswith("weight") else weight_name + ".bias"
+
+        if self.qkv_bias:
+            specs.append(ParamSpec(
+                self.name + ".qkv_bias", (q_rows + 2 * kv_rows,), "vector",
+                (Source(p + bias_of(n["q"]), q_rows), Source(p + bias_of(n["k"]), kv_rows),
+                 Source(p + bias_of(n["v"]), kv_rows)),
+            ))
+        if self.o_bias:
+            specs.append(ParamSpec(
+                self.name + ".o_bias", (self.hidden_size,), "vector", (Source(p + bias_of(n["o"]), self.hidden_size),)
+            ))
         return specs
 
     def bind(self, params, runtime) -> None:
-        self.qkv.bind(params[self.name + ".qkv"])
-        self.o.bind(params[self.name + ".o"])
+        self.qkv.bind(params[self.name + ".qkv"], params[self.name + ".qkv_bias"] if self.qkv_bias else None)
+        self.o.bind(params[self.name + ".o"], params[self.name + ".o_bias"] if self.o_bias else None)
         if self.qk_norm_eps is not None:
             self.q_norm_w = params[self.name + ".q_norm"]
             self.k_norm_w = params[self.name + ".k_norm"]

@@ -1,4 +1,6 @@
-"""``y = x W^T`` with ``W [out, in]`` as the checkpoint stores it (no bias in this family).
+"""``y = x W^T (+ b)`` with ``W [out, in]`` as the checkpoint stores it.  This family has no
+bias; a part of another architecture binds one, which is added by a kernel of its own after
+the product (a product with a bias folds no norm into itself).
 
 Which product runs is decided by the weight's storage type:
 
@@ -25,13 +27,17 @@ class Linear:
         self.in_features = in_features
         self.out_features = out_features
         self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
 
-    def bind(self, weight: torch.Tensor) -> None:
+    def bind(self, weight: torch.Tensor, bias: torch.Tensor | None = None) -> None:
         if tuple(weight.shape) != (self.out_features, self.in_features):
             raise ValueError(
                 f"linear weight must be {(self.out_features, self.in_features)}, is {tuple(weight.shape)}"
             )
+        if bias is not None and (tuple(bias.shape) != (self.out_features,) or bias.dtype != torch.float32):
+            raise ValueError(f"linear bias must be float32 of shape {(self.out_features,)}, is {bias.dtype} {tuple(bias.shape)}")
         self.weight = weight
+        self.bias = bias
 
     # ---- folding a neighbouring norm into the product (decode steps, bfloat16) ----------
     def skinny(self, x) -> bool:
@@ -40,6 +46,11 @@ class Linear:
             self.weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
             and x.shape[0] <= ops.SKINNY_MAX_ROWS and self.in_features % 8 == 0
         )
+
+    def folds(self, x) -> bool:
+        """Whether this product may absorb the residual add and norm that follow it: one of the
+        two kernels with that epilogue runs it, and no bias comes between."""
+        return self.bias is None and (self.skinny(x) or self.midsize(x))
 
     def takes_scaled_rows(self) -> bool:
         """Whether this product can finish a norm whose rows arrive unscaled (whatever the
@@ -63,7 +74,7 @@ class Linear:
         """The product, or a :class:`DeferredProduct` of it where one of this product's kernels
         could fold a neighbouring norm into itself (bfloat16, up to 16 rows, or 17 to 64 rows of a
         narrow matrix).  Whoever receives it and has no use for that simply materialises it."""
-        if isinstance(x, torch.Tensor) and (self.skinny(x) or self.midsize(x)):
+        if isinstance(x, torch.Tensor) and self.folds(x):
             return DeferredProduct(self, x)
         return self(x)
 
@@ -80,7 +91,10 @@ class Linear:
         if isinstance(x, ScaledRows):
             if not self.skinny(x):
                 raise ValueError("scaled rows reached a product that cannot apply their factor")
-            return ops.gemm_bf16(x.rows, w, out_dtype or x.dtype, scaled=x)
+            y = ops.gemm_bf16(x.rows, w, out_dtype or x.dtype, scaled=x)
+            if self.bias is not None:
+                ops.add_bias(y, self.bias)
+            return y
         rows = x.shape[0]
         out_dtype = out_dtype or x.dtype
         if w.dtype == torch.float32:
@@ -96,4 +110,6 @@ class Linear:
             narrow = torch.empty(y.shape, dtype=out_dtype, device=y.device)
             ops.cast(y, narrow)
             y = narrow
+        if self.bias is not None:
+            ops.add_bias(y, self.bias)
         return y

@@ -45,14 +45,15 @@ class RMSNorm(Norm):
         if isinstance(delta, DeferredProduct):
             if (
                 scaled_ok and rows is None and delta.linear.out_features == self.size
-                and self.dtype == torch.bfloat16 and delta.linear.skinny(delta.x)
+                and self.dtype == torch.bfloat16 and delta.linear.bias is None and delta.linear.skinny(delta.x)
             ):
                 # the producer's kernel adds into the residual and leaves what the consumer's
                 # kernel needs to finish the norm: no kernel of this norm's own runs
                 return delta.linear.add_to_residual(delta.x, residual, self.weight, self.eps)
             if (
                 rows is None and delta.linear.out_features == self.size and self.dtype == torch.bfloat16
-                and self.size % 4 == 0 and self.size <= 16 * 1024 and delta.linear.midsize(delta.x)
+                and self.size % 4 == 0 and self.size <= 16 * 1024 and delta.linear.bias is None
+                and delta.linear.midsize(delta.x)
             ):
                 # the product arrives as float32 runs of K, which this norm's kernel adds
                 out = torch.empty((residual.shape[0], self.size), dtype=self.dtype, device=residual.device)

@@ -138,19 +138,20 @@ class ToyConfig:
     toynorm: bool = False  # layer 1 uses a norm defined here, which knows nothing of unfinished products
     ends: bool = False  # an embedding that scales its rows and an output projection that caps its logits
     replay: bool = False  # the toy mixer runs on the device alone and declares itself replayable
+    bias: bool = False  # the attention's projections have biases (Qwen3 has none; the part can)
 
     @classmethod
     def from_dict(cls, data, overrides=None):
         return cls(data["hidden"], data["vocab"], data["heads"], data["head_dim"], data["inter"],
                    data["decay"], data.get("twice", False), data.get("share", False),
                    data.get("experts", 0), data.get("period", 0.0), data.get("toynorm", False),
-                   data.get("ends", False), data.get("replay", False))
+                   data.get("ends", False), data.get("replay", False), data.get("bias", False))
 
     def to_dict(self):
         return dict(architectures=["ToyForCausalLM"], hidden=self.hidden, vocab=self.vocab, heads=self.heads,
                     head_dim=self.head_dim, inter=self.inter, decay=self.decay, twice=self.twice,
                     share=self.share, experts=self.experts, period=self.period, toynorm=self.toynorm,
-                    ends=self.ends, replay=self.replay, torch_dtype="float32")
+                    ends=self.ends, replay=self.replay, bias=self.bias, torch_dtype="float32")
 
 
 CAP = 0.3  # the toy output projection's cap: logits = CAP * tanh(h W^T / CAP)
@@ -383,7 +384,8 @@ def _toy_spec(cfg: ToyConfig):
 
     def attn(i):
         return PartSpec("gqa_attention", {"hidden_size": cfg.hidden, "num_heads": cfg.heads, "num_kv_heads": 1,
-                                          "head_dim": cfg.head_dim, "checkpoint_prefix": f"l{i}.attn."})
+                                          "head_dim": cfg.head_dim, "checkpoint_prefix": f"l{i}.attn.",
+                                          "qkv_bias": cfg.bias, "o_bias": cfg.bias})
 
     ff0 = ff(0)
     if cfg.experts:
@@ -444,19 +446,23 @@ def _toy_plain(w, cfg: ToyConfig, toks):
             rows.append(s)
         return ffn(0, h + torch.stack(rows) @ w["l0.mix.w"].T)
 
+    def proj(i, which, x):
+        y = x @ w[f"l{i}.attn.{which}_proj.weight"].T
+        return y + w[f"l{i}.attn.{which}_proj.bias"] if cfg.bias else y
+
     def kv_of(i, h):
         x = plain_rmsnorm(h, w[f"l{i}.n1"], 1e-5)
         c, s = plain_rope_tables(pos, cfg.head_dim, 100.0)
-        k = plain_rope_apply((x @ w[f"l{i}.attn.k_proj.weight"].T).view(t, 1, cfg.head_dim), c, s)
-        return k, (x @ w[f"l{i}.attn.v_proj.weight"].T).view(t, 1, cfg.head_dim)
+        k = plain_rope_apply(proj(i, "k", x).view(t, 1, cfg.head_dim), c, s)
+        return k, proj(i, "v", x).view(t, 1, cfg.head_dim)
 
     def attn(i, h, kv=None):
         x = plain_rmsnorm(h, w[f"l{i}.n1"], 1e-5)
         c, s = plain_rope_tables(pos, cfg.head_dim, 100.0)
-        q = plain_rope_apply((x @ w[f"l{i}.attn.q_proj.weight"].T).view(t, cfg.heads, cfg.head_dim), c, s)
+        q = plain_rope_apply(proj(i, "q", x).view(t, cfg.heads, cfg.head_dim), c, s)
         k, v = kv if kv is not None else kv_of(i, h)
         o = plain_attention(q, k, v, cfg.head_dim**-0.5).reshape(t, -1)
-        return ffn(i, h + o @ w[f"l{i}.attn.o_proj.weight"].T)
+        return ffn(i, h + proj(i, "o", o))
 
     if cfg.twice:
         h = attn(1, toy(h))
@@ -488,9 +494,9 @@ def _unregister_toys():
 
 @pytest.mark.parametrize("variant,dtype", [("plain", "float32"), ("twice", "float32"), ("share", "float32"),
                                            ("routed", "float32"), ("toynorm", "float32"), ("ends", "float32"),
-                                           ("replay", "float32"),
+                                           ("replay", "float32"), ("bias", "float32"),
                                            ("routed", "bfloat16"), ("toynorm", "bfloat16"), ("twice", "bfloat16"),
-                                           ("ends", "bfloat16")])
+                                           ("ends", "bfloat16"), ("bias", "bfloat16")])
 def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
     """In bfloat16 the built-in parts hand unfinished products and unscaled rows to each other
     in steps of few tokens; the toy parts declare nothing and must only ever see tensors."""
@@ -505,7 +511,8 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
         cfg = ToyConfig(hidden=48, vocab=97, heads=3, head_dim=16, inter=80, decay=0.8,
                         twice=variant == "twice", share=variant == "share",
                         experts=3 if variant == "routed" else 0, period=9.0 if variant == "routed" else 0.0,
-                        toynorm=variant == "toynorm", ends=variant == "ends", replay=variant == "replay")
+                        toynorm=variant == "toynorm", ends=variant == "ends", replay=variant == "replay",
+                        bias=variant == "bias")
         folder = write_random_model(cfg.to_dict(), 3, tmp_path / "toy", dtype=dtype)
         weights = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
         if variant == "share":  # the sharing layer's own k/v projections exist but are never used
@@ -515,6 +522,10 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
         if variant == "toynorm":
             assert type(runner.model.blocks[1].mixer_norm).__name__ == "PlainTorchNorm"
         assert needs[0].kind == "state" and needs[1].kind == "kv"
+        if variant == "bias":
+            assert weights["l1.attn.q_proj.bias"].shape == (cfg.heads * cfg.head_dim,)
+            assert weights["l1.attn.o_proj.bias"].abs().max() > 0
+            assert runner.params["layers.1.mixer.qkv_bias"].dtype == torch.float32
         if variant == "ends":
             assert type(runner.model.embed).__name__ == "ScaledEmbedding"
             assert type(runner.model.output).__name__ == "CappedOutput"
