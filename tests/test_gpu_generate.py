@@ -2,6 +2,7 @@
 and sampling kernels; the plain implementation re-runs the whole sequence for every token."""
 
 import pytest
+import torch
 
 import parity
 from plain_model import plain_forward, plain_load
@@ -407,6 +408,27 @@ def test_text_prompts_with_a_tokenizer(tmp_path, capsys, monkeypatch):
     assert main(["chat", *common]) == 0
     text = capsys.readouterr().out
     assert text.count("w") > 10  # two streamed answers of six words each
+
+
+def test_the_page_pool_is_what_memory_is_left_and_a_budget_of_nothing_is_refused(tmp_path):
+    """Without ``num_pages`` the pool is sized from the free memory less the state tensors and
+    the recorded steps' estimate; a utilisation that leaves nothing raises instead of making a
+    pool of two pages."""
+    from rapid_llm_amd import EngineConfig, ModelRunner
+
+    cfg, page, seed = TINY["B"]
+    model_dir = make_model_dir(tmp_path, "B", "bfloat16")
+    free, total = torch.cuda.mem_get_info()
+    common = dict(dtype="bfloat16", max_seq_len=128, page_size=page, max_num_seqs=4)
+    runner = ModelRunner(model_dir, EngineConfig(**common))
+    assert runner.cache.pools[0].num_usable == 4 * (128 // page)  # capped: every slot at full length
+    estimate = runner._graph_pool_estimate()
+    assert estimate > 0 and runner.state_bytes == 0
+    assert ModelRunner(model_dir, EngineConfig(use_graph=False, **common))._graph_pool_estimate() == 0
+    # keep back more than is free: nothing is left for pages
+    too_little = max(1e-6, min(0.5, 0.5 * free / total) * 1e-3)
+    with pytest.raises(ValueError, match="no memory is left for the cache"):
+        ModelRunner(model_dir, EngineConfig(gpu_memory_utilization=too_little, **common))
 
 
 def test_template_and_stop_token_of_the_model_folder(tmp_path, capsys):
