@@ -721,27 +721,42 @@ _PREFILL_SLOTS = 512  # wave groups of four the chip holds at a time (two on eac
 # what a step costs more when the two wave groups of a compute unit walk one tile in lockstep
 # than when they belong to two tiles and drift apart (measured: 3.17 against 2.83 us)
 _PREFILL_PAIRED_COST = 1.12
+# a tile that outlasts the others ends alone on its compute unit and steps faster there than
+# beside a second workgroup (2,048 tokens behind 2,048: 139 us with one wave group a tile,
+# 157 us with two, where whole steps at the shared rate would say 181 against 152)
+_PREFILL_ALONE = 0.8
+# what cutting the tiles' keys into runs costs, in steps: the runs' partial results are
+# written, and read and folded by a second kernel (1,024 tokens from their start: 33 us whole,
+# 47 us in two runs)
+_PREFILL_MERGE_STEPS = 5
 
 
 def _prefill_shape(plan: "AttentionPlan", nkv: int, window: int, tile_rows: int) -> tuple[int, int]:
     """(wave groups per workgroup, runs the keys of every tile are cut into) for a launch of
-    the prefill kernel.  Few, long tiles (a portion of one long prompt) have their keys cut
-    into runs, folded by the merge kernel, so that the launch fills the chip.  Two wave groups
-    share each tile when the longest tile would otherwise outlast the work there is for
-    every other slot."""
+    the prefill kernel, from an estimate of the launch's length in steps: the longest tile's
+    steps (halved where two wave groups share it, divided where its keys are cut into runs) or
+    the steps there are for every slot of the chip, whichever is more.  Few, long tiles (a
+    portion of one long prompt) come out with their keys cut into runs, folded by the merge
+    kernel; a prompt from its start, whose last rows alone see many keys, with two wave groups
+    a tile; a launch with work for every slot with neither."""
     keys = plan.tile_keys
     if window > 0:
         keys = [min(k, window + tile_rows) for k in keys]
     items = plan.num_tiles * nkv
-    longest = max(keys)
-    nsplit = 1
-    if items < _PREFILL_SPLIT_BELOW and longest >= 2 * _PREFILL_SPLIT_KEYS:
-        nsplit = min(_PREFILL_MAX_SPLITS, -(-_PREFILL_SPLIT_BELOW // items), longest // _PREFILL_SPLIT_KEYS)
     steps = [-(-k // _PREFILL_STEP_KEYS) for k in keys]
-    longest_steps = -(-max(steps) // nsplit)
+    longest = max(steps)
     share = nkv * sum(steps) / _PREFILL_SLOTS  # steps per slot if the work were spread evenly
-    paired = max(-(-longest_steps // 2), share) * _PREFILL_PAIRED_COST
-    return (2 if paired < max(longest_steps, share) else 1), nsplit
+    best = (max(longest * _PREFILL_ALONE, share), 1, 1)
+    paired = max(-(-longest // 2), share) * _PREFILL_PAIRED_COST
+    if paired < best[0]:
+        best = (paired, 2, 1)
+    if items < _PREFILL_SPLIT_BELOW:
+        most = min(_PREFILL_MAX_SPLITS, -(-_PREFILL_SPLIT_BELOW // items), max(keys) // _PREFILL_SPLIT_KEYS)
+        for nsplit in range(2, most + 1):
+            cost = max(-(-longest // nsplit), share) + _PREFILL_MERGE_STEPS
+            if cost < best[0]:
+                best = (cost, 1, nsplit)
+    return best[1], best[2]
 
 
 def _static(ctx) -> dict:

@@ -177,7 +177,10 @@ def test_prefill_shape_follows_the_launch():
         return ops._prefill_shape(ops.AttentionPlan(ctx, group, 128), nkv, window, 128)
 
     assert shape([(0, 2048)]) == (2, 1)
+    assert shape([(0, 1024)]) == (2, 1)  # runs would cost more than they save: the tiles are short on average
     assert shape([(0, 8192)]) == (1, 1)
+    assert shape([(0, 4096)]) == (1, 1)
+    assert shape([(2048, 2048)]) == (1, 1)  # work for every slot; the longest tile ends alone and fast
     assert shape([(3584, 512)]) == (1, 4)
     assert shape([(0, 2048)] * 4) == (1, 1)
     assert shape([(0, 20)]) == (1, 1)  # one step: nothing to share
