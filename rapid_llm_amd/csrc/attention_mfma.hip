@@ -245,8 +245,16 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
     const int* table = block_table + (size_t)token_slot[t] * table_stride;
     const int kend = pos + 1;
     const int kstart = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-    const int lo = (kstart & ~31) + split * split_chunk;  // split_chunk is a multiple of 32
-    const int hi = min(kend, lo + split_chunk);
+    // The launch has nsplit splits of at most split_chunk keys, laid out for the longest context
+    // it may meet (a recorded step serves every context of its bucket).  This request's keys are
+    // dealt to the splits evenly: runs of a multiple of 32 keys, at least 128 (shorter runs only
+    // add merge work), never more than split_chunk (the page ids of a run are staged in LDS).
+    // nsplit * split_chunk covers the longest context, so the runs cover this one.
+    const int first = kstart & ~31;
+    int run = ((kend - first + nsplit - 1) / nsplit + 31) & ~31;
+    run = min(max(run, 128), split_chunk);
+    const int lo = first + split * run;
+    const int hi = min(kend, lo + run);
 
     const int hh = hc * 16 + col;  // head within the group
     const bool head_ok = hh < G;

@@ -247,12 +247,16 @@ def test_attention_finds_a_far_key(dtype, far):
 
 
 def _decode_splits(ops, context, nkv, page):
-    """(keys per split, splits) of a decode launch of one request of ``context`` keys."""
+    """(keys per split, splits) of a decode launch of one request of ``context`` keys: the host
+    lays out splits of at most ``chunk`` keys, the kernel deals the request's keys to them evenly
+    in runs of a multiple of 32, at least 128."""
     pairs = nkv
     want = max(1, ops._TARGET_BLOCKS // pairs)
     chunk = max(ops._MIN_SPLIT_KEYS, -(-(-(-context // want)) // 128) * 128)
     chunk = min(chunk, max(32, ((ops._MAX_SPLIT_PAGES - 1) * page - 31) // 32 * 32))
-    return chunk, -(-context // chunk)
+    nsplit = -(-context // chunk)
+    run = min(max((-(-context // nsplit) + 31) // 32 * 32, 128), chunk)
+    return run, nsplit
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
