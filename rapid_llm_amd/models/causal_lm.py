@@ -8,9 +8,9 @@ product (:625-630), output projection (:631).
 
 from __future__ import annotations
 
-import torch
-
 from dataclasses import replace
+
+import torch
 
 from ..parts.base import (
     BLOCKS,

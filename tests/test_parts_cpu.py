@@ -80,3 +80,76 @@ def test_command_line_init_writes_a_model_folder_and_names_a_missing_one(tmp_pat
     monkeypatch.setenv("RAPID_LLM_MODEL_DIR", str(tmp_path / "nowhere"))
     with pytest.raises(SystemExit, match="does not exist"):
         main(["batch"])
+
+
+def test_a_product_with_a_bias_folds_no_norm_into_itself():
+    """The residual add and norm that follow a product are folded into its kernel only where
+    nothing comes between: a bias is added by a kernel of its own after the product."""
+    plain = _bound(128, 128, torch.bfloat16)
+    x = torch.zeros(4, 128, dtype=torch.bfloat16)
+    assert plain.folds(x) and plain.folds(torch.zeros(40, 128, dtype=torch.bfloat16))
+    assert not plain.folds(torch.zeros(80, 128, dtype=torch.bfloat16))  # the library's product
+    biased = Linear(128, 128)
+    biased.bind(torch.zeros(128, 128, dtype=torch.bfloat16), torch.zeros(128))
+    assert not biased.folds(x) and biased.skinny(x)
+    import pytest
+
+    with pytest.raises(ValueError, match="bias"):
+        Linear(128, 64).bind(torch.zeros(64, 128, dtype=torch.bfloat16), torch.zeros(128))
+    with pytest.raises(ValueError, match="bias"):
+        Linear(128, 64).bind(torch.zeros(64, 128, dtype=torch.bfloat16), torch.zeros(64, dtype=torch.bfloat16))
+
+
+def test_a_mixer_may_ask_for_several_state_tensors():
+    import pytest
+
+    from rapid_llm_amd.cache.storage import state_bytes
+    from rapid_llm_amd.parts import CacheNeed, StateSpec
+
+    one = CacheNeed("state", state_shape=(48,), state_dtype="float32")
+    assert [(s.name, s.shape, s.dtype) for s in one.state_specs()] == [("state", (48,), "float32")]
+    two = CacheNeed("kv", num_kv_heads=2, head_dim=16,
+                    states=(StateSpec("conv", (3, 48)), StateSpec("count", (1,), "int32")))
+    assert [s.name for s in two.state_specs()] == ["conv", "count"]
+    assert CacheNeed("kv", num_kv_heads=1, head_dim=16).state_specs() == ()
+    # five slots: 48 float32 each; 3 x 48 in the engine's type (2 bytes) and one int32 each
+    assert state_bytes([one, two], 5, 2) == 5 * 48 * 4 + 5 * (3 * 48 * 2 + 4)
+    with pytest.raises(ValueError, match="alike"):
+        CacheNeed("state", state_shape=(4,), states=(StateSpec("state", (2,)),)).state_specs()
+
+
+def test_the_ends_of_a_model_are_parts_named_in_its_description():
+    from rapid_llm_amd.models import linear_output, token_embedding
+    from rapid_llm_amd.parts import EMBEDDINGS, OUTPUT_PROJECTIONS
+
+    assert "token_embedding" in EMBEDDINGS.kinds() and "linear_output" in OUTPUT_PROJECTIONS.kinds()
+    emb = token_embedding(100, 16, "model.embed_tokens.weight")
+    part = EMBEDDINGS.create(emb.kind, **emb.params, name="embed")
+    assert [(s.name, s.shape) for s in part.param_specs()] == [("embed.weight", (100, 16))]
+    tied = linear_output(100, 16, "lm_head.weight", True)
+    out = OUTPUT_PROJECTIONS.create(tied.kind, **tied.params, name="output")
+    assert out.param_specs()[0].fallback == "embed.weight"
+    assert OUTPUT_PROJECTIONS.create("linear_output", **linear_output(100, 16, "h", False).params, name="output").param_specs()[0].fallback is None
+
+
+def test_prefill_launch_shapes_follow_an_estimate_of_the_launch():
+    """Two wave groups on a tile where the longest tile would outlast everyone else's work (a
+    prompt from its start), one where there is work for every slot, key runs for few, long tiles
+    and only where they save more than their merge costs.  The choice is the host's alone."""
+    from types import SimpleNamespace
+
+    from rapid_llm_amd.kernels import ops
+
+    def shape(seqs, nkv=8, group=4, window=0, rows=128):
+        keys = []
+        for start, n in seqs:
+            for row0 in range(0, n * group, rows):
+                keys.append(start + min(n, (row0 + rows) // group))
+        return ops._prefill_shape(SimpleNamespace(tile_keys=keys, num_tiles=len(keys)), nkv, window, rows)
+
+    assert shape([(0, 2048)]) == (2, 1) and shape([(0, 1024)]) == (2, 1) and shape([(0, 512)]) == (2, 1)
+    assert shape([(0, 8192)]) == (1, 1) and shape([(0, 4096)]) == (1, 1) and shape([(2048, 2048)]) == (1, 1)
+    assert shape([(3584, 512)]) == (1, 4) and shape([(7680, 512)]) == (1, 4) and shape([(16000, 150)]) == (1, 8)
+    assert shape([(0, 2048)] * 4) == (1, 1) and shape([(0, 20)]) == (1, 1)
+    # a window bounds what every tile reads: the long prefix no longer counts
+    assert shape([(16000, 150)], window=256) == (2, 1)
