@@ -27,7 +27,7 @@
 //                    one is multiplied; one softmax step per 64 keys.
 //   rl_attn_decode:  single tokens.  Workgroup = (request, kv head, split of the keys); its
 //                    4 waves stride over 32-key steps reading K and V^T straight from
-//                    global memory one step ahead (nothing is reused), combine through LDS,
+//                    global memory (nothing is reused), combine through LDS,
 //                    and a merge kernel folds the splits (rapid_llm/kernels/ops/attention/
 //                    flashdecoding.py:115-263 stage 1, :334-407 stage 2).  In its fused form
 //                    it also norms and rotates q and k and writes the token's k and v.
@@ -376,18 +376,17 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
         }
         __syncthreads();
 
-        // the loads of the next step are issued before this step's arithmetic (two steps ahead
-        // was measured: never faster, and slower wherever a compute unit holds several waves)
-        DecodeFrags cur, nxt;
+        // A wave asks for one step's keys and values, waits for them and multiplies; what hides
+        // the wait is the other waves of the compute unit.  Keeping the next step's loads in
+        // flight as well (a second set of 64 registers) left room for two waves a SIMD instead of
+        // three and was 2 to 5% slower at every batch size and context length measured (256
+        // requests of 64 to 1,152 keys 182.7 -> 174.3 us, 64 of 2,100 keys 107.5 -> 103.6, 8 of
+        // 16,000 keys 95.5 -> 94.0); forcing four waves a SIMD spills and loses again.
+        DecodeFrags cur;
         int base = lo + 32 * wave;
-        if (base < hi)
+        for (; base < hi; base += 32 * DEC_WAVES) {
             decode_load<V16>(cur, k_cache, v_cache, lds_pages, page0, page_size, nkv, hk, base,
                              last_key, col, g);
-        for (; base < hi; base += 32 * DEC_WAVES) {
-            const int next = base + 32 * DEC_WAVES;
-            if (next < hi)
-                decode_load<V16>(nxt, k_cache, v_cache, lds_pages, page0, page_size, nkv, hk, next,
-                                 last_key, col, g);
             // ---- S^T = K Q^T for two blocks of 16 keys --------------------------------
             f32x4 s[2];
 #pragma unroll
@@ -423,7 +422,6 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
                 }
                 acc[b] = mfma(v, p, acc[b]);
             }
-            cur = nxt;
         }
 
         // ---- combine the waves pairwise, in the accumulators' own layout --------------------
