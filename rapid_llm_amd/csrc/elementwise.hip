@@ -764,6 +764,49 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
 }
 
 // --------------------------------------------------------------------------- //
+// order[r] = the single-token request with the r-th longest context of the step: request i's
+// last position is positions[seq_token ? seq_token[i] : i]; equal lengths keep their order.
+// Every thread counts the requests that come before its own (n^2 comparisons through LDS:
+// a step has hundreds of requests, not millions).  The decode attention hands its workgroups
+// out in this order.
+// --------------------------------------------------------------------------- //
+__global__ __launch_bounds__(256) void order_by_length_kernel(const int* __restrict__ positions,
+                                                              const int* __restrict__ seq_token,
+                                                              int n, int* __restrict__ order) {
+    __shared__ __attribute__((aligned(16))) int keys[256];
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int mine = i < n ? positions[seq_token ? seq_token[i] : i] : 0;
+    int rank = 0;
+    for (int base = 0; base < n; base += 256) {  // the same trips for every thread
+        const int j = base + threadIdx.x;
+        __syncthreads();
+        // beyond the last request: shorter than any (positions are never negative)
+        keys[threadIdx.x] = j < n ? positions[seq_token ? seq_token[j] : j] : -1;
+        __syncthreads();
+        // requests base + k before mine: longer ones, and equal ones with a smaller index
+        const int before = i - base;  // k < before: a smaller index
+#pragma unroll 8
+        for (int k4 = 0; k4 < 256; k4 += 4) {
+            const int4 o = *reinterpret_cast<const int4*>(&keys[k4]);
+            rank += (o.x > mine || (o.x == mine && k4 + 0 < before)) ? 1 : 0;
+            rank += (o.y > mine || (o.y == mine && k4 + 1 < before)) ? 1 : 0;
+            rank += (o.z > mine || (o.z == mine && k4 + 2 < before)) ? 1 : 0;
+            rank += (o.w > mine || (o.w == mine && k4 + 3 < before)) ? 1 : 0;
+        }
+    }
+    if (i < n) order[rank] = i;
+}
+
+extern "C" int rl_order_by_length(const int* positions, const int* seq_token, int n, int* order,
+                                  hipStream_t stream) {
+    if (n <= 0) return RL_OK;
+    if (!positions || !order) return RL_ERR_ARG;
+    hipLaunchKernelGGL(order_by_length_kernel, dim3((n + 255) / 256), dim3(256), 0, stream,
+                       positions, seq_token, n, order);
+    return rl_launch_status();
+}
+
+// --------------------------------------------------------------------------- //
 // A plain read of a buffer, for measuring what the memory system delivers: every thread
 // keeps eight 16-byte loads in flight; nothing is written unless the data match a pattern
 // that never occurs (so that the loads cannot be dropped).

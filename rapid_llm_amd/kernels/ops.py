@@ -631,9 +631,10 @@ class AttentionPlan:
     portions of the others are cut into row tiles (prefill kernel)."""
 
     __slots__ = ("num_decode", "seq_token", "max_decode_ctx", "num_tiles", "tile_info", "tile_keys", "orders",
-                 "_prefill_tokens", "_prefill_list")
+                 "_prefill_tokens", "_prefill_list", "_decode_order")
 
     def __init__(self, ctx, group: int, tile_rows: int) -> None:
+        self._decode_order = None
         fixed = _static(ctx).get("decode_only_tokens")
         if fixed is not None:
             # a step of single tokens whose index list is already on the device (graphs)
@@ -677,6 +678,18 @@ class AttentionPlan:
             self._prefill_tokens = upload_ints(self._prefill_list, device)
         return self._prefill_tokens
 
+    def decode_order(self, ctx) -> torch.Tensor:
+        """The step's single-token requests, longest context first, sorted on the device from the
+        step's positions (a replayed step has nothing else); made once a step, for every layer."""
+        if self._decode_order is None:
+            order = torch.empty(self.num_decode, dtype=torch.int32, device=ctx.positions.device)
+            _ok(
+                core().rl_order_by_length(_p(ctx.positions), _p(self.seq_token), self.num_decode, _p(order), _stream()),
+                "rl_order_by_length",
+            )
+            self._decode_order = order
+        return self._decode_order
+
     def work_order(self, nkv: int, device, resident: int = 1) -> torch.Tensor:
         """Order in which the (tile, kv head) pairs of the prefill kernel are handed out:
         longest first, so that the short ones fill the gaps at the end.  Where a compute unit
@@ -703,6 +716,9 @@ class AttentionPlan:
 # splits only add merge work).
 _TARGET_BLOCKS = 256
 _FIRST_ROUND = 256  # workgroups that start first, one on each compute unit
+# decode workgroups the chip holds at a time (three on each compute unit): a launch of more
+# hands them out longest request first
+_DECODE_ORDER_ABOVE = 768
 _MIN_SPLIT_KEYS = 128
 _MAX_SPLIT_PAGES = 1024  # page ids of one split are staged in LDS
 # The prefill kernel cuts its tiles' keys into runs when a launch has fewer workgroups than
@@ -926,6 +942,10 @@ def _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_s
     chunk = max(_MIN_SPLIT_KEYS, -(-(-(-span // want)) // 128) * 128)
     chunk = min(chunk, max(32, ((_MAX_SPLIT_PAGES - 1) * page_size - 31) // 32 * 32))
     nsplit = -(-span // chunk)
+    if plan.num_decode > 65535:
+        raise KernelError(f"{plan.num_decode} single-token requests exceed the decode kernel's launch grid")
+    # with more workgroups than start at once, the longest requests go first
+    order = plan.decode_order(ctx) if pairs * nsplit > _DECODE_ORDER_ABOVE else None
     part_o = part_ml = None
     if nsplit > 1:
         part_o = torch.empty((plan.num_decode, nq, nsplit, d), dtype=torch.float32, device=q.device)
@@ -937,7 +957,7 @@ def _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_s
     _ok(
         lib.rl_attn_decode(
             _p(q), _p(k_cache), _p(v_cache), _p(out), _p(part_o), _p(part_ml),
-            _p(plan.seq_token), _p(ctx.positions), _p(ctx.token_slot), _p(block_table),
+            _p(plan.seq_token), _p(order), _p(ctx.positions), _p(ctx.token_slot), _p(block_table),
             block_table.stride(0), page_size, plan.num_decode, nq, nkv, window,
             ctypes.c_float(scale), chunk, nsplit, int(fused is not None), _p(qn), _p(kn), _p(cos),
             _p(sin), _p(kw), _p(vw), ctypes.c_float(eps), _stream(),

@@ -119,6 +119,78 @@ def test_graph_of_a_batch_beyond_the_skinny_product(tmp_path, which, batch):
     assert any(key[0] >= batch for key in graph._graphs)  # padded up to a size of the ladder
 
 
+# four kv heads of 64 channels: the fused decode kernel, and many workgroups from few requests
+MANY_HEADS = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=72, num_attention_heads=8, num_key_value_heads=4,
+    head_dim=64, intermediate_size=152, vocab_size=307, rope_theta=60000.0,
+    rms_norm_eps=2e-6, tie_word_embeddings=True, max_position_embeddings=64,
+    hidden_act="silu", attention_bias=False,
+)
+
+
+def test_graph_of_more_requests_than_the_chip_holds_workgroups(tmp_path):
+    """200 requests on 4 kv heads are 800 decode workgroups, more than run at a time: the
+    decode attention then takes the requests longest first, from an order that a kernel of the
+    recorded step makes from the step's positions.  Between replays requests leave and others
+    of other lengths take rows of the batch, so that a replay which kept the recording's
+    order, or its lengths, would read other requests' keys or stop short of a request's own."""
+    from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry, write_random_model
+    from rapid_llm_amd.kernels import ops
+
+    batch, page, seed = 200, 8, 91
+    assert batch * MANY_HEADS["num_key_value_heads"] > ops._DECODE_ORDER_ABOVE
+    model_dir = tmp_path / "many_heads"
+    write_random_model(dict(MANY_HEADS), seed, model_dir, dtype="bfloat16", norm_std=0.1)
+    make = lambda graph: ModelRunner(
+        model_dir,
+        EngineConfig(dtype="bfloat16", max_seq_len=64, page_size=page, num_pages=batch * (64 // page + 1) + 8,
+                     max_num_seqs=batch + 1, use_graph=graph),
+    )
+    eager, graph = make(False), make(True)
+    pcfg, pw = plain_load(model_dir)
+    vocab = MANY_HEADS["vocab_size"]
+    nxt, seqs = {}, {}
+
+    def admit(rid, length, s):
+        prompt = random_tokens(length, vocab, s)
+        a = eager.step([StepEntry(rid, prompt, [length - 1])]).clone()
+        graph.step([StepEntry(rid, prompt, [length - 1])])
+        nxt[rid] = int(a[0].argmax())
+        seqs[rid] = list(prompt)
+
+    for i in range(batch):
+        admit(f"m{i}", 2 + (i * 7) % 47, seed + i)
+    for step in range(8):
+        entries = [StepEntry(rid, [tok], [0]) for rid, tok in nxt.items()]
+        a = eager.step(entries).clone()
+        b = graph.step(entries).clone()
+        torch.cuda.synchronize()
+        for rid, tok in nxt.items():
+            seqs[rid].append(tok)
+        rids = list(nxt)
+        parity.assert_bf16_close(b.cpu(), a.cpu(), f"graph of {batch} rows against eager/step {step}")
+        if step in (0, 4, 7):  # against the plain implementation: the shortest, the longest, some between
+            by_len = sorted(range(batch), key=lambda k: len(seqs[rids[k]]))
+            rows = by_len[:3] + by_len[-3:] + by_len[batch // 2 :: 37]
+            want = torch.stack([plain_forward(pcfg, pw, seqs[rids[k]])[-1] for k in rows])
+            parity.assert_bf16_close(b.cpu()[rows], want, f"graph of {batch} rows/step {step}")
+        for k, rid in enumerate(rids):
+            nxt[rid] = int(a[k].argmax())
+        if step == 3:  # twenty leave, twenty of other lengths arrive: the rows' lengths change
+            for i in range(0, batch, 10):
+                for r in (eager, graph):
+                    r.finish(f"m{i}")
+                del nxt[f"m{i}"], seqs[f"m{i}"]
+            for j in range(batch // 10):
+                admit(f"n{j}", 50 - (j * 11) % 49, seed + 1000 + j)
+    assert any(key[0] >= batch for key in graph._graphs)
+    for r in (eager, graph):
+        for rid in nxt:
+            r.finish(rid)
+        r.cache.check_invariants()
+
+
 def test_ragged_batches_share_a_few_graphs(tmp_path):
     """Requests that end at different times walk the batch size down one by one: the steps are
     padded with filler rows to a ladder of sizes, so few graphs are captured; with and without

@@ -140,6 +140,66 @@ def test_paged_attention(case, dtype):
         _close_bf16_attention(got, want, seqs, "paged")
 
 
+def test_order_by_length_names_the_longest_first():
+    """The order the decode attention hands its workgroups out in: the requests' indices by
+    descending last position, equal ones in their own order; with and without a list of the
+    requests' tokens, at sizes around the kernel's blocks of 256."""
+    import ctypes
+
+    ops = _ops()
+    core = ops.core()
+    gen = torch.Generator().manual_seed(5)
+    for n, spread in [(1, 10), (7, 3), (256, 40), (257, 100000), (700, 5)]:
+        lengths = torch.randint(0, spread, (n,), generator=gen, dtype=torch.int32)
+        want = sorted(range(n), key=lambda i: (-int(lengths[i]), i))
+        # (a) request i is token i
+        order = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+        dev_lengths = lengths.to(DEV)
+        rc = core.rl_order_by_length(ctypes.c_void_p(dev_lengths.data_ptr()), None, n,
+                                     ctypes.c_void_p(order.data_ptr()), ops._stream())
+        assert rc == 0 and order.cpu().tolist() == want, (n, spread)
+        # (b) the requests' tokens lie scattered among others
+        perm = torch.randperm(3 * n, generator=gen)[:n].to(torch.int32)
+        positions = torch.full((3 * n,), 10**6, dtype=torch.int32)
+        positions[perm.long()] = lengths
+        order.fill_(-1)
+        dev_positions, dev_tokens = positions.to(DEV), perm.to(DEV)
+        rc = core.rl_order_by_length(ctypes.c_void_p(dev_positions.data_ptr()),
+                                     ctypes.c_void_p(dev_tokens.data_ptr()), n,
+                                     ctypes.c_void_p(order.data_ptr()), ops._stream())
+        assert rc == 0 and order.cpu().tolist() == want, (n, spread, "scattered")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_decode_attention_of_many_requests_of_mixed_lengths(dtype):
+    """More workgroups than the chip holds at a time: the decode kernel then takes the requests
+    longest first, from an order made on the device, and every die a different head of each.
+    260 single tokens over contexts of 1 to 700 keys beside two portions, 3 kv heads of 2 query
+    heads; the request with the one-key context and the longest are both there."""
+    ops = _ops()
+    rng = random.Random(11)
+    nq, nkv, d, page = 6, 3, 64, 8
+    seqs = [(rng.randint(0, 699), 1) for _ in range(258)] + [(0, 1), (699, 1), (40, 9), (0, 3)]
+    rng.shuffle(seqs)
+    q, kc, vc, table, ctx, want = _paged_problem(seqs, nq, nkv, d, page, dtype, seed=77)
+    out = torch.full_like(q, float("nan"))
+    ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, 0, 1.0 / math.sqrt(d))
+    if dtype == torch.bfloat16:
+        plan = ops.attention_plan(ctx, nq // nkv, d)
+        assert plan.num_decode == 260 and plan.num_decode * nkv > ops._DECODE_ORDER_ABOVE
+        order = plan._decode_order
+        assert order is not None, "the launch was not ordered"
+        tokens = plan.seq_token.cpu().tolist()
+        lengths = [int(ctx.positions[t]) for t in tokens]
+        assert order.cpu().tolist() == sorted(range(260), key=lambda i: (-lengths[i], i))
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=2e-6)
+    else:
+        _close_bf16_attention(got, want, seqs, "mixed lengths")
+
+
 PREFILL_SHAPE_CASES = [
     # nq, nkv, d, page, window, seqs: portions only
     (8, 2, 128, 16, 0, [(0, 200), (700, 90), (0, 3)]),     # tiles of one step (the second wave group idle) and of many
