@@ -588,3 +588,178 @@ extern "C" int rl_gemm_mid_parts(const void* X, const void* W, float* part, int 
         hipLaunchKernelGGL((gemm_mid_kernel<4>), grid, block, 0, stream, x, w, part, M, N, K, ldx, ldw, per);
     return rl_launch_status();
 }
+
+// =========================================================================== //
+// 17 .. 256 rows over matrices of a few megabytes: the whole product in one launch
+// =========================================================================== //
+// Where a model's matrices are a few megabytes (Qwen3-0.6B: 4 to 13 MB) a decode step of tens
+// or hundreds of rows is bound by how long each kernel takes to get going, not by its bytes,
+// and the library's kernels for such shapes take 10 to 15 us each (few, large tiles that
+// walk K in sixteen dependent steps).  This is the mid-size kernel's tile (four waves of 16
+// weight rows, a chunk of X through LDS, two chunks of weights in flight) over a grid of
+// weight-row blocks x row blocks of X, writing bfloat16 directly; MB blocks of 16 rows of X a
+// workgroup.  SWIGLU: waves 0, 1 hold gate rows n .. n + 31, waves 2, 3 the up rows of the same
+// columns; the up halves cross LDS and the gate waves write silu(gate) * up, both rounded to
+// bfloat16 first as a stored product would be.
+template <int MB, bool SWIGLU>
+__global__ __launch_bounds__(MW* RL_WAVE) void gemm_tile_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, bf16_t* __restrict__ out, int M,
+    int N, int K, int ldx, int ldw, int ldo) {
+    __shared__ __attribute__((aligned(16))) unsigned char xs[2][MB * 16 * WT_PITCH];
+    __shared__ __attribute__((aligned(16))) unsigned char wtile[MW][16 * WT_PITCH];
+    const int tid = threadIdx.x, lane = tid & (RL_WAVE - 1), wave = tid / RL_WAVE;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int m0 = blockIdx.y * (16 * MB);
+    // first output column of the wave's tile, and the weight row that holds it
+    const int n0 = SWIGLU ? blockIdx.x * 32 + 16 * (wave & 1) : (blockIdx.x * MW + wave) * 16;
+    const int w0 = (SWIGLU && wave >= 2) ? N : 0;  // the up rows follow the N gate rows
+    const bf16_t* wld[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        wld[j] = W + (size_t)(w0 + min(n0 + 4 * j + g, N - 1)) * ldw + 8 * r16;
+    const bf16_t* xld[MB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+        xld[i] = X + (size_t)min(m0 + tid / 16 + 16 * i, M - 1) * ldx + 8 * (tid % 16);
+    unsigned char* mytile = wtile[wave];
+    f32x4 acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    bf16x8 wa[4], wb[4], xa[MB], xb[MB];
+    auto load = [&](bf16x8 (&w)[4], bf16x8 (&x)[MB], int c) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = ld16(wld[j] + c * KSTEP);
+#pragma unroll
+        for (int i = 0; i < MB; ++i) x[i] = ld16(xld[i] + c * KSTEP);
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay in front of the other chunk's products
+    };
+    auto stage = [&](bf16x8 (&x)[MB], int buf) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            *reinterpret_cast<bf16x8*>(xs[buf] + (tid / 16 + 16 * i) * WT_PITCH + 16 * (tid % 16)) = x[i];
+    };
+    auto products = [&](bf16x8 (&w)[4], int buf) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<bf16x8*>(mytile + (4 * j + g) * WT_PITCH + 16 * r16) = w[j];
+        bf16x8 a[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            a[j] = *reinterpret_cast<const bf16x8*>(mytile + r16 * WT_PITCH + 64 * g + 16 * j);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            bf16x8 xf[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                xf[j] = *reinterpret_cast<const bf16x8*>(xs[buf] + (mb * 16 + r16) * WT_PITCH + 64 * g + 16 * j);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], xf[j], acc[mb], 0, 0, 0);
+        }
+    };
+    // as in the mid-size kernel: chunk c's X lives in buffer c & 1, one barrier per chunk
+    int left = K / KSTEP;  // at least one (host-checked)
+    int c = 0;
+    load(wa, xa, c);
+    stage(xa, 0);
+    while (left > 2) {
+        load(wb, xb, c + 1);
+        __syncthreads();
+        products(wa, 0);
+        stage(xb, 1);
+        load(wa, xa, c + 2);
+        __syncthreads();
+        products(wb, 1);
+        stage(xa, 0);
+        c += 2;
+        left -= 2;
+    }
+    if (left == 2) {
+        load(wb, xb, c + 1);
+        __syncthreads();
+        products(wa, 0);
+        stage(xb, 1);
+        __syncthreads();
+        products(wb, 1);
+    } else {
+        __syncthreads();
+        products(wa, 0);
+    }
+    // acc[mb][i]: row m0 + 16 mb + r16 of X, column n0 + 4 g + i
+    if (SWIGLU) {
+        float* up = reinterpret_cast<float*>(xs);  // [2 waves][MB][4][64 lanes], where X was
+        static_assert(sizeof(float) * 2 * MB * 4 * RL_WAVE <= sizeof(xs), "the up halves fit where X was");
+        __syncthreads();  // every wave has read its last chunk of X
+        if (wave >= 2) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) up[(((wave - 2) * MB + mb) * 4 + i) * RL_WAVE + lane] = acc[mb][i];
+        }
+        __syncthreads();
+        if (wave >= 2) return;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float gate = bf16_to_float(float_to_bf16(acc[mb][i]));
+                const float u = bf16_to_float(float_to_bf16(up[((wave * MB + mb) * 4 + i) * RL_WAVE + lane]));
+                acc[mb][i] = gate / (1.f + expf(-gate)) * u;
+            }
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = m0 + mb * 16 + r16;
+        if (m >= M) continue;
+        bf16_t* dst = out + (size_t)m * ldo + n0 + 4 * g;
+        if (n0 + 4 * g + 3 < N) {
+            struct {
+                bf16_t v[4];
+            } o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o.v[i] = float_to_bf16(acc[mb][i]);
+            *reinterpret_cast<uint2*>(dst) = __builtin_bit_cast(uint2, o);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n0 + 4 * g + i < N) dst[i] = float_to_bf16(acc[mb][i]);
+        }
+    }
+}
+
+// out[M, N] = X W^T as bfloat16 (swiglu == 0), or out[M, N] = silu(X Wg^T) * (X Wu^T) with
+// W = [Wg | Wu] stacked by rows, [2N, K].  K a multiple of 128, ldo a multiple of 4.
+extern "C" int rl_gemm_tile(const void* X, const void* W, void* out, int M, int N, int K, int ldx,
+                            int ldw, int ldo, int swiglu, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return RL_OK;
+    if (K < KSTEP || K % KSTEP || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ldo % 4 || ldo < N || !out)
+        return RL_ERR_ARG;
+    const int row_blocks = (M + 63) / 64;
+    const int mb = ((M + row_blocks - 1) / row_blocks + 15) / 16;  // 16-row blocks a workgroup
+    if (row_blocks > 65535) return RL_ERR_ARG;
+    const int cols = swiglu ? 32 : MW * 16;
+    dim3 grid((N + cols - 1) / cols, (M + 16 * mb - 1) / (16 * mb)), block(MW * RL_WAVE);
+    const bf16_t* x = (const bf16_t*)X;
+    const bf16_t* w = (const bf16_t*)W;
+    bf16_t* o = (bf16_t*)out;
+#define RL_TILE(MBV)                                                                              \
+    do {                                                                                          \
+        if (swiglu)                                                                               \
+            hipLaunchKernelGGL((gemm_tile_kernel<MBV, true>), grid, block, 0, stream, x, w, o, M, \
+                               N, K, ldx, ldw, ldo);                                              \
+        else                                                                                      \
+            hipLaunchKernelGGL((gemm_tile_kernel<MBV, false>), grid, block, 0, stream, x, w, o,   \
+                               M, N, K, ldx, ldw, ldo);                                           \
+    } while (0)
+    if (mb == 1)
+        RL_TILE(1);
+    else if (mb == 2)
+        RL_TILE(2);
+    else if (mb == 3)
+        RL_TILE(3);
+    else
+        RL_TILE(4);
+#undef RL_TILE
+    return rl_launch_status();
+}

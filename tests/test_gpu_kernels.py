@@ -554,6 +554,64 @@ def test_gemm_bf16_swiglu_fused(shape):
     assert ops.gemm_bf16_swiglu(torch.zeros(33, k, dtype=torch.bfloat16, device=DEV), w.to(DEV)) is None
 
 
+# rows, result columns, K: row counts around the blocks of 16 and 64 rows, column counts that end
+# inside a workgroup's 64 (or 32) columns and inside a lane's four, one chunk of K and many
+TILE_SHAPES = [(17, 2048, 128), (33, 2052, 384), (64, 4096, 1024), (96, 2116, 256), (130, 3000, 640),
+               (256, 6144, 1024), (200, 2048, 3072)]
+
+
+@pytest.mark.parametrize("shape", TILE_SHAPES)
+def test_tile_product_of_small_matrices(shape):
+    """17 to 256 rows over a matrix of a few megabytes run one kernel of this package instead of
+    the library's; against the float32 product of the same bfloat16 operands."""
+    ops = _ops()
+    m, n, k = shape
+    assert ops._tile_applies(m, n, k, n)
+    a = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    w[n - 1] = 3.0 / math.sqrt(k)  # the last weight row and the last row of x stand out:
+    a[m - 1] = 1.0                 # a clamped or dropped edge shows
+    got = ops.gemm_bf16(a.to(DEV), w.to(DEV), torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and got.shape == (m, n)
+    want = a.float() @ w.float().T
+    torch.testing.assert_close(got.float().cpu(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("shape", [(17, 1024, 128), (40, 1028, 384), (64, 3072, 1024), (100, 1500, 256), (256, 3072, 1024)])
+def test_tile_product_with_swiglu(shape):
+    """The same kernel on the packed gate and up matrices, the activation in its epilogue:
+    silu(gate) * up of the products rounded to bfloat16, as the unfused path computes it."""
+    ops = _ops()
+    m, inter, k = shape
+    assert ops._tile_applies(m, 2 * inter, k, inter)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(2 * inter, k) / math.sqrt(k)).bfloat16()
+    w[inter - 1] = 2.0 / math.sqrt(k)      # the last gate row
+    w[2 * inter - 1] = -2.0 / math.sqrt(k)  # and the last up row
+    x[m - 1] = 1.0
+    got = ops.gemm_bf16_swiglu(x.to(DEV), w.to(DEV))
+    assert got is not None and got.shape == (m, inter)
+    gu = (x.float() @ w.float().T).bfloat16().float()
+    want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    torch.testing.assert_close(got.float().cpu(), want, rtol=2e-2, atol=2e-2)
+
+
+def test_tile_product_keeps_to_its_sizes():
+    """Few rows, many rows, large matrices, narrow ones and a K that is no multiple of 128 go
+    where they went before (the few-row kernel, the library)."""
+    ops = _ops()
+    assert not ops._tile_applies(16, 4096, 1024, 4096)
+    assert not ops._tile_applies(257, 4096, 1024, 4096)
+    assert not ops._tile_applies(64, 4096, 2048, 4096)   # 16 MB: the library is as fast
+    assert not ops._tile_applies(64, 1024, 2048, 1024)   # too few workgroups
+    assert not ops._tile_applies(64, 4096, 1000, 4096)
+    assert not ops._tile_applies(64, 4098, 1024, 4098)
+    x = torch.randn(64, 1000).bfloat16()
+    w = (torch.randn(4096, 1000) / 30).bfloat16()
+    got = ops.gemm_bf16(x.to(DEV), w.to(DEV), torch.bfloat16)
+    torch.testing.assert_close(got.float().cpu(), x.float() @ w.float().T, rtol=1e-2, atol=1e-2)
+
+
 @pytest.mark.parametrize("shape", [(1, 96, 64), (8, 4096, 4096), (16, 304, 1000), (5, 4096, 12288), (3, 40, 48)])
 def test_products_fold_the_norm_between_them(shape):
     """producer: residual += x W^T, rows * weight, pieces of the sums of squares; consumer:

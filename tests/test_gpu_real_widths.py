@@ -141,3 +141,58 @@ def test_benchmark_widths_match_plain(model, reference, dtype):
         runner.finish(rid)
     runner.cache.check_invariants()
     assert not runner.cache.live_requests()
+
+
+# Two layers at the widths of the family's smallest model (hidden 1,024, 16 query and 8 kv heads
+# of 128, intermediate 3,072), a short vocabulary: its QKV and gate/up matrices are the few
+# megabytes for which steps of 17 to 256 rows run the one-launch tile product (with SwiGLU in
+# its epilogue) instead of the library's kernels, and 200 requests on 8 kv heads are more decode
+# workgroups than run at once, so that the attention takes them longest first.
+SMALL = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8,
+    head_dim=128, intermediate_size=3072, vocab_size=1500, rope_theta=1000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=256,
+    hidden_act="silu", attention_bias=False,
+)
+
+
+@pytest.mark.parametrize("graph", [False, True], ids=["eager", "graph"])
+def test_smallest_widths_in_steps_of_tens_and_hundreds_of_rows(tmp_path, monkeypatch, graph):
+    from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry, write_random_model
+    from rapid_llm_amd.kernels import ops
+
+    folder = tmp_path / "small"
+    write_random_model(dict(SMALL), 3, folder, dtype="bfloat16", norm_std=0.1)
+    pcfg, pw = plain_load(folder)
+    took = []
+    applies = ops._tile_applies
+    monkeypatch.setattr(ops, "_tile_applies", lambda *a: took.append(applies(*a)) or took[-1])
+    runner = ModelRunner(
+        folder, EngineConfig(dtype="bfloat16", max_seq_len=128, page_size=16, num_pages=200 * 8 + 8,
+                             max_num_seqs=201, use_graph=graph),
+    )
+    vocab = SMALL["vocab_size"]
+    seqs = {f"r{i}": random_tokens(2 + (i * 13) % 90, vocab, 500 + i) for i in range(200)}
+    # prompts, several a step: portions of 100 to 400 rows beside nothing else (the library's sizes)
+    rids = list(seqs)
+    for at in range(0, 200, 8):
+        runner.step([StepEntry(r, seqs[r], []) for r in rids[at : at + 8]])
+    gen = torch.Generator().manual_seed(9)
+    for live in (40, 200, 17, 130):  # single tokens: 17 to 256 rows
+        chosen = [rids[int(i)] for i in torch.randperm(200, generator=gen)[:live]]
+        tokens = {r: int(torch.randint(0, vocab, (1,), generator=gen)) for r in chosen}
+        took.clear()
+        logits = runner.step([StepEntry(r, [tokens[r]], [0]) for r in chosen]).cpu()
+        assert any(took), f"{live} rows: the tile product was not used"
+        for r in chosen:
+            seqs[r].append(tokens[r])
+        order = sorted(range(live), key=lambda i: len(seqs[chosen[i]]))
+        rows = order[:4] + order[-4:] + order[live // 2 : live // 2 + 4]
+        want = torch.stack([plain_forward(pcfg, pw, seqs[chosen[i]])[-1] for i in rows])
+        parity.assert_bf16_close(logits[rows], want, f"smallest widths/{live} rows/graph={graph}")
+    if graph:
+        assert runner._graphs, "no step was replayed from a graph"
+    for r in rids:
+        runner.finish(r)
+    runner.cache.check_invariants()
