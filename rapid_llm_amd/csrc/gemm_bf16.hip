@@ -590,7 +590,7 @@ extern "C" int rl_gemm_mid_parts(const void* X, const void* W, float* part, int 
 }
 
 // =========================================================================== //
-// 17 .. 256 rows over matrices of a few megabytes: the whole product in one launch
+// 17 .. 512 rows over matrices of a few megabytes: the whole product in one launch
 // =========================================================================== //
 // Where a model's matrices are a few megabytes (Qwen3-0.6B: 4 to 13 MB) a decode step of tens
 // or hundreds of rows is bound by how long each kernel takes to get going, not by its bytes,

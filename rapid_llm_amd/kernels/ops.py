@@ -555,7 +555,7 @@ def gemm_bf16_residual(
     return rows, partial
 
 
-TILE_MAX_ROWS = 256  # rows up to which small matrices run the one-launch tile product
+TILE_MAX_ROWS = 512  # rows up to which small matrices run the one-launch tile product
 _TILE_MAX_WEIGHTS = 7 << 20  # elements of a matrix (14 MB) up to which it is used
 _TILE_MIN_COLS = 2048  # fewer columns leave too few workgroups
 
@@ -570,7 +570,11 @@ def _tile_applies(m: int, weight_rows: int, k: int, cols: int) -> bool:
     13.4 / 8.2, 13.5 / 10.9, 17.9 / 14.8 (inside a Qwen3-0.6B decode step the library's two
     take 11.5 and 13.8 + 4.6).  From 4,096 x 2,048 on the library is as fast or faster (11.1 /
     11.3, 11.6 / 14.4, 13.1 / 13.8), and matrices of 1,024 rows leave too few workgroups
-    (1,024 x 2,048: 8.2 / 9.0, 8.2 / 12.1, 8.6 / 12.3)."""
+    (1,024 x 2,048: 8.2 / 9.0, 8.2 / 12.1, 8.6 / 12.3).  Beyond 256 rows the library's kernels
+    are the faster ones on the device (512 rows: 10.6 / 12.2, with the activation 20.1 / 19.1;
+    1,024 rows: 13.5 / 21.3 and 25.7 / 32.6), but a step of a few hundred tokens of so small a
+    model is bound by the host, where a call of the library costs 18 us and one of this kernel
+    6: a 512-token prompt of the Qwen3-0.6B shape 5.4 -> 4.2 ms.  Hence up to 512 rows."""
     return (
         SKINNY_MAX_ROWS < m <= TILE_MAX_ROWS
         and k % 128 == 0
@@ -634,7 +638,7 @@ def add_rmsnorm_parts(
 
 def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> torch.Tensor | None:
     """``silu(x Wg^T) * (x Wu^T)`` for the packed ``[gate | up]`` matrix in one kernel: for
-    few rows, and for up to 256 rows over a small matrix; ``None`` when the shape is not one a
+    few rows, and for up to 512 rows over a small matrix; ``None`` when the shape is not one a
     fused kernel takes.  ``scaled``: as in ``gemm_bf16``."""
     m, k = x.shape
     two_i = w_gate_up.shape[0]

@@ -557,12 +557,12 @@ def test_gemm_bf16_swiglu_fused(shape):
 # rows, result columns, K: row counts around the blocks of 16 and 64 rows, column counts that end
 # inside a workgroup's 64 (or 32) columns and inside a lane's four, one chunk of K and many
 TILE_SHAPES = [(17, 2048, 128), (33, 2052, 384), (64, 4096, 1024), (96, 2116, 256), (130, 3000, 640),
-               (256, 6144, 1024), (200, 2048, 3072)]
+               (256, 6144, 1024), (200, 2048, 3072), (300, 2048, 256), (512, 4096, 1024)]
 
 
 @pytest.mark.parametrize("shape", TILE_SHAPES)
 def test_tile_product_of_small_matrices(shape):
-    """17 to 256 rows over a matrix of a few megabytes run one kernel of this package instead of
+    """17 to 512 rows over a matrix of a few megabytes run one kernel of this package instead of
     the library's; against the float32 product of the same bfloat16 operands."""
     ops = _ops()
     m, n, k = shape
@@ -577,7 +577,7 @@ def test_tile_product_of_small_matrices(shape):
     torch.testing.assert_close(got.float().cpu(), want, rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("shape", [(17, 1024, 128), (40, 1028, 384), (64, 3072, 1024), (100, 1500, 256), (256, 3072, 1024)])
+@pytest.mark.parametrize("shape", [(17, 1024, 128), (40, 1028, 384), (64, 3072, 1024), (100, 1500, 256), (256, 3072, 1024), (500, 1024, 384)])
 def test_tile_product_with_swiglu(shape):
     """The same kernel on the packed gate and up matrices, the activation in its epilogue:
     silu(gate) * up of the products rounded to bfloat16, as the unfused path computes it."""
@@ -601,7 +601,7 @@ def test_tile_product_keeps_to_its_sizes():
     where they went before (the few-row kernel, the library)."""
     ops = _ops()
     assert not ops._tile_applies(16, 4096, 1024, 4096)
-    assert not ops._tile_applies(257, 4096, 1024, 4096)
+    assert not ops._tile_applies(513, 4096, 1024, 4096)
     assert not ops._tile_applies(64, 4096, 2048, 4096)   # 16 MB: the library is as fast
     assert not ops._tile_applies(64, 1024, 2048, 1024)   # too few workgroups
     assert not ops._tile_applies(64, 4096, 1000, 4096)

@@ -145,7 +145,7 @@ def test_benchmark_widths_match_plain(model, reference, dtype):
 
 # Two layers at the widths of the family's smallest model (hidden 1,024, 16 query and 8 kv heads
 # of 128, intermediate 3,072), a short vocabulary: its QKV and gate/up matrices are the few
-# megabytes for which steps of 17 to 256 rows run the one-launch tile product (with SwiGLU in
+# megabytes for which steps of 17 to 512 rows run the one-launch tile product (with SwiGLU in
 # its epilogue) instead of the library's kernels, and 200 requests on 8 kv heads are more decode
 # workgroups than run at once, so that the attention takes them longest first.
 SMALL = dict(
@@ -174,7 +174,7 @@ def test_smallest_widths_in_steps_of_tens_and_hundreds_of_rows(tmp_path, monkeyp
     )
     vocab = SMALL["vocab_size"]
     seqs = {f"r{i}": random_tokens(2 + (i * 13) % 90, vocab, 500 + i) for i in range(200)}
-    # prompts, several a step: portions of 100 to 400 rows beside nothing else (the library's sizes)
+    # prompts, several a step: 100 to 500 rows, mostly the tile product's sizes, some the library's
     rids = list(seqs)
     for at in range(0, 200, 8):
         runner.step([StepEntry(r, seqs[r], []) for r in rids[at : at + 8]])
