@@ -153,3 +153,29 @@ def test_prefill_launch_shapes_follow_an_estimate_of_the_launch():
     assert shape([(0, 2048)] * 4) == (1, 1) and shape([(0, 20)]) == (1, 1)
     # a window bounds what every tile reads: the long prefix no longer counts
     assert shape([(16000, 150)], window=256) == (2, 1)
+
+
+def test_which_products_run_in_one_launch_of_this_package():
+    """The host's rule for the tile product (17 to 512 rows over a matrix of a few megabytes with
+    enough result columns for every compute unit): the smallest model's QKV and gate/up products
+    take it, its narrow products, larger models' matrices and steps of few or many rows do not."""
+    from rapid_llm_amd.kernels import ops
+
+    assert ops._tile_applies(64, 4096, 1024, 4096)        # Qwen3-0.6B QKV
+    assert ops._tile_applies(256, 6144, 1024, 3072)       # its packed gate and up rows, 3,072 results
+    assert ops._tile_applies(512, 4096, 1024, 4096)
+    assert not ops._tile_applies(16, 4096, 1024, 4096)    # the few-row kernel's
+    assert not ops._tile_applies(513, 4096, 1024, 4096)   # the library's
+    assert not ops._tile_applies(64, 1024, 2048, 1024)    # output projection: 16 workgroups a row block
+    assert not ops._tile_applies(64, 4096, 2048, 4096)    # 16 MB: the library is as fast
+    assert not ops._tile_applies(64, 6144, 4096, 6144)    # Qwen3-8B QKV
+    assert not ops._tile_applies(64, 4096, 1000, 4096)    # K in chunks of 128 only
+    assert not ops._tile_applies(64, 4098, 1024, 4098)    # four result columns a lane
+
+
+def test_the_decode_launch_is_ordered_only_beyond_what_runs_at_once():
+    """Decode attention asks for the requests' order by length only when the launch has more
+    workgroups than the chip holds at a time (three on each of 256 compute units)."""
+    from rapid_llm_amd.kernels import ops
+
+    assert ops._DECODE_ORDER_ABOVE == 3 * 256
