@@ -542,15 +542,14 @@ __global__ void qknorm_rope_kvwrite_kernel(
 // 128, else 32) take one head, a wave takes 64 / LPH heads, and every load and store moves 8
 // or 16 bytes.  Needs d % 8 == 0.
 template <typename T, int LPH>
-__global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
-    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
+__device__ inline void qknorm_rope_kvwrite_vec(
+    int t, int head_group, const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const float* __restrict__ q_norm_w,
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values) {
     constexpr int HPW = RL_WAVE / LPH;  // heads per wave
-    const int t = blockIdx.x;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
     const int sub = lane / LPH;  // which of the wave's heads
@@ -565,7 +564,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
         page = (size_t)block_table[(size_t)token_slot[t] * table_stride + pos / page_size];
         off = pos % page_size;
     }
-    const int head = (blockIdx.y * (blockDim.x / RL_WAVE) + wave) * HPW + sub;
+    const int head = (head_group * (blockDim.x / RL_WAVE) + wave) * HPW + sub;
     if (head >= total_heads) return;  // whole groups of LPH lanes leave together
     const T* x = row + (size_t)head * d;
     const bool active = 4 * li < half;
@@ -627,6 +626,19 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
     *reinterpret_cast<Vec4<T>*>(dst + half + 4 * li) = ob;
 }
 
+template <typename T, int LPH>
+__global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, const int* __restrict__ positions,
+    const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
+    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values) {
+    qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x, blockIdx.y, qkv, q_out, k_cache, v_cache, q_norm_w, k_norm_w,
+                                    cos_tab, sin_tab, positions, token_slot, block_table, table_stride,
+                                    page_size, nq, nkv, d, eps, write_cache, write_values);
+}
+
 template <typename T>
 static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const float* q_norm_w,
                           const float* k_norm_w, const float* cos_tab, const float* sin_tab,
@@ -670,15 +682,14 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
 #define VT_TOKENS 16
 
 template <typename T>
-__global__ __launch_bounds__(256) void v_tile_write_kernel(
-    const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
+__device__ inline void v_tile_write(
+    int tile, int h, const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int tokens, int nq, int nkv, int d) {
     __shared__ T vt[VT_TOKENS][256 + 8];
     __shared__ int s_page[VT_TOKENS];
     __shared__ int s_off[VT_TOKENS];
-    const int t0 = blockIdx.x * VT_TOKENS;
-    const int h = blockIdx.y;
+    const int t0 = tile * VT_TOKENS;
     const int row_width = (nq + 2 * nkv) * d;
     if (threadIdx.x < VT_TOKENS) {
         const int t = t0 + threadIdx.x;
@@ -721,6 +732,63 @@ __global__ __launch_bounds__(256) void v_tile_write_kernel(
     }
 }
 
+// One launch for a step of many tokens: the first tokens * head_groups workgroups norm, rotate
+// and write the query and key heads of one token each, the rest write the values of 16 tokens
+// and one kv head each.  A workgroup is wholly one or the other.
+template <typename T, int LPH>
+__global__ __launch_bounds__(256) void qkv_prepare_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, const int* __restrict__ positions,
+    const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
+    int page_size, int tokens, int head_groups, int nq, int nkv, int d, float eps) {
+    const int qk_blocks = tokens * head_groups;
+    if ((int)blockIdx.x < qk_blocks) {
+        qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x / head_groups, blockIdx.x % head_groups, qkv, q_out, k_cache,
+                                        v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
+                                        block_table, table_stride, page_size, nq, nkv, d, eps, 1, 0);
+    } else {
+        const int b = blockIdx.x - qk_blocks;
+        v_tile_write<T>(b / nkv, b % nkv, qkv, v_cache, positions, token_slot, block_table, table_stride,
+                        page_size, tokens, nq, nkv, d);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void v_tile_write_kernel(
+    const T* __restrict__ qkv, T* __restrict__ v_cache, const int* __restrict__ positions,
+    const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
+    int page_size, int tokens, int nq, int nkv, int d) {
+    v_tile_write<T>(blockIdx.x, blockIdx.y, qkv, v_cache, positions, token_slot, block_table, table_stride,
+                    page_size, tokens, nq, nkv, d);
+}
+
+// true if it launched: head sizes in steps of 8, and a grid that fits
+template <typename T>
+static bool launch_qkv_prepare(const T* qkv, T* q_out, T* k_cache, T* v_cache, const float* q_norm_w,
+                               const float* k_norm_w, const float* cos_tab, const float* sin_tab,
+                               const int* positions, const int* token_slot, const int* block_table,
+                               int table_stride, int page_size, int tokens, int nq, int nkv, int d,
+                               float eps, hipStream_t stream) {
+    if (d % 8) return false;
+    const int lph = d <= 128 ? 16 : 32;
+    const int heads_per_block = 4 * (RL_WAVE / lph);
+    const int head_groups = (nq + nkv + heads_per_block - 1) / heads_per_block;
+    const long blocks = (long)tokens * head_groups + (long)((tokens + VT_TOKENS - 1) / VT_TOKENS) * nkv;
+    if (blocks > 0x7fffffffL) return false;
+    dim3 grid((unsigned)blocks), block(256);
+    if (lph == 16)
+        hipLaunchKernelGGL((qkv_prepare_kernel<T, 16>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
+                           q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
+                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps);
+    else
+        hipLaunchKernelGGL((qkv_prepare_kernel<T, 32>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
+                           q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
+                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps);
+    return true;
+}
+
 extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cache, void* v_cache,
                                       const float* q_norm_w, const float* k_norm_w,
                                       const float* cos_tab, const float* sin_tab,
@@ -739,6 +807,16 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
     if ((long)nq + 2 * nkv > 65535 * 4) return RL_ERR_ARG;
     dim3 block(256);
     dim3 vgrid((tokens + VT_TOKENS - 1) / VT_TOKENS, nkv);
+    if (tile_values && act_type == RL_F32 &&
+        launch_qkv_prepare<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, q_norm_w,
+                                  k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
+                                  table_stride, page_size, tokens, nq, nkv, d, eps, stream))
+        return rl_launch_status();
+    if (tile_values && act_type == RL_BF16 &&
+        launch_qkv_prepare<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                                   q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
+                                   table_stride, page_size, tokens, nq, nkv, d, eps, stream))
+        return rl_launch_status();
     if (act_type == RL_F32) {
         launch_qknorm<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
                              q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
