@@ -1,6 +1,6 @@
 // Bandwidth-bound bfloat16 product for few rows (decode): out[M,N] = X[M,K] * W[N,K]^T with
 // M <= 16, float32 accumulation on the matrix cores, optionally fused with SwiGLU.  (The last
-// section of the file holds the product for 17 to 64 rows of the narrow matrices.)
+// section of the file holds the products for 17 rows and more of narrow and of small matrices.)
 //
 // Every weight byte is read once, in long contiguous runs: a workgroup owns NT tiles of 16
 // weight rows and its 8 waves interleave over K in steps of 128 elements, so that at any
@@ -446,7 +446,7 @@ extern "C" int rl_gemm_skinny_residual(const void* X, const void* W, int M, int 
 }
 
 // =========================================================================== //
-// 17 .. 64 rows: the runs of K of a product whose result feeds the residual
+// 17 .. 192 rows: the runs of K of a product whose result feeds the residual
 // =========================================================================== //
 // The library's product reads X once for every 16 or 32 weight rows at these sizes and
 // stays near 3 TB/s.  Here a workgroup is four waves with 16 weight rows each; the chunk of X
@@ -457,7 +457,9 @@ extern "C" int rl_gemm_skinny_residual(const void* X, const void* W, int M, int 
 // them (rl_add_rmsnorm_parts).  Measured against the library at 64 rows (Qwen3-8B shapes,
 // microseconds): 4,096 x 4,096 11.8 / 14.9, 4,096 x 12,288 26.6 / 38.1; at 32 rows 9.9 / 13.9
 // and 23.0 / 28.6.  The wide products (6,144 and 24,576 rows) gain nothing (18.3 / 18.1 and
-// 55 / 46) and stay with the library.
+// 55 / 46) and stay with the library.  More than 64 rows run as blocks of 64 rows (grid.z), each
+// reading the weights again: up to about 192 rows that is still faster than the library's kernels
+// for such shapes (the host's rule holds the measurements).
 #define MW 4  // waves per workgroup
 
 template <int MB>
@@ -470,6 +472,7 @@ __global__ __launch_bounds__(MW* RL_WAVE) void gemm_mid_kernel(
     const int r16 = lane & 15, g = lane >> 4;
     const int n0 = (blockIdx.x * MW + wave) * 16;
     const int run = blockIdx.y;
+    const int m0 = blockIdx.z * 64;  // more than 64 rows: blocks of 64 (grid.z)
     const int c_lo = run * chunks_per_run, c_hi = min(K / KSTEP, c_lo + chunks_per_run);
     // weights: instruction j reads row 4j + g of the wave's tile at bytes 16 r16 (as the skinny
     // product does); rows beyond the matrix read its last row, their results are dropped
@@ -479,7 +482,7 @@ __global__ __launch_bounds__(MW* RL_WAVE) void gemm_mid_kernel(
     // X: thread reads bytes 16 (tid % 16) of rows tid / 16 + 16 i; rows beyond M read the last
     const bf16_t* xld[MB];
 #pragma unroll
-    for (int i = 0; i < MB; ++i) xld[i] = X + (size_t)min(tid / 16 + 16 * i, M - 1) * ldx + 8 * (tid % 16);
+    for (int i = 0; i < MB; ++i) xld[i] = X + (size_t)min(m0 + tid / 16 + 16 * i, M - 1) * ldx + 8 * (tid % 16);
     unsigned char* mytile = wtile[wave];
     f32x4 acc[MB];
 #pragma unroll
@@ -552,7 +555,7 @@ __global__ __launch_bounds__(MW* RL_WAVE) void gemm_mid_kernel(
     // acc[mb][i]: row 16 mb + r16 of X, weight row n0 + 4 g + i
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-        const int m = mb * 16 + r16;
+        const int m = m0 + mb * 16 + r16;
         if (m >= M) continue;
         float* dst = part + ((size_t)run * M + m) * N + n0 + 4 * g;
         if (n0 + 4 * g + 3 < N) {
@@ -566,16 +569,16 @@ __global__ __launch_bounds__(MW* RL_WAVE) void gemm_mid_kernel(
 }
 
 // part [ks, M, N] float32: run r holds X[:, r-th run of K] W[:, the same]^T.  K a multiple of
-// 128, N a multiple of 4, 1 <= M <= 64.
+// 128, N a multiple of 4; more than 64 rows run as blocks of 64.
 extern "C" int rl_gemm_mid_parts(const void* X, const void* W, float* part, int M, int N, int K,
                                  int ldx, int ldw, int ks, hipStream_t stream) {
     if (M <= 0 || N <= 0) return RL_OK;
-    if (M > 64 || K < KSTEP || K % KSTEP || N % 4 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ks < 1 ||
+    if (M > 64 * 65535 || K < KSTEP || K % KSTEP || N % 4 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || ks < 1 ||
         ks > K / KSTEP || !part)
         return RL_ERR_ARG;
     const int chunks = K / KSTEP, per = (chunks + ks - 1) / ks;
     if ((per * (ks - 1)) >= chunks) return RL_ERR_ARG;  // every run holds a chunk
-    dim3 grid((N + MW * 16 - 1) / (MW * 16), ks), block(MW * RL_WAVE);
+    dim3 grid((N + MW * 16 - 1) / (MW * 16), ks, (M + 63) / 64), block(MW * RL_WAVE);
     const bf16_t* x = (const bf16_t*)X;
     const bf16_t* w = (const bf16_t*)W;
     if (M <= 16)

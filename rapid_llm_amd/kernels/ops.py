@@ -584,7 +584,16 @@ def _tile_applies(m: int, weight_rows: int, k: int, cols: int) -> bool:
     )
 
 
-MID_MAX_ROWS = 64  # rows up to which a product's runs of K may be left to the norm that follows
+# Rows up to which a product's runs of K may be left to the norm that follows.  Beyond 64 rows the
+# kernel runs blocks of 64 rows.  Against the library's product and the plain norm, microseconds
+# (the library first): Qwen3-8B output projection 18.7 / 15.2 at 64 rows, 28.1 / 19.9 at 128,
+# 36.5 / 24.4 at 192, 27.1 / 30.1 at 256; down projection 40.6 / 30.6, 68.8 / 42.4, 92.6 / 56.4,
+# 57.4 / 72.6; the 32B shape's down projection 160 / 65, 184 / 100, 214 / 137, 265 / 180.  The
+# library's time jumps between neighbouring row counts (the 8B down projection: 51.8 at 144 rows,
+# 78.8 at 160, 55.4 at 176), this kernel's grows with the blocks of 64; from about 200 rows on
+# the library's best kernels are the faster ones.  Small matrices (the 0.6B and 1.7B shapes) are
+# within a microsecond either way from 144 rows on.
+MID_MAX_ROWS = 192
 _MID_BLOCK_ROWS = 64  # weight rows per workgroup of the mid-size product
 _MID_TARGET_BLOCKS = 256  # workgroups to reach by cutting K
 _MID_MAX_BLOCKS = 128  # wider matrices than this many workgroups stay with the library
@@ -604,7 +613,7 @@ def mid_runs(n: int, k: int) -> int:
 
 
 def gemm_bf16_parts(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """``x[M,K] @ w[N,K]^T`` for 17 to 64 rows as float32 runs of K, ``[runs, M, N]``: their sum
+    """``x[M,K] @ w[N,K]^T`` for 17 to 192 rows as float32 runs of K, ``[runs, M, N]``: their sum
     is the product.  For products whose result goes into the residual: the norm that follows
     adds the runs (``add_rmsnorm_parts``)."""
     _need(x, "x", torch.bfloat16)

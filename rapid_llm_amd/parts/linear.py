@@ -9,7 +9,7 @@ Which product runs is decided by the weight's storage type:
   checkpoint stores in 32-bit is used at full precision in a bfloat16 engine too.
 * bfloat16 weight: few rows (decode) go to the hand-written bandwidth-bound matrix-core
   kernel; many rows go to the library product, as in the reference, whose dense products
-  are ``F.linear`` (rapid_llm/kernels/ops/gemm/linear.py:17-40).  In between (17 to 64 rows) a
+  are ``F.linear`` (rapid_llm/kernels/ops/gemm/linear.py:17-40).  In between (17 to 192 rows) a
   narrow matrix whose result a norm adds to the residual may hand that norm float32 runs of
   K instead (``partial_sums``).
 """
@@ -72,7 +72,7 @@ class Linear:
 
     def deferred(self, x: torch.Tensor, ctx=None):
         """The product, or a :class:`DeferredProduct` of it where one of this product's kernels
-        could fold a neighbouring norm into itself (bfloat16, up to 16 rows, or 17 to 64 rows of a
+        could fold a neighbouring norm into itself (bfloat16, up to 16 rows, or 17 to 192 rows of a
         narrow matrix).  Whoever receives it and has no use for that simply materialises it."""
         if isinstance(x, torch.Tensor) and self.folds(x):
             return DeferredProduct(self, x)

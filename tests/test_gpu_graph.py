@@ -72,10 +72,11 @@ def test_graph_replays_match_eager(tmp_path, which, dtype):
         r.cache.check_invariants()
 
 
-@pytest.mark.parametrize("which,batch", [("B", 17), ("B", 40), ("E", 23), ("E", 64)])
+@pytest.mark.parametrize("which,batch", [("B", 17), ("B", 40), ("E", 23), ("E", 64), ("E", 100), ("E", 150)])
 def test_graph_of_a_batch_beyond_the_skinny_product(tmp_path, which, batch):
     """More than 16 rows: the bfloat16 products are the library's, and in configuration E the
-    output and down projections run as runs of K that the norms add.  The graph replays are
+    output and down projections run as runs of K that the norms add (up to 192 rows, beyond 64 in
+    blocks of 64 rows: the batches of 100 and 150 are recorded at 128 and 192 rows).  The graph replays are
     checked one by one against eager steps of a second engine, with eager work between."""
     from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
 

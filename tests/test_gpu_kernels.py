@@ -659,14 +659,18 @@ def test_products_fold_the_norm_between_them(shape):
     assert torch.equal(rows2, rows) and torch.equal(partial2, partial) and torch.equal(res2, res)
 
 
-@pytest.mark.parametrize("shape", [(17, 4096, 4096), (64, 4096, 12288), (33, 200, 256), (48, 1000, 1280), (20, 64, 128)])
+@pytest.mark.parametrize("shape", [(17, 4096, 4096), (64, 4096, 12288), (33, 200, 256), (48, 1000, 1280), (20, 64, 128),
+                                   (65, 200, 256), (100, 4096, 4096), (130, 1000, 1280), (192, 1024, 2048)])
 def test_product_in_runs_of_k_and_the_norm_that_adds_them(shape):
-    """17 to 64 rows: the product of a narrow matrix as float32 runs of K, and the norm kernel
-    that adds the runs, against the library product followed by the ordinary norm."""
+    """17 to 192 rows (beyond 64 in blocks of 64 rows): the product of a narrow matrix as float32
+    runs of K, and the norm kernel that adds the runs, against the library product followed by
+    the ordinary norm."""
     ops = _ops()
     m, n, k = shape
+    assert m <= ops.MID_MAX_ROWS
     gen = torch.Generator().manual_seed(m + n)
     x = (torch.randn((m, k), generator=gen)).bfloat16()
+    x[m - 1] = 1.0  # the last row stands out: a block of rows that stops short shows
     w = (torch.randn((n, k), generator=gen) * 0.05).bfloat16()
     assert ops.mid_runs(n, k) >= 1
     parts = ops.gemm_bf16_parts(x.to(DEV), w.to(DEV))
