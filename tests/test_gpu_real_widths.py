@@ -27,7 +27,11 @@ CONFIG = dict(
     hidden_act="silu", attention_bias=False,
 )
 PAGE = 16
-DECODE_STEPS = 2  # single-token steps at each batch size
+DECODE_STEPS = 2  # single-token steps at batch 1 and 8
+# at batch 64 the recorded step holds the library's products, some of them kernels that clear a
+# workspace first: three replays, with an eager prompt step of another request between them,
+# each checked against the plain implementation
+BATCH64_STEPS = 3
 # float32: sums of 4,096 to 12,288 terms in another order than the plain product's
 F32_TOL = dict(rtol=1e-4, atol=5e-5)
 
@@ -37,10 +41,12 @@ class _Sequences:
 
     def __init__(self):
         vocab = CONFIG["vocab_size"]
-        tail = 3 * DECODE_STEPS  # the longest-lived request decodes at batch 1, 8 and 64
+        tail = 2 * DECODE_STEPS + 1 + BATCH64_STEPS  # the longest-lived request decodes at batch 1 and 8, in the mixed step and at batch 64
         self.prompt = {"a": 2048, "b": 2560, "c": 700}
         for i in range(61):
             self.prompt[f"s{i}"] = 3 + (i * 7) % 90
+        for i in range(BATCH64_STEPS):
+            self.prompt[f"z{i}"] = 40 + 30 * i  # admitted between the replays at batch 64, never decoded
         self.tokens = {rid: random_tokens(n + tail, vocab, 1000 + k) for k, (rid, n) in enumerate(self.prompt.items())}
         self.rows: dict[str, list[int]] = {rid: [] for rid in self.prompt}
 
@@ -87,8 +93,10 @@ def _plan(seqs):
     rest = [f"s{i}" for i in range(5, 61)]
     steps.append(("mixed", [entry(r, 1, [0]) for r in eight] + [entry(r, seqs.prompt[r], [seqs.prompt[r] - 1]) for r in rest], False))
     everyone = eight + rest
-    for i in range(DECODE_STEPS - 1):
+    for i in range(BATCH64_STEPS):
         steps.append((f"batch 64 step {i}", [entry(r, 1, [0]) for r in everyone], True))
+        z = f"z{i}"
+        steps.append((f"a prompt between the replays ({z})", [entry(z, seqs.prompt[z], [seqs.prompt[z] - 1])], False))
     return steps
 
 
@@ -115,7 +123,7 @@ def test_benchmark_widths_match_plain(model, reference, dtype):
     seqs, steps, plain = reference
     runner = ModelRunner(
         model,
-        EngineConfig(dtype=dtype, max_seq_len=4096, page_size=PAGE, num_pages=1200, max_num_seqs=64, use_graph=True),
+        EngineConfig(dtype=dtype, max_seq_len=4096, page_size=PAGE, num_pages=1200, max_num_seqs=68, use_graph=True),
     )
     for label, entries, graph in steps:
         before = set(runner._graphs)
