@@ -358,6 +358,202 @@ static int launch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int
     return rl_launch_status();
 }
 
+// --------------------------------------------------------------------------- //
+// The gate/up product where the matrix has more (gate, up) pairs of tiles than the chip has
+// compute units.  The kernel above needs the registers of a whole compute unit for one
+// workgroup (two chunks of two tiles in flight per wave), so its workgroups follow each other
+// on a unit, and between two of them the unit streams nothing: the last waves drain, the
+// epilogue runs, the next workgroup asks for its first weights (cycle stamps: three workgroups
+// of 12.3 us a unit for the 24,576 rows of Qwen3-8B, 1.5 us of each the epilogue and as much
+// again before its loads come back).  Here a unit gets one workgroup that walks its pairs
+// b, b + G, b + 2G, .. as one stream of chunks: a wave that has its last chunk of a pair in
+// flight asks for its first of the next, puts the pair's sums into LDS when they are complete,
+// and the one epilogue at the end folds the waves' sums of every pair, in the order of the
+// waves: bit for bit what the kernel above computes.
+// --------------------------------------------------------------------------- //
+#define SW_MAX_TILES 7  // pairs a workgroup may walk (their partial sums wait in LDS: 16 KB a pair)
+
+template <bool SCALED>
+__global__ __launch_bounds__(GW* RL_WAVE) void gemm_swiglu_stream_kernel(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, bf16_t* __restrict__ out, int M,
+    int I, int K, int ldx, int ldw, int ldo, int pairs, SkinnyExtra ex) {
+    __shared__ float red[SW_MAX_TILES][GW][2 * 256];
+    __shared__ __attribute__((aligned(16))) unsigned char wtile[GW][16 * WT_PITCH];
+    __shared__ float wave_part[SCALED ? GW : 1][16];
+
+    const int lane = threadIdx.x & (RL_WAVE - 1);
+    const int wave = threadIdx.x / RL_WAVE;
+    const int r16 = lane & 15;
+    const int g = lane >> 4;
+    // pairs of this workgroup: blockIdx.x, + gridDim.x, ..  (host: at most SW_MAX_TILES)
+    const int T = (pairs - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    const size_t pair_stride = (size_t)gridDim.x * 16 * ldw;  // elements between two of its pairs
+    // instruction j of tile nt (0: gate, 1: up) reads row 4j + g of the tile at bytes 16 r16
+    const bf16_t* wld[2][4];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            wld[nt][j] = W + (size_t)(nt * I + blockIdx.x * 16 + 4 * j + g) * ldw + 8 * r16;
+    const bf16_t* xrow = X + (size_t)(r16 < M ? r16 : 0) * ldx + 32 * g;
+    unsigned char* mytile = wtile[wave];
+
+    f32x4 acc[2];
+    acc[0] = acc[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    constexpr int XP_AHEAD = 8;
+    float x_part[XP_AHEAD];
+    constexpr int S = GW * KSTEP;
+    const int k0 = wave * KSTEP;
+    const int nchunk = (K - k0 + S - 1) / S;  // chunks of this wave in a pair: at least one (host)
+    {
+        bf16x8 wa[2][4], wb[2][4], xa[4], xb[4];
+        auto load = [&](bf16x8 (&r)[2][4], bf16x8 (&xx)[4], int t, int kw) {
+            const size_t off = (size_t)t * pair_stride + kw;
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) r[nt][j] = ld16(wld[nt][j] + off);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xx[j] = ld16(xrow + kw + 8 * j);
+        };
+        // the chunk's products; `last`: the wave's last chunk of pair t, whose sums go to LDS
+        auto products = [&](bf16x8 (&r)[2][4], bf16x8 (&xx)[4], int t, bool last) {
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    *reinterpret_cast<bf16x8*>(mytile + (4 * j + g) * WT_PITCH + 16 * r16) = r[nt][j];
+                bf16x8 a[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    a[j] = *reinterpret_cast<const bf16x8*>(mytile + r16 * WT_PITCH + 64 * g + 16 * j);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], xx[j], acc[nt], 0, 0, 0);
+            }
+            if (last) {  // the same for every lane of the wave
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        red[t][wave][(nt * 4 + i) * 64 + lane] = acc[nt][i];
+                        acc[nt][i] = 0.f;
+                    }
+            }
+        };
+        auto partial_loads = [&]() {
+            if constexpr (SCALED) {
+                const int m = threadIdx.x & 15, j = threadIdx.x >> 4;  // 512 threads: 32 runs
+#pragma unroll
+                for (int i = 0; i < XP_AHEAD; ++i)
+                    x_part[i] = ex.x_partial[min(j + 32 * i, ex.x_parts - 1) * 16 + m];
+            }
+        };
+        // the wave's chunks of all its pairs as one sequence: (pair t, chunk i), two in flight
+        int ta = 0, ia = 0, tb = 0, ib = 0;
+        auto next = [&](int& t, int& i, int t0, int i0) {
+            i = i0 + 1;
+            t = t0;
+            if (i == nchunk) {
+                i = 0;
+                t = t0 + 1;
+            }
+        };
+        int left = T * nchunk;
+        load(wa, xa, 0, k0);
+        while (left > 2) {
+            next(tb, ib, ta, ia);
+            load(wb, xb, tb, k0 + ib * S);
+            products(wa, xa, ta, ia == nchunk - 1);
+            next(ta, ia, tb, ib);
+            load(wa, xa, ta, k0 + ia * S);
+            products(wb, xb, tb, ib == nchunk - 1);
+            left -= 2;
+        }
+        if (left == 2) {
+            next(tb, ib, ta, ia);
+            load(wb, xb, tb, k0 + ib * S);
+            partial_loads();
+            products(wa, xa, ta, ia == nchunk - 1);
+            products(wb, xb, tb, true);
+        } else {
+            partial_loads();
+            products(wa, xa, ta, true);
+        }
+    }
+    if constexpr (SCALED) {
+        const int m = threadIdx.x & 15, j = threadIdx.x >> 4;
+        float run = 0.f;
+#pragma unroll
+        for (int i = 0; i < XP_AHEAD; ++i) run += (j + 32 * i < ex.x_parts) ? x_part[i] : 0.f;
+        for (int p = j + 32 * XP_AHEAD; p < ex.x_parts; p += 32) run += ex.x_partial[p * 16 + m];
+        run = sum_rows_of_16(run);
+        if (g == 0) wave_part[wave][m] = run;
+    }
+    __syncthreads();  // every wave's sums of every pair are in LDS
+
+    // thread -> (pair t, lane of its tile); sums the waves in order
+    for (int e = threadIdx.x; e < T * 64; e += GW * RL_WAVE) {
+        const int ln = e & 63;
+        const int t = e >> 6;
+        const int m = ln & 15;
+        if (m >= M) continue;
+        const int nbase = ((int)blockIdx.x + t * (int)gridDim.x) * 16 + 4 * (ln >> 4);
+        float scale = 1.f;
+        if constexpr (SCALED) {
+            float ss = 0.f;
+#pragma unroll
+            for (int w = 0; w < GW; ++w) ss += wave_part[w][m];
+            scale = rsqrtf(ss * ex.x_inv_size + ex.x_eps);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float gate = 0.f, up = 0.f;
+#pragma unroll
+            for (int w = 0; w < GW; ++w) {
+                gate += red[t][w][i * 64 + ln];
+                up += red[t][w][(4 + i) * 64 + ln];
+            }
+            // operands rounded to bfloat16, as where the product's result is stored first
+            gate = bf16_to_float(float_to_bf16(gate * scale));
+            up = bf16_to_float(float_to_bf16(up * scale));
+            out[(size_t)m * ldo + nbase + i] = float_to_bf16(gate / (1.f + expf(-gate)) * up);
+        }
+    }
+}
+
+// the chip's compute units (one workgroup of the stream kernel each)
+static int compute_units() {
+    static int units[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (units[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        units[dev] = n;
+    }
+    return units[dev];
+}
+
+// true (and *rc set) if the stream kernel took the product
+static bool swiglu_stream(const bf16_t* X, const bf16_t* W, bf16_t* out, int M, int I, int K, int ldx,
+                          int ldw, int ldo, const SkinnyExtra& ex, hipStream_t stream, int* rc) {
+    const int units = compute_units();
+    const int pairs = I / 16;
+    if (units <= 0 || I % 16 || K % KSTEP || K < GW * KSTEP || pairs <= units) return false;
+    const int per = (pairs + units - 1) / units;  // pairs a workgroup
+    if (per > SW_MAX_TILES) return false;
+    dim3 grid((pairs + per - 1) / per), block(GW * RL_WAVE);
+    if (ex.x_partial)
+        hipLaunchKernelGGL((gemm_swiglu_stream_kernel<true>), grid, block, 0, stream, X, W, out, M, I, K,
+                           ldx, ldw, ldo, pairs, ex);
+    else
+        hipLaunchKernelGGL((gemm_swiglu_stream_kernel<false>), grid, block, 0, stream, X, W, out, M, I, K,
+                           ldx, ldw, ldo, pairs, ex);
+    *rc = rl_launch_status();
+    return true;
+}
+
 template <typename OutT, bool SWIGLU>
 static int dispatch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
                     int ldw, int ldo, int nt, const SkinnyExtra& ex, hipStream_t stream) {
@@ -413,16 +609,22 @@ extern "C" int rl_gemm_skinny(const void* X, const void* W, void* out, int M, in
     return RL_ERR_ARG;
 }
 
-// out[M, I] = silu(X Wg^T) * (X Wu^T) with W = [Wg | Wu] stacked by rows, [2I, K].
+// out[M, I] = silu(X Wg^T) * (X Wu^T) with W = [Wg | Wu] stacked by rows, [2I, K].  A matrix
+// with more pairs of tiles than compute units goes to the stream kernel (nt < 0: never, the
+// kernel of one pair a workgroup with -nt tiles: for comparing the two).
 extern "C" int rl_gemm_skinny_swiglu(const void* X, const void* W, void* out, int M, int I, int K,
                                      int ldx, int ldw, int ldo, int nt, const float* x_partial,
                                      int x_parts, int x_size, float x_eps, hipStream_t stream) {
     if (M <= 0 || I <= 0) return RL_OK;
     if (!skinny_args_ok(M, K, ldx, ldw) || ldo < I || (x_partial && (x_parts < 1 || x_size < 1)))
         return RL_ERR_ARG;
+    const SkinnyExtra ex = scaled_input(x_partial, x_parts, x_size, x_eps);
+    int rc = RL_OK;
+    if (nt >= 0 && swiglu_stream((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx, ldw, ldo, ex,
+                                 stream, &rc))
+        return rc;
     return dispatch<bf16_t, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx,
-                                  ldw, ldo, nt, scaled_input(x_partial, x_parts, x_size, x_eps),
-                                  stream);
+                                  ldw, ldo, nt < 0 ? -nt : nt, ex, stream);
 }
 
 // The product with the residual epilogue: residual[M, N] += X W^T (rounded to bfloat16),

@@ -612,6 +612,50 @@ def test_tile_product_keeps_to_its_sizes():
     torch.testing.assert_close(got.float().cpu(), x.float() @ w.float().T, rtol=1e-2, atol=1e-2)
 
 
+# rows, result columns, K: more (gate, up) pairs of tiles than the chip has compute units; pairs that
+# do not divide among the workgroups; a K whose chunks do not divide among the waves
+STREAM_SHAPES = [(8, 12288, 4096), (1, 11200, 1024), (16, 4112, 1152), (5, 25600, 1280), (13, 8192, 2048)]
+
+
+@pytest.mark.parametrize("shape", STREAM_SHAPES)
+@pytest.mark.parametrize("scaled", [False, True], ids=["plain", "scaled"])
+def test_gate_up_product_that_streams_several_pairs_a_workgroup(shape, scaled):
+    """The few-row gate/up product of a matrix with more pairs of tiles than compute units walks
+    several pairs in one workgroup.  Against the float32 reference, and bit for bit against the
+    kernel of one pair a workgroup (the same sums in the same order)."""
+    import ctypes
+
+    ops = _ops()
+    core = ops.core()
+    m, inter, k = shape
+    gen = torch.Generator().manual_seed(inter + k)
+    x = torch.randn((m, k), generator=gen).bfloat16()
+    w = (torch.randn((2 * inter, k), generator=gen) / math.sqrt(k)).bfloat16()
+    w[inter - 1] = 2.0 / math.sqrt(k)       # the last gate row
+    w[2 * inter - 1] = -2.0 / math.sqrt(k)  # and the last up row stand out
+    xd, wd = x.to(DEV), w.to(DEV)
+    partial = None
+    factor = torch.ones(m, 1)
+    if scaled:
+        parts = 7
+        partial = torch.rand((parts, 16), generator=gen) * k / parts
+        factor = torch.rsqrt(partial[:, :m].sum(0) / k + 1e-6).reshape(m, 1)
+        partial = partial.to(DEV)
+    def run(nt):
+        out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+        rc = core.rl_gemm_skinny_swiglu(
+            ctypes.c_void_p(xd.data_ptr()), ctypes.c_void_p(wd.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+            m, inter, k, k, k, inter, nt, ctypes.c_void_p(partial.data_ptr() if scaled else 0),
+            7 if scaled else 0, k if scaled else 0, ctypes.c_float(1e-6), ops._stream())
+        assert rc == 0
+        return out
+    streamed, single = run(2), run(-2)
+    assert torch.equal(streamed, single)
+    gu = ((x.float() @ w.float().T) * factor).bfloat16().float()
+    want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
+    torch.testing.assert_close(streamed.float().cpu(), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("shape", [(1, 96, 64), (8, 4096, 4096), (16, 304, 1000), (5, 4096, 12288), (3, 40, 48)])
 def test_products_fold_the_norm_between_them(shape):
     """producer: residual += x W^T, rows * weight, pieces of the sums of squares; consumer:
