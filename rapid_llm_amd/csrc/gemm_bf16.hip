@@ -99,7 +99,10 @@ struct SkinnyExtra {
     float* partial;       // [workgroups][16]
 };
 
-template <int NT, typename OutT, bool SWIGLU, bool SCALED>
+// LASTQ: groups of four rows of the last tile that belong to the workgroup: 4, or 2 for
+// workgroups of 24 rows (NT == 2), which put a matrix of 384 tiles on 256 compute units
+// evenly; the other rows of that tile are neither read nor stored.
+template <int NT, typename OutT, bool SWIGLU, bool SCALED, int LASTQ = 4>
 __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, OutT* __restrict__ out, int M,
     int N, int K, int ldx, int ldw, int ldo, SkinnyExtra ex) {
@@ -107,6 +110,8 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
 
     __shared__ __attribute__((aligned(16))) unsigned char wtile[GW][16 * WT_PITCH];
     __shared__ float wave_part[SCALED ? GW : 1][16];  // a scaled input's sums of squares by wave
+    static_assert(LASTQ == 4 || (LASTQ == 2 && NT == 2 && !SWIGLU), "half a last tile: two plain tiles only");
+    constexpr int ROWS = (NT - 1) * 16 + 4 * LASTQ;  // weight rows of a workgroup (not SWIGLU)
 
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -121,7 +126,7 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
         if (SWIGLU)
             tile_row[nt] = (blockIdx.x * (NT / 2) + nt / 2) * 16 + ((nt & 1) ? N : 0);
         else
-            tile_row[nt] = (blockIdx.x * NT + nt) * 16;
+            tile_row[nt] = blockIdx.x * ROWS + nt * 16;
     }
     const int row_limit = SWIGLU ? 2 * N - 1 : N - 1;
     const int seg_limit = N - 1;  // within the gate (or up) half
@@ -167,10 +172,11 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     float res_in[4] = {0.f, 0.f, 0.f, 0.f}, nw_in[4] = {0.f, 0.f, 0.f, 0.f};
     if (!SWIGLU && ex.residual && threadIdx.x < NT * 64) {
         const int ln = threadIdx.x & 63, ot = threadIdx.x >> 6, m = ln & 15;
-        const int nbase = (blockIdx.x * NT + ot) * 16 + 4 * (ln >> 4);
+        const int nbase = blockIdx.x * ROWS + ot * 16 + 4 * (ln >> 4);
+        const bool mine = ot * 16 + 4 * (ln >> 4) < ROWS;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            if (m < M && nbase + i < N) {
+            if (m < M && mine && nbase + i < N) {
                 res_in[i] = ex.residual[(size_t)m * N + nbase + i];
                 nw_in[i] = ex.norm_w[nbase + i];
             }
@@ -191,7 +197,7 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) r[nt][j] = ld16(wld[nt][j] + kw);
+                for (int j = 0; j < (nt == NT - 1 ? LASTQ : 4); ++j) r[nt][j] = ld16(wld[nt][j] + kw);
 #pragma unroll
             for (int j = 0; j < 4; ++j) xx[j] = ld16(xrow + kw + 8 * j);
         };
@@ -199,7 +205,7 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < (nt == NT - 1 ? LASTQ : 4); ++j)  // rows beyond stay what they were
                     *reinterpret_cast<bf16x8*>(mytile + (4 * j + g) * WT_PITCH + 16 * r16) = r[nt][j];
                 bf16x8 a[4];
 #pragma unroll
@@ -291,7 +297,9 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
         const int ln = e & 63;
         const int ot = e >> 6;
         const int m = ln & 15;
-        const int nbase = (blockIdx.x * OUT_TILES + ot) * 16 + 4 * (ln >> 4);
+        const int nbase = SWIGLU ? (blockIdx.x * OUT_TILES + ot) * 16 + 4 * (ln >> 4)
+                                 : blockIdx.x * ROWS + ot * 16 + 4 * (ln >> 4);
+        const bool mine = SWIGLU || ot * 16 + 4 * (ln >> 4) < ROWS;  // not in the unused part of the last tile
         float scale = 1.f;
         if constexpr (SCALED) {
             float ss = 0.f;
@@ -300,7 +308,7 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
             scale = rsqrtf(ss * ex.x_inv_size + ex.x_eps);
         }
         float sumsq = 0.f;
-        if (m < M) {
+        if (m < M && mine) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int n = nbase + i;
@@ -348,13 +356,13 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_skinny_kernel(
     }
 }
 
-template <int NT, typename OutT, bool SWIGLU, bool SCALED>
+template <int NT, typename OutT, bool SWIGLU, bool SCALED, int LASTQ = 4>
 static int launch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, int K, int ldx,
                   int ldw, int ldo, const SkinnyExtra& ex, hipStream_t stream) {
-    constexpr int rows_per_block = (SWIGLU ? NT / 2 : NT) * 16;
+    constexpr int rows_per_block = SWIGLU ? (NT / 2) * 16 : (NT - 1) * 16 + 4 * LASTQ;
     dim3 grid((N + rows_per_block - 1) / rows_per_block), block(GW * RL_WAVE);
-    hipLaunchKernelGGL((gemm_skinny_kernel<NT, OutT, SWIGLU, SCALED>), grid, block, 0, stream, X, W, out,
-                       M, N, K, ldx, ldw, ldo, ex);
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, OutT, SWIGLU, SCALED, LASTQ>), grid, block, 0, stream, X, W,
+                       out, M, N, K, ldx, ldw, ldo, ex);
     return rl_launch_status();
 }
 
@@ -568,6 +576,11 @@ static int dispatch(const bf16_t* X, const bf16_t* W, OutT* out, int M, int N, i
         RL_CASE(2)
     } else {
         RL_CASE(1) RL_CASE(2)
+        // nt == 3: workgroups of 24 rows, one tile and a half; plain results only
+        if (nt == 3 && !ex.residual)
+            return ex.x_partial
+                       ? launch<2, OutT, false, true, 2>(X, W, out, M, N, K, ldx, ldw, ldo, ex, stream)
+                       : launch<2, OutT, false, false, 2>(X, W, out, M, N, K, ldx, ldw, ldo, ex, stream);
     }
 #undef RL_CASE
     return RL_ERR_ARG;
@@ -591,7 +604,8 @@ static SkinnyExtra scaled_input(const float* x_partial, int x_parts, int x_size,
     return ex;
 }
 
-// out_type: RL_F32 or RL_BF16.  nt: weight-row tiles per workgroup (see the host wrapper).
+// out_type: RL_F32 or RL_BF16.  nt: weight-row tiles per workgroup, 1 or 2, or 3 for one and a
+// half (24 rows), see the host wrapper.
 extern "C" int rl_gemm_skinny(const void* X, const void* W, void* out, int M, int N, int K,
                               int ldx, int ldw, int ldo, int out_type, int nt,
                               const float* x_partial, int x_parts, int x_size, float x_eps,

@@ -460,14 +460,28 @@ def sample_uniform(seed: int, counter: int) -> float:
 
 
 SKINNY_MAX_ROWS = 16  # rows up to which the hand-written bandwidth-bound product is used
-def _skinny_tiles(rows: int, out_features: int) -> int:
-    """Weight-row tiles of 16 per workgroup of the skinny product: one, which leaves the most
-    workgroups, except where two were measured faster (Qwen3-8B shapes, microseconds, one tile
-    against two): from 8 rows on when one tile would leave some compute units with two
-    workgroups and some with one (6,144 outputs: 14.0 / 12.5 at 8 rows, 17.2 / 15.9 at 16, but
-    11.8 / 12.5 at 1 row); and with more than 12 rows on matrices of a thousand tiles and more
-    (151,936 outputs: 275 / 244 at 16 rows, but 216 / 233 at 8)."""
+def _skinny_tiles(rows: int, out_features: int, plain: bool = False) -> int:
+    """Weight rows per workgroup of the skinny product, as the kernel's code for them: 1 (16 rows,
+    one tile, which leaves the most workgroups), 2 (32 rows) or, for a product that only stores
+    its result (``plain``), 3 (24 rows: one tile and a half).
+
+    A compute unit streams at most so fast, so what counts is the most rows a unit gets: the
+    rounds of workgroups times their rows.  A matrix of 257 to 1,023 tiles takes 24 rows where
+    that gives the fewest (6,144 outputs = 384 tiles: 256 workgroups, one a unit; microseconds at
+    1 / 8 / 16 rows of X with 16, 32 and 24 weight rows a workgroup: 11.6 12.3 11.0 / 13.9 12.8
+    11.1 / 16.6 14.1 12.0; 5,120 outputs 11.4 11.2 9.8 / 13.1 12.1 10.3 / 16.2 13.7 11.6; but
+    7,168 outputs = 448 tiles, where 24 rows make 299 workgroups and a second round, 14.9 15.0
+    18.6 / 17.8 15.6 20.4).  Otherwise one tile, except where two were measured faster: from 8
+    rows of X on when one tile would leave some units with two workgroups and some with one; and
+    with more than 12 rows on matrices of a thousand tiles and more (151,936 outputs: 275 / 244
+    at 16 rows, but 216 / 233 at 8)."""
     blocks = -(-out_features // 16)
+    if plain and _FIRST_ROUND < blocks < 1024:
+        def most_rows(rows_per_group: int) -> int:
+            groups = -(-out_features // rows_per_group)
+            return -(-groups // _FIRST_ROUND) * rows_per_group
+        if most_rows(24) < min(most_rows(16), most_rows(32)):
+            return 3
     if rows >= 8 and 256 < blocks < 512:
         return 2
     if rows > 12 and blocks >= 1024:
@@ -506,7 +520,7 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, scaled=N
         if out_dtype not in (torch.bfloat16, torch.float32):
             raise KernelError(f"gemm_bf16 writes bfloat16 or float32, not {out_dtype}")
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-        nt = _skinny_tiles(m, n)
+        nt = _skinny_tiles(m, n, plain=True)
         _ok(
             core().rl_gemm_skinny(
                 _p(x), _p(w), _p(out), m, n, k, k, k, n, _tag(out_dtype), nt, *_scaled_args(scaled, m, k), _stream()

@@ -528,7 +528,8 @@ def test_gemm_f32_keeps_what_bfloat16_would_lose():
     assert out.item() == k + 2.0 ** -12
 
 
-@pytest.mark.parametrize("shape", [(1, 503, 96), (8, 4096, 4096), (16, 300, 1000), (64, 1000, 12288), (17, 6144, 4096), (200, 331, 80), (3, 24, 48)])
+@pytest.mark.parametrize("shape", [(1, 503, 96), (8, 4096, 4096), (16, 300, 1000), (64, 1000, 12288), (17, 6144, 4096), (200, 331, 80), (3, 24, 48),
+                                   (8, 6144, 4096), (1, 5000, 256), (16, 4618, 1160), (11, 6120, 96)])  # the last four: workgroups of 24 weight rows
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16out", "f32out"])
 def test_gemm_bf16(shape, out_dtype):
     ops = _ops()
@@ -687,11 +688,24 @@ def test_products_fold_the_norm_between_them(shape):
     scaled = ScaledRows(rows, partial, hidden, eps)
     normed = plain_rmsnorm(res.cpu(), norm_w, eps)
     n2 = 208
+    # the second width takes workgroups of 24 weight rows (a tile and a half), the last of them short
     w2 = (torch.randn(n2, hidden) / math.sqrt(hidden)).bfloat16()
     for out_dtype, tol in ((torch.bfloat16, 2e-2), (torch.float32, 1e-2)):
         got = ops.gemm_bf16(rows, w2.to(DEV), out_dtype, scaled=scaled)
         want = normed.bfloat16().float() @ w2.float().T
         torch.testing.assert_close(got.float().cpu(), want, rtol=tol, atol=tol)
+    # a width that takes workgroups of 24 weight rows (a tile and a half), the last of them short:
+    # against the kernel's own order of operations (the rows as the producer rounded them, the
+    # factor applied to the result), which leaves only the order of the float32 sums
+    wide = 4616
+    assert ops._skinny_tiles(m, wide, plain=True) == 3
+    w3 = (torch.randn(wide, hidden) / math.sqrt(hidden)).bfloat16()
+    factor = torch.rsqrt(ss / hidden + eps).reshape(m, 1)
+    want = (rows.float().cpu() @ w3.float().T) * factor
+    got = ops.gemm_bf16(rows, w3.to(DEV), torch.float32, scaled=scaled)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-4)
+    got = ops.gemm_bf16(rows, w3.to(DEV), torch.bfloat16, scaled=scaled)
+    torch.testing.assert_close(got.float().cpu(), want, rtol=1e-2, atol=1e-2)
     wgu = (torch.randn(2 * n2, hidden) / math.sqrt(hidden)).bfloat16()
     act = ops.gemm_bf16_swiglu(rows, wgu.to(DEV), scaled=scaled)
     gu = (normed.bfloat16().float() @ wgu.float().T).bfloat16().float()
