@@ -88,7 +88,8 @@ def test_a_product_with_a_bias_folds_no_norm_into_itself():
     plain = _bound(128, 128, torch.bfloat16)
     x = torch.zeros(4, 128, dtype=torch.bfloat16)
     assert plain.folds(x) and plain.folds(torch.zeros(40, 128, dtype=torch.bfloat16))
-    assert not plain.folds(torch.zeros(80, 128, dtype=torch.bfloat16))  # the library's product
+    assert plain.folds(torch.zeros(192, 128, dtype=torch.bfloat16))  # runs of K, in blocks of 64 rows
+    assert not plain.folds(torch.zeros(193, 128, dtype=torch.bfloat16))  # the library's product
     biased = Linear(128, 128)
     biased.bind(torch.zeros(128, 128, dtype=torch.bfloat16), torch.zeros(128))
     assert not biased.folds(x) and biased.skinny(x)
