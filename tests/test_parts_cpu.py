@@ -180,3 +180,17 @@ def test_the_decode_launch_is_ordered_only_beyond_what_runs_at_once():
     from rapid_llm_amd.kernels import ops
 
     assert ops._DECODE_ORDER_ABOVE == 3 * 256
+
+
+def test_weight_rows_a_workgroup_of_the_few_row_product():
+    """The host's rule: 24 rows (code 3) only for a product that just stores its result, on a
+    matrix of 257 to 1,023 tiles, where that puts the fewest rows on a compute unit."""
+    from rapid_llm_amd.kernels import ops
+
+    assert ops._skinny_tiles(8, 6144, plain=True) == 3      # 384 tiles: 256 workgroups of 24 rows
+    assert ops._skinny_tiles(1, 5120, plain=True) == 3      # 320 tiles: 214 workgroups
+    assert ops._skinny_tiles(8, 7168, plain=True) == 2      # 448 tiles: 24 rows would need a second round
+    assert ops._skinny_tiles(8, 6144) == 2                  # the residual epilogue keeps whole tiles
+    assert ops._skinny_tiles(8, 4096, plain=True) == 1      # one tile a unit already
+    assert ops._skinny_tiles(16, 151936, plain=True) == 2   # a thousand tiles and more: as measured
+    assert ops._skinny_tiles(8, 151936, plain=True) == 1
