@@ -1,14 +1,18 @@
 """Device side of the cache: the page tensors of every layer, the block tables, the state slots.
 
-Layout of one layer's pages (chosen for the attention kernels' matrix-core operands):
+What a layer's pages hold is the mixer's to say: it names its paged tensors, each with a
+per-position shape and the place of the page's positions among its axes
+(:class:`~rapid_llm_amd.parts.base.PagedSpec`), and finds them here by name.  Nothing in this
+file knows of keys, values or heads.  The attention of this package asks for
 
-* keys   ``K[page, kv_head, slot_in_page, head_dim]``: a key is one contiguous row;
-* values ``V[page, kv_head, head_dim, slot_in_page]``: stored transposed, so the positions
-  of a page are contiguous for one channel, which is how the ``P @ V`` product reads them.
+* keys   ``k[page, kv_head, slot_in_page, head_dim]``: a key is one contiguous row;
+* values ``v[page, kv_head, head_dim, slot_in_page]``: stored transposed, so the positions
+  of a page are contiguous for one channel, which is how the ``P @ V`` product reads them,
 
-One page of one group therefore costs ``2 * kv_heads * head_dim * page_size`` elements in
-each layer of the group.  (The reference keeps token-granular rows ``[tokens, 2 * kv_heads,
-head_dim]``, rapid_llm/executor/kv_cache_manager.py:230-249.)
+so one page of one group costs ``2 * kv_heads * head_dim * page_size`` elements in each of its
+layers of the group.  (The reference keeps token-granular rows ``[tokens, 2 * kv_heads,
+head_dim]``, rapid_llm/executor/kv_cache_manager.py:230-249, and a latent row per token for
+another mixer, rapid_llm/engine/kv_cache_spec.py:171-188.)
 """
 
 from __future__ import annotations
@@ -30,12 +34,24 @@ class LayerCache:
     layer: int
     group_id: int | None  # None: the mixer has no paged cache
     page_size: int
-    k: torch.Tensor | None  # [pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor | None  # [pages, kv_heads, head_dim, page_size]
+    # the mixer's paged tensors by the names it gave them, each
+    # [pages, *shape[:slot_axis], page_size, *shape[slot_axis:]]
+    pages: dict[str, torch.Tensor]
     owns_pages: bool  # False: reads another layer's pages and must not write them
     # fixed-size per-request tensors by name, each [max_seqs + 1, *shape], zeroed when a slot
     # is taken (the last row belongs to the filler slot of padded batches)
     states: dict[str, torch.Tensor]
+
+    @property
+    def k(self) -> torch.Tensor | None:
+        """The paged tensor named ``"k"`` (keys ``[pages, kv_heads, page_size, head_dim]`` of the
+        layout :meth:`CacheNeed.keys_and_values` asks for)."""
+        return self.pages.get("k")
+
+    @property
+    def v(self) -> torch.Tensor | None:
+        """The paged tensor named ``"v"`` (values ``[pages, kv_heads, head_dim, page_size]``)."""
+        return self.pages.get("v")
 
     @property
     def state(self) -> torch.Tensor | None:
@@ -51,16 +67,21 @@ def plan_groups(needs: list[CacheNeed]) -> tuple[list[GroupSpec], list[int | Non
     layers_of: dict[int, list[int]] = {}
     group_of: list[int | None] = [None] * len(needs)
     for i, need in enumerate(needs):
-        if need.kind != "kv" or need.share_with is not None:
+        if need.kind != "paged" or need.share_with is not None:
             continue
         gid = keys.setdefault(need.window, len(keys))
         layers_of.setdefault(gid, []).append(i)
         group_of[i] = gid
     for i, need in enumerate(needs):
-        if need.kind == "kv" and need.share_with is not None:
+        if need.kind == "paged" and need.share_with is not None:
             src = need.share_with
-            if not 0 <= src < len(needs) or needs[src].kind != "kv" or needs[src].share_with is not None:
+            if not 0 <= src < len(needs) or needs[src].kind != "paged" or needs[src].share_with is not None:
                 raise ValueError(f"layer {i} shares the cache of layer {src}, which owns none")
+            if needs[src].paged != need.paged:
+                raise ValueError(
+                    f"layer {i} shares the cache of layer {src} but names other paged tensors: "
+                    f"{need.paged} against {needs[src].paged}"
+                )
             if needs[src].window != need.window:
                 raise ValueError(
                     f"layer {i} (window {need.window}) shares the cache of layer {src} "
@@ -84,12 +105,15 @@ def state_bytes(needs: list[CacheNeed], slots: int, elem: int) -> int:
 
 
 def page_bytes(needs: list[CacheNeed], group_of: list[int | None], page_size: int, elem: int) -> dict[int, int]:
-    """Bytes one page id costs in each group (summed over the group's owning layers)."""
+    """Bytes one page id costs in each group: every paged tensor of every owning layer of the
+    group (``elem``: bytes of an element of the engine's compute type)."""
     out: dict[int, int] = {}
     for need, gid in zip(needs, group_of):
         if gid is None or need.share_with is not None:
             continue
-        out[gid] = out.get(gid, 0) + 2 * need.num_kv_heads * need.head_dim * page_size * elem
+        for spec in need.paged:
+            size = getattr(torch, spec.dtype).itemsize if spec.dtype else elem
+            out[gid] = out.get(gid, 0) + spec.elements() * page_size * size
     return out
 
 
@@ -108,16 +132,21 @@ class DeviceCache:
         P = manager.page_size
         self.layers: list[LayerCache] = []
         for i, need in enumerate(needs):
-            k = v = None
+            paged: dict[str, torch.Tensor] = {}
             gid = group_of[i]
             owns = False
-            if need.kind == "kv" and need.share_with is None:
+            if need.kind == "paged" and need.share_with is None:
                 pages = manager.pools[gid].num_pages
                 # zero-filled once.  Page 0, the null page, is written by rows that only pad a
-                # batch (their keys and values land in its first slot) and never read unmasked;
+                # batch (what they write lands in its first slot) and never read unmasked;
                 # nothing is ever read from a page beyond what the masks allow
-                k = torch.zeros((pages, need.num_kv_heads, P, need.head_dim), dtype=dtype, device=device)
-                v = torch.zeros((pages, need.num_kv_heads, need.head_dim, P), dtype=dtype, device=device)
+                paged = {
+                    spec.name: torch.zeros(
+                        spec.page_shape(pages, P),
+                        dtype=getattr(torch, spec.dtype) if spec.dtype else dtype, device=device,
+                    )
+                    for spec in need.paged
+                }
                 owns = True
             states = {
                 spec.name: torch.zeros(
@@ -126,11 +155,10 @@ class DeviceCache:
                 )
                 for spec in need.state_specs()
             }
-            self.layers.append(LayerCache(i, gid, P, k, v, owns, states))
+            self.layers.append(LayerCache(i, gid, P, paged, owns, states))
         for i, need in enumerate(needs):
-            if need.kind == "kv" and need.share_with is not None:
-                src = self.layers[need.share_with]
-                self.layers[i].k, self.layers[i].v = src.k, src.v
+            if need.kind == "paged" and need.share_with is not None:
+                self.layers[i].pages = self.layers[need.share_with].pages
         # One row more than there are slots: the filler slot, whose row maps every position to
         # the null page for good.  Rows that only pad a batch to a captured size name it (the
         # reference keeps its last table row for the same purpose,

@@ -253,6 +253,16 @@ def cmd_bench(args) -> int:
         "prefill_tok_s": round(statistics.median(r["prompt_tokens"] / r["ttft_s"] for r in rows), 1),
         "preemptions": sum(r["preemptions"] for r in rows),
     }))
+    if args.profile:
+        # one more run of the same workload with every step eager and a pair of events around
+        # every part: where the device's time goes, by part and by kind of step
+        from .engine.timeline import Timeline, instrument
+
+        timeline = Timeline()
+        instrument(engine.runner, timeline)
+        lengths = sample_prompt_lengths(args.batch_size, low, high, args.seed)
+        measure_offline(engine, [[rng.randrange(vocab) for _ in range(n)] for n in lengths], args.gen_len)
+        print(timeline.summary(), file=sys.stderr)
     return 0
 
 
@@ -301,6 +311,9 @@ def main(argv=None) -> int:
     bench.add_argument("--gen-len", type=int, default=128)
     bench.add_argument("--iterations", type=int, default=3)
     bench.add_argument("--warmup", type=int, default=1)
+    bench.add_argument("--profile", action="store_true",
+                       help="after the measurement, run the workload once more eagerly and print the "
+                            "device time of every part (HIP events) to stderr")
     bench.set_defaults(fn=cmd_bench)
 
     init = subs.add_parser("init", help="Write a model folder with random weights")

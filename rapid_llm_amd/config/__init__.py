@@ -1,11 +1,11 @@
 from .engine_config import EngineConfig
 from .model_config import (
     ConfigError,
-    Qwen3Config,
     normalise_dtype_name,
     read_architecture,
     read_config_json,
 )
+from .qwen3 import Qwen3Config
 from .registry import (
     ArchitectureEntry,
     config_from_dict,

@@ -23,6 +23,10 @@ class ArchitectureEntry:
     config_cls: Any  # has from_dict(data, overrides) and to_dict()
     build_spec: Callable[[Any], Any]  # config -> ModelSpec
     aliases: tuple[str, ...] = ()
+    # a checkpoint of this architecture whose folder name says neither "base" nor "instruct"
+    # is a chat model and gets its folder's chat template (the reference keeps a list of such
+    # model types beside its prompt code, rapid_llm/utils/prompt_templates.py:106-107)
+    chat_by_default: bool = False
 
 
 _ENTRIES: dict[str, ArchitectureEntry] = {}
@@ -41,10 +45,11 @@ def register_architecture(
     aliases: tuple[str, ...] = (),
     *,
     replace: bool = False,
+    chat_by_default: bool = False,
 ) -> ArchitectureEntry:
     if name in _ENTRIES and not replace:
         raise ValueError(f"architecture {name!r} is already registered")
-    entry = ArchitectureEntry(name, config_cls, build_spec, tuple(aliases))
+    entry = ArchitectureEntry(name, config_cls, build_spec, tuple(aliases), bool(chat_by_default))
     _ENTRIES[name] = entry
     for alias in aliases:
         _ALIASES[alias.lower()] = name
@@ -75,6 +80,15 @@ def resolve_architecture(name: str) -> ArchitectureEntry:
     raise ConfigError(
         f"unsupported architecture {name!r}; supported: {', '.join(supported_architectures())}"
     )
+
+
+def chat_by_default(config_body: Mapping[str, Any]) -> bool:
+    """Whether the architecture a ``config.json`` body names registers its releases as chat
+    models; ``False`` for a body that names none or one that is not registered."""
+    try:
+        return resolve_architecture(read_architecture(config_body)).chat_by_default
+    except ConfigError:
+        return False
 
 
 def config_from_dict(data: Mapping[str, Any], overrides: Mapping[str, Any] | None = None):

@@ -437,14 +437,19 @@ extern "C" int rl_rope_table(const float* inv_freq, float* cos_out, float* sin_o
 }
 
 // --------------------------------------------------------------------------- //
-// Fused per-head RMSNorm (optional) + half-split rotation (optional) of q and k, and the
-// write of k and v into the paged cache.  One wave per (token, head); a workgroup of four
-// waves takes four heads of a token.
+// Fused per-head RMSNorm (optional) + rotation (optional) of q and k, and the write of k and v
+// into the paged cache.  One wave per (token, head); a workgroup of four waves takes four
+// heads of a token.
 //
 // qkv row layout: [q heads | k heads | v heads], heads adjacent (rapid_llm/modules/linear.py:
 // 236-251).  Norm over head_dim before the rotation (rapid_llm/models/base.py:134-140).
-// Rotation: o1 = x1*c - x2*s, o2 = x2*c + x1*s on the halves
-// (rapid_llm/kernels/ops/rope/rope_emb.py:47-82).
+// Rotation of a pair (x1, x2) by the position's angle of that pair: o1 = x1*c - x2*s,
+// o2 = x2*c + x1*s (rapid_llm/kernels/ops/rope/rope_emb.py:47-82).  Which channels pair, and
+// how many of a head's channels rotate, is the position encoding's to say: the first
+// 2 * rotary_half channels rotate, pair p of them being channels (p, p + rotary_half) with the
+// half-split pairing (the reference's) and (2p, 2p + 1) with the interleaved one; the channels
+// beyond pass with the norm alone.  This kernel takes every such case; the vectorised ones
+// below take the half-split rotation of the whole head.
 //
 // Cache layout of one layer, page p, kv head h:
 //   keys   K[p][h][slot_in_page][d]      (row-major, d contiguous)
@@ -459,8 +464,8 @@ __global__ void qknorm_rope_kvwrite_kernel(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int d, int rotary_half, float eps, int write_cache,
-    int write_values) {
+    int page_size, int nq, int nkv, int d, int rotary_half, int interleaved, float eps,
+    int write_cache, int write_values) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -490,17 +495,23 @@ __global__ void qknorm_rope_kvwrite_kernel(
         const bool is_q = head < nq;
         if (!is_q && !write_cache) continue;
         const float* w = is_q ? q_norm_w : k_norm_w;
-        // lane handles element pairs (i, i + half) for i = lane, lane + 64 (half <= 128)
+        // lane handles the pairs p = lane, lane + 64 (half <= 128) of channels (e1, e2): the
+        // pairs that rotate first, as the pairing says, then the channels beyond two by two
+        const int rot = cos_tab ? rotary_half : 0;
+        int e1[2], e2[2];
         float x1[2], x2[2];
         float ss = 0.f;
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-            const int i = lane + r * RL_WAVE;
+            const int p = lane + r * RL_WAVE;
+            const bool split = p < rot && !interleaved;
+            e1[r] = split ? p : 2 * p;
+            e2[r] = split ? p + rot : 2 * p + 1;
             x1[r] = 0.f;
             x2[r] = 0.f;
-            if (i < half) {
-                x1[r] = to_float(x[i]);
-                x2[r] = to_float(x[i + half]);
+            if (p < half) {
+                x1[r] = to_float(x[e1[r]]);
+                x2[r] = to_float(x[e2[r]]);
                 ss += x1[r] * x1[r] + x2[r] * x2[r];
             }
         }
@@ -516,23 +527,23 @@ __global__ void qknorm_rope_kvwrite_kernel(
             dst = k_cache + ((page * nkv + (head - nq)) * page_size + off) * d;
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-            const int i = lane + r * RL_WAVE;
-            if (i < half) {
+            const int p = lane + r * RL_WAVE;
+            if (p < half) {
                 float a = x1[r], b = x2[r];
                 if (w) {
-                    a = a * rrms * w[i];
-                    b = b * rrms * w[i + half];
+                    a = a * rrms * w[e1[r]];
+                    b = b * rrms * w[e2[r]];
                 }
-                if (cos_tab && i < rotary_half) {
-                    const float c = cos_tab[(size_t)pos * rotary_half + i];
-                    const float s = sin_tab[(size_t)pos * rotary_half + i];
+                if (p < rot) {
+                    const float c = cos_tab[(size_t)pos * rotary_half + p];
+                    const float s = sin_tab[(size_t)pos * rotary_half + p];
                     const float ra = a * c - b * s;
                     const float rb = b * c + a * s;
                     a = ra;
                     b = rb;
                 }
-                dst[i] = from_float<T>(a);
-                dst[i + half] = from_float<T>(b);
+                dst[e1[r]] = from_float<T>(a);
+                dst[e2[r]] = from_float<T>(b);
             }
         }
     }
@@ -644,10 +655,11 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
                           const float* k_norm_w, const float* cos_tab, const float* sin_tab,
                           const int* positions, const int* token_slot, const int* block_table,
                           int table_stride, int page_size, int tokens, int nq, int nkv, int d,
-                          int rotary_half, float eps, int write_cache, int write_values,
-                          hipStream_t stream) {
+                          int rotary_half, int interleaved, float eps, int write_cache,
+                          int write_values, hipStream_t stream) {
     const int total_heads = nq + (write_values ? 2 * nkv : nkv);
-    if (d % 8 == 0) {
+    // the vectorised kernel: head sizes in steps of 8, the half-split rotation of the whole head
+    if (d % 8 == 0 && (!cos_tab || (rotary_half == d / 2 && !interleaved))) {
         const int lph = d <= 128 ? 16 : 32;
         const int heads_per_block = 4 * (RL_WAVE / lph);
         const int groups = (total_heads + heads_per_block - 1) / heads_per_block;
@@ -668,7 +680,7 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
     dim3 grid(tokens, head_groups > 65535 ? 65535 : head_groups), block(256);
     hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, grid, block, 0, stream, qkv, q_out, k_cache,
                        v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
-                       block_table, table_stride, page_size, nq, nkv, d, rotary_half, eps,
+                       block_table, table_stride, page_size, nq, nkv, d, rotary_half, interleaved, eps,
                        write_cache, write_values);
 }
 
@@ -795,24 +807,25 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
                                       const int* positions, const int* token_slot,
                                       const int* block_table, int table_stride, int page_size,
                                       int tokens, int nq, int nkv, int d, int rotary_half,
-                                      float eps, int write_cache, int act_type,
+                                      int interleaved, float eps, int write_cache, int act_type,
                                       hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (d % 2 || d > 256) return RL_ERR_ARG;
-    // only a rotation over the whole head is implemented (pairs i, i + d/2)
-    if (cos_tab && rotary_half != d / 2) return RL_ERR_ARG;
+    // the first 2 * rotary_half channels of a head rotate: at least one pair, at most all
+    if (cos_tab && (rotary_half < 1 || rotary_half > d / 2)) return RL_ERR_ARG;
+    const bool whole_split = !cos_tab || (rotary_half == d / 2 && !interleaved);
     // with enough tokens the values go through the tile kernel, and the per-head kernel
     // covers the query and key heads only
     const int tile_values = write_cache && tokens >= 8 && nkv <= 65535;
     if ((long)nq + 2 * nkv > 65535 * 4) return RL_ERR_ARG;
     dim3 block(256);
     dim3 vgrid((tokens + VT_TOKENS - 1) / VT_TOKENS, nkv);
-    if (tile_values && act_type == RL_F32 &&
+    if (tile_values && whole_split && act_type == RL_F32 &&
         launch_qkv_prepare<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, q_norm_w,
                                   k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
                                   table_stride, page_size, tokens, nq, nkv, d, eps, stream))
         return rl_launch_status();
-    if (tile_values && act_type == RL_BF16 &&
+    if (tile_values && whole_split && act_type == RL_BF16 &&
         launch_qkv_prepare<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                    q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
                                    table_stride, page_size, tokens, nq, nkv, d, eps, stream))
@@ -821,7 +834,7 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
         launch_qknorm<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
                              q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                              block_table, table_stride, page_size, tokens, nq, nkv, d, rotary_half,
-                             eps, write_cache, !tile_values, stream);
+                             interleaved, eps, write_cache, !tile_values, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, block, 0, stream,
                                (const float*)qkv, (float*)v_cache, positions, token_slot,
@@ -830,7 +843,7 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
         launch_qknorm<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
                               (bf16_t*)v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions,
                               token_slot, block_table, table_stride, page_size, tokens, nq, nkv, d,
-                              rotary_half, eps, write_cache, !tile_values, stream);
+                              rotary_half, interleaved, eps, write_cache, !tile_values, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, block, 0, stream,
                                (const bf16_t*)qkv, (bf16_t*)v_cache, positions, token_slot,

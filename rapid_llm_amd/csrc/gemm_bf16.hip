@@ -530,23 +530,10 @@ __global__ __launch_bounds__(GW* RL_WAVE) void gemm_swiglu_stream_kernel(
     }
 }
 
-// the chip's compute units (one workgroup of the stream kernel each)
-static int compute_units() {
-    static int units[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-    if (units[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-        units[dev] = n;
-    }
-    return units[dev];
-}
-
-// true (and *rc set) if the stream kernel took the product
+// true (and *rc set) if the stream kernel took the product; `units`: the chip's compute units
+// as the host read them (one workgroup of the stream kernel each)
 static bool swiglu_stream(const bf16_t* X, const bf16_t* W, bf16_t* out, int M, int I, int K, int ldx,
-                          int ldw, int ldo, const SkinnyExtra& ex, hipStream_t stream, int* rc) {
-    const int units = compute_units();
+                          int ldw, int ldo, int units, const SkinnyExtra& ex, hipStream_t stream, int* rc) {
     const int pairs = I / 16;
     if (units <= 0 || I % 16 || K % KSTEP || K < GW * KSTEP || pairs <= units) return false;
     const int per = (pairs + units - 1) / units;  // pairs a workgroup
@@ -624,18 +611,19 @@ extern "C" int rl_gemm_skinny(const void* X, const void* W, void* out, int M, in
 }
 
 // out[M, I] = silu(X Wg^T) * (X Wu^T) with W = [Wg | Wu] stacked by rows, [2I, K].  A matrix
-// with more pairs of tiles than compute units goes to the stream kernel (nt < 0: never, the
-// kernel of one pair a workgroup with -nt tiles: for comparing the two).
+// with more pairs of tiles than the chip has compute units (`units`, as the host's launch rules
+// read them) goes to the stream kernel (nt < 0: never, the kernel of one pair a workgroup with
+// -nt tiles: for comparing the two).
 extern "C" int rl_gemm_skinny_swiglu(const void* X, const void* W, void* out, int M, int I, int K,
-                                     int ldx, int ldw, int ldo, int nt, const float* x_partial,
+                                     int ldx, int ldw, int ldo, int nt, int units, const float* x_partial,
                                      int x_parts, int x_size, float x_eps, hipStream_t stream) {
     if (M <= 0 || I <= 0) return RL_OK;
     if (!skinny_args_ok(M, K, ldx, ldw) || ldo < I || (x_partial && (x_parts < 1 || x_size < 1)))
         return RL_ERR_ARG;
     const SkinnyExtra ex = scaled_input(x_partial, x_parts, x_size, x_eps);
     int rc = RL_OK;
-    if (nt >= 0 && swiglu_stream((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx, ldw, ldo, ex,
-                                 stream, &rc))
+    if (nt >= 0 && swiglu_stream((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx, ldw, ldo, units,
+                                 ex, stream, &rc))
         return rc;
     return dispatch<bf16_t, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)out, M, I, K, ldx,
                                   ldw, ldo, nt < 0 ? -nt : nt, ex, stream);

@@ -6,8 +6,9 @@ templates expect (``messages``, ``add_generation_prompt``, ``bos_token``, ``eos_
 the reference renders it through its tokenizer (rapid_llm/utils/prompt_templates.py:19-57).
 A folder without a template, or one that looks like a base checkpoint, gets its prompts
 verbatim (:76-150): a name containing ``base`` is a base checkpoint; ``instruct``, ``chat`` or
-``-it`` an instruction-tuned one; otherwise the ``model_type`` decides, ``qwen3`` releases
-being chat models unless named otherwise.
+``-it`` an instruction-tuned one; otherwise the architecture decides, through the flag its
+registry entry carries (``register_architecture(..., chat_by_default=True)``): no
+architecture is named here.
 """
 
 from __future__ import annotations
@@ -17,7 +18,6 @@ from pathlib import Path
 from typing import Any
 
 _INSTRUCT_HINTS = ("instruct", "chat", "-it")
-_CHAT_BY_DEFAULT_TYPES = ("qwen3",)
 
 
 def _special_token(entry: Any) -> str | None:
@@ -60,24 +60,42 @@ def is_instruct(model_dir: str | Path) -> bool:
         return False
     if any(h in name for h in _INSTRUCT_HINTS):
         return True
+    from ..config.registry import chat_by_default
+
     try:
-        model_type = json.loads((Path(model_dir) / "config.json").read_text()).get("model_type", "")
+        body = json.loads((Path(model_dir) / "config.json").read_text())
     except (OSError, json.JSONDecodeError):
-        model_type = ""
-    return model_type in _CHAT_BY_DEFAULT_TYPES
+        return False
+    return isinstance(body, dict) and chat_by_default(body)
 
 
 class ChatPrompter:
     """Formats conversations with one template."""
 
     def __init__(self, template: str, bos_token: str | None = None, eos_token: str | None = None) -> None:
+        from datetime import datetime
+
         from jinja2.sandbox import ImmutableSandboxedEnvironment
 
         def raise_exception(message):
             raise ValueError(f"the chat template refused the conversation: {message}")
 
-        env = ImmutableSandboxedEnvironment(trim_blocks=True, lstrip_blocks=True)
+        def tojson(value, ensure_ascii=False, indent=None, separators=None, sort_keys=False):
+            # the dialect's own filter: plain JSON text (jinja2's escapes <, >, & and quotes
+            # for HTML, which would change the prompt's tokens)
+            return json.dumps(value, ensure_ascii=ensure_ascii, indent=indent, separators=separators,
+                              sort_keys=sort_keys)
+
+        # what the templates of model folders may use beyond plain jinja2, as the tokenizer-side
+        # rendering that the reference delegates to provides it
+        # (rapid_llm/utils/prompt_templates.py:19-57): break / continue in loops, a tojson that
+        # writes plain JSON, strftime_now and raise_exception
+        env = ImmutableSandboxedEnvironment(
+            trim_blocks=True, lstrip_blocks=True, extensions=["jinja2.ext.loopcontrols"]
+        )
+        env.filters["tojson"] = tojson
         env.globals["raise_exception"] = raise_exception
+        env.globals["strftime_now"] = lambda fmt: datetime.now().strftime(fmt)
         self._template = env.from_string(template)
         self.bos_token = bos_token or ""
         self.eos_token = eos_token or ""

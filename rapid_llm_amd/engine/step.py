@@ -194,22 +194,34 @@ class ModelRunner:
         return int(min(pages, cap))
 
     def _graph_pool_estimate(self) -> int:
-        """Bytes the recorded decode steps may come to hold: every batch size of the ladder up
-        to ``max_num_seqs``, in every context bucket, keeps its float32 logits and a few rows of
-        activations."""
+        """Bytes the recorded decode steps may come to hold.  A batch is padded up to the next
+        size of the ladder, so every size up to and including the first that holds
+        ``max_num_seqs`` may be recorded, in every context bucket; each recording keeps its
+        float32 logits, a few rows of activations and what its parts say they keep between
+        their kernels (``Part.recorded_step_bytes``; a recording's pool reuses what one layer
+        frees for the next, so the largest part counts, twice over)."""
         e = self.engine
         if not (e.use_graph and self.model.replayable()):
             return 0
-        rows = sum(b for b in GRAPH_BATCHES if b <= max(1, e.max_num_seqs)) or 1
-        buckets, bound = 1, 512
-        while bound < e.max_seq_len:
+        most = max(1, min(e.max_num_seqs, GRAPH_BATCHES[-1]))
+        sizes = [b for b in GRAPH_BATCHES if b < most] + [next(b for b in GRAPH_BATCHES if b >= most)]
+        bounds, bound = [], 512
+        while True:
+            bounds.append(min(bound, e.max_seq_len))
+            if bound >= e.max_seq_len:
+                break
             bound *= 2
-            buckets += 1
         widest = max(
             [self.spec.hidden_size]
             + [p.shape[0] for p in self.params.values() if p.dim() == 2 and p.shape[0] != self.spec.vocab_size]
         )
-        return rows * buckets * 4 * (self.spec.vocab_size + 8 * widest)
+        parts = list(self.model.all_parts())
+        total = 0
+        for rows in sizes:
+            for bound in bounds:
+                kept = max((p.recorded_step_bytes(rows, bound, e.page_size) for p in parts), default=0)
+                total += rows * 4 * (self.spec.vocab_size + 8 * widest) + 2 * kept
+        return total
 
     # ------------------------------------------------------------------ requests
     def tokens_cached(self, request_id: str) -> int:

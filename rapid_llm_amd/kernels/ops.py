@@ -26,6 +26,35 @@ class KernelError(RuntimeError):
     pass
 
 
+class Chip:
+    """What the launch rules know about the device: its number of compute units, read once on
+    the host (the kernels that decide by it are handed the same number), and what follows
+    from it.  Without a device the rules are asked about the chip they were measured on."""
+
+    def __init__(self, units: int) -> None:
+        if units < 1:
+            raise KernelError(f"a chip has at least one compute unit, got {units}")
+        self.units = units
+        self.first_round = units  # workgroups that start first, one on each compute unit
+        self.decode_resident = 3 * units  # decode-attention workgroups the chip holds at a time
+        self.prefill_slots = 2 * units  # wave groups of four the prefill kernel keeps at a time
+
+
+MEASURED_CHIP = Chip(256)  # MI355X
+_chips: dict[int, Chip] = {}
+
+
+def chip() -> Chip:
+    """The current device's geometry (the measured chip's where no device is visible)."""
+    if not torch.cuda.is_available():
+        return MEASURED_CHIP
+    dev = torch.cuda.current_device()
+    found = _chips.get(dev)
+    if found is None:
+        found = _chips[dev] = Chip(torch.cuda.get_device_properties(dev).multi_processor_count)
+    return found
+
+
 def require_gpu() -> None:
     if not torch.cuda.is_available():
         raise KernelError(
@@ -191,6 +220,11 @@ def rope_table(inv_freq: torch.Tensor, positions: int) -> tuple[torch.Tensor, to
     return cos, sin
 
 
+# which channels of a head form a rotated pair, as the kernels number them: channel i with
+# i + (rotated channels) / 2, or channel 2i with 2i + 1
+ROTARY_PAIRINGS = {"half_split": 0, "interleaved": 1}
+
+
 def qknorm_rope_kvwrite(
     qkv: torch.Tensor,
     q_out: torch.Tensor,
@@ -209,10 +243,15 @@ def qknorm_rope_kvwrite(
     d: int,
     eps: float,
     max_position: int,
+    pairing: str = "half_split",
 ) -> None:
     """Norm + rotate q and k, write k and v to the cache pages (skipped when the caches
     are ``None``: a layer that reads another layer's cache).  ``max_position`` is the
-    largest position in the batch, checked against the rotation table and block table."""
+    largest position in the batch, checked against the rotation table and block table.
+    The tables' width says how many channels rotate (``2 * cos.shape[1]``, the first of a
+    head), ``pairing`` which of them form a pair (:data:`ROTARY_PAIRINGS`)."""
+    if pairing not in ROTARY_PAIRINGS:
+        raise KernelError(f"rotation pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
     tokens = qkv.shape[0]
     _need(qkv, "qkv", None, (tokens, (nq + 2 * nkv) * d))
     _need(q_out, "q_out", qkv.dtype, (tokens, nq * d))
@@ -237,6 +276,8 @@ def qknorm_rope_kvwrite(
         half = cos.shape[1]
         _need(cos, "cos table", torch.float32, (None, half))
         _need(sin, "sin table", torch.float32, tuple(cos.shape))
+        if not 1 <= half <= d // 2:
+            raise KernelError(f"rotation tables of {half} pairs do not fit a head of {d} channels")
         if max_position >= cos.shape[0]:
             raise KernelError(
                 f"position {max_position} is beyond the rotation table of {cos.shape[0]} positions"
@@ -245,8 +286,8 @@ def qknorm_rope_kvwrite(
         core().rl_qknorm_rope_kvwrite(
             _p(qkv), _p(q_out), _p(k_cache), _p(v_cache), _p(q_norm_w), _p(k_norm_w), _p(cos),
             _p(sin), _p(positions), _p(token_slot), _p(block_table), block_table.stride(0),
-            page_size, tokens, nq, nkv, d, half, ctypes.c_float(eps), int(write), _tag(qkv.dtype),
-            _stream(),
+            page_size, tokens, nq, nkv, d, half, ROTARY_PAIRINGS[pairing], ctypes.c_float(eps), int(write),
+            _tag(qkv.dtype), _stream(),
         ),
         "rl_qknorm_rope_kvwrite",
     )
@@ -460,7 +501,7 @@ def sample_uniform(seed: int, counter: int) -> float:
 
 
 SKINNY_MAX_ROWS = 16  # rows up to which the hand-written bandwidth-bound product is used
-def _skinny_tiles(rows: int, out_features: int, plain: bool = False) -> int:
+def _skinny_tiles(rows: int, out_features: int, plain: bool = False, units: int | None = None) -> int:
     """Weight rows per workgroup of the skinny product, as the kernel's code for them: 1 (16 rows,
     one tile, which leaves the most workgroups), 2 (32 rows) or, for a product that only stores
     its result (``plain``), 3 (24 rows: one tile and a half).
@@ -475,16 +516,17 @@ def _skinny_tiles(rows: int, out_features: int, plain: bool = False) -> int:
     rows of X on when one tile would leave some units with two workgroups and some with one; and
     with more than 12 rows on matrices of a thousand tiles and more (151,936 outputs: 275 / 244
     at 16 rows, but 216 / 233 at 8)."""
+    units = chip().units if units is None else units
     blocks = -(-out_features // 16)
-    if plain and _FIRST_ROUND < blocks < 1024:
+    if plain and units < blocks < 4 * units:
         def most_rows(rows_per_group: int) -> int:
             groups = -(-out_features // rows_per_group)
-            return -(-groups // _FIRST_ROUND) * rows_per_group
+            return -(-groups // units) * rows_per_group
         if most_rows(24) < min(most_rows(16), most_rows(32)):
             return 3
-    if rows >= 8 and 256 < blocks < 512:
+    if rows >= 8 and units < blocks < 2 * units:
         return 2
-    if rows > 12 and blocks >= 1024:
+    if rows > 12 and blocks >= 4 * units:
         return 2
     return 1
 
@@ -609,18 +651,18 @@ def _tile_applies(m: int, weight_rows: int, k: int, cols: int) -> bool:
 # within a microsecond either way from 144 rows on.
 MID_MAX_ROWS = 192
 _MID_BLOCK_ROWS = 64  # weight rows per workgroup of the mid-size product
-_MID_TARGET_BLOCKS = 256  # workgroups to reach by cutting K
 _MID_MAX_BLOCKS = 128  # wider matrices than this many workgroups stay with the library
 
 
-def mid_runs(n: int, k: int) -> int:
+def mid_runs(n: int, k: int, units: int | None = None) -> int:
     """Runs of K for the mid-size product of an ``[n, k]`` matrix, 0 where it does not apply:
     enough to put a workgroup on every compute unit, at least four chunks of 128 each."""
+    units = chip().units if units is None else units
     blocks = -(-n // _MID_BLOCK_ROWS)
     if k % 128 or n % 4 or blocks > _MID_MAX_BLOCKS:
         return 0
     chunks = k // 128
-    ks = max(1, min(_MID_TARGET_BLOCKS // blocks, chunks // 4, 8))
+    ks = max(1, min(units // blocks, chunks // 4, 8))
     while ks > 1 and -(-chunks // ks) * (ks - 1) >= chunks:  # every run holds a chunk
         ks -= 1
     return ks
@@ -682,7 +724,8 @@ def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> t
     nt = 2  # one (gate, up) pair of tiles per workgroup
     _ok(
         core().rl_gemm_skinny_swiglu(
-            _p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, *_scaled_args(scaled, m, k), _stream()
+            _p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, nt, chip().units,
+            *_scaled_args(scaled, m, k), _stream()
         ),
         "rl_gemm_skinny_swiglu",
     )
@@ -764,30 +807,27 @@ class AttentionPlan:
         if order is None:
             items = sorted(range(self.num_tiles * nkv), key=lambda i: (-self.tile_keys[i // nkv], i))
             if resident == 2:
-                first = items[:_FIRST_ROUND]
-                rest = items[_FIRST_ROUND:]
-                second = rest[::-1][:_FIRST_ROUND]
-                middle = rest[: max(0, len(rest) - _FIRST_ROUND)]
+                round_one = chip().first_round
+                first = items[:round_one]
+                rest = items[round_one:]
+                second = rest[::-1][:round_one]
+                middle = rest[: max(0, len(rest) - round_one)]
                 items = first + second + middle
             order = upload_ints(items, device)
             self.orders[(nkv, resident)] = order
         return order
 
 
-# Workgroups a decode launch should reach before it stops splitting the keys, and the fewest
-# keys a split is worth (measured at 2,048 keys, 8 kv heads: 1 request 128 keys a split,
-# 8 requests 512, 64 requests no split; at 512 keys 128 a split for 1 and 8 requests; finer
-# splits only add merge work).
-_TARGET_BLOCKS = 256
-_FIRST_ROUND = 256  # workgroups that start first, one on each compute unit
-# decode workgroups the chip holds at a time (three on each compute unit): a launch of more
-# hands them out longest request first
-_DECODE_ORDER_ABOVE = 768
+# A decode launch splits the keys until it has a workgroup for every compute unit; the fewest
+# keys a split is worth (measured at 2,048 keys, 8 kv heads on 256 units: 1 request 128 keys a
+# split, 8 requests 512, 64 requests no split; at 512 keys 128 a split for 1 and 8 requests;
+# finer splits only add merge work).  A launch of more workgroups than the chip holds at a
+# time (``Chip.decode_resident``) hands them out longest request first.
 _MIN_SPLIT_KEYS = 128
 _MAX_SPLIT_PAGES = 1024  # page ids of one split are staged in LDS
-# The prefill kernel cuts its tiles' keys into runs when a launch has fewer workgroups than
-# this and tiles of at least twice that many keys (a portion of one long prompt).
-_PREFILL_SPLIT_BELOW = 512
+# The prefill kernel cuts its tiles' keys into runs when a launch has fewer workgroups than the
+# chip has slots for (``Chip.prefill_slots``) and tiles of at least twice this many keys (a
+# portion of one long prompt).
 _PREFILL_SPLIT_KEYS = 512
 _PREFILL_MAX_SPLITS = 8
 
@@ -797,7 +837,6 @@ def tile_rows_of(lib) -> int:
 
 
 _PREFILL_STEP_KEYS = 64  # keys per step of the prefill kernel
-_PREFILL_SLOTS = 512  # wave groups of four the chip holds at a time (two on each compute unit)
 # what a step costs more when the two wave groups of a compute unit walk one tile in lockstep
 # than when they belong to two tiles and drift apart (measured: 3.17 against 2.83 us)
 _PREFILL_PAIRED_COST = 1.12
@@ -811,7 +850,8 @@ _PREFILL_ALONE = 0.8
 _PREFILL_MERGE_STEPS = 5
 
 
-def _prefill_shape(plan: "AttentionPlan", nkv: int, window: int, tile_rows: int) -> tuple[int, int]:
+def _prefill_shape(plan: "AttentionPlan", nkv: int, window: int, tile_rows: int,
+                   units: int | None = None) -> tuple[int, int]:
     """(wave groups per workgroup, runs the keys of every tile are cut into) for a launch of
     the prefill kernel, from an estimate of the launch's length in steps: the longest tile's
     steps (halved where two wave groups share it, divided where its keys are cut into runs) or
@@ -819,19 +859,20 @@ def _prefill_shape(plan: "AttentionPlan", nkv: int, window: int, tile_rows: int)
     portion of one long prompt) come out with their keys cut into runs, folded by the merge
     kernel; a prompt from its start, whose last rows alone see many keys, with two wave groups
     a tile; a launch with work for every slot with neither."""
+    slots = (chip() if units is None else Chip(units)).prefill_slots
     keys = plan.tile_keys
     if window > 0:
         keys = [min(k, window + tile_rows) for k in keys]
     items = plan.num_tiles * nkv
     steps = [-(-k // _PREFILL_STEP_KEYS) for k in keys]
     longest = max(steps)
-    share = nkv * sum(steps) / _PREFILL_SLOTS  # steps per slot if the work were spread evenly
+    share = nkv * sum(steps) / slots  # steps per slot if the work were spread evenly
     best = (max(longest * _PREFILL_ALONE, share), 1, 1)
     paired = max(-(-longest // 2), share) * _PREFILL_PAIRED_COST
     if paired < best[0]:
         best = (paired, 2, 1)
-    if items < _PREFILL_SPLIT_BELOW:
-        most = min(_PREFILL_MAX_SPLITS, -(-_PREFILL_SPLIT_BELOW // items), max(keys) // _PREFILL_SPLIT_KEYS)
+    if items < slots:
+        most = min(_PREFILL_MAX_SPLITS, -(-slots // items), max(keys) // _PREFILL_SPLIT_KEYS)
         for nsplit in range(2, most + 1):
             cost = max(-(-longest // nsplit), share) + _PREFILL_MERGE_STEPS
             if cost < best[0]:
@@ -995,21 +1036,13 @@ def _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_s
     """Split-key decode attention of the step's single tokens.  ``fused`` is ``None`` (``q``
     holds finished queries) or ``(q_norm_w, k_norm_w, cos, sin, k_write, v_write, eps)`` with
     ``q`` the packed [q | k | v] rows."""
-    group = nq // nkv
     # under a graph the split is laid out for the longest context of the graph's bucket
     span = _static(ctx).get("context_bound", plan.max_decode_ctx)
-    if window > 0:
-        span = min(span, window + 31)
-    chunks = (group + 15) // 16
-    pairs = plan.num_decode * nkv * chunks
-    want = max(1, _TARGET_BLOCKS // pairs)
-    chunk = max(_MIN_SPLIT_KEYS, -(-(-(-span // want)) // 128) * 128)
-    chunk = min(chunk, max(32, ((_MAX_SPLIT_PAGES - 1) * page_size - 31) // 32 * 32))
-    nsplit = -(-span // chunk)
+    pairs, chunk, nsplit = _decode_split(plan.num_decode, nq, nkv, span, page_size, window)
     if plan.num_decode > 65535:
         raise KernelError(f"{plan.num_decode} single-token requests exceed the decode kernel's launch grid")
     # with more workgroups than start at once, the longest requests go first
-    order = plan.decode_order(ctx) if pairs * nsplit > _DECODE_ORDER_ABOVE else None
+    order = plan.decode_order(ctx) if pairs * nsplit > chip().decode_resident else None
     part_o = part_ml = None
     if nsplit > 1:
         part_o = torch.empty((plan.num_decode, nq, nsplit, d), dtype=torch.float32, device=q.device)
@@ -1030,10 +1063,37 @@ def _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_s
     )
 
 
-def decode_attention_fusable(ctx, x_dtype: torch.dtype, group: int, d: int, rotary_half: int) -> bool:
+def _decode_split(num_decode: int, nq: int, nkv: int, span: int, page_size: int, window: int,
+                  units: int | None = None) -> tuple[int, int, int]:
+    """(workgroups before splitting, keys a split, splits) of a decode launch of ``num_decode``
+    single tokens over at most ``span`` keys: splits of a multiple of 128 keys, as many as put a
+    workgroup on every compute unit, each within what the kernel stages of page ids."""
+    units = chip().units if units is None else units
+    if window > 0:
+        span = min(span, window + 31)
+    chunks = (nq // nkv + 15) // 16
+    pairs = num_decode * nkv * chunks
+    want = max(1, units // pairs)
+    chunk = max(_MIN_SPLIT_KEYS, -(-(-(-span // want)) // 128) * 128)
+    chunk = min(chunk, max(32, ((_MAX_SPLIT_PAGES - 1) * page_size - 31) // 32 * 32))
+    return pairs, chunk, -(-span // chunk)
+
+
+def decode_scratch_bytes(rows: int, nq: int, nkv: int, d: int, span: int, page_size: int, window: int) -> int:
+    """Bytes of split results (float32 outputs, maxima and sums) that a decode launch of
+    ``rows`` single tokens over at most ``span`` keys keeps between its two kernels."""
+    _, _, nsplit = _decode_split(rows, nq, nkv, span, page_size, window)
+    return 0 if nsplit == 1 else rows * nq * nsplit * (d + 2) * 4
+
+
+def decode_attention_fusable(ctx, x_dtype: torch.dtype, group: int, d: int, rotary_half: int,
+                             pairing: str = "half_split") -> bool:
     """Whether the step is one the fused decode kernel takes: bfloat16, single tokens only,
-    a head size whose rotation pairs stay within a lane, rotation over the whole head or none."""
+    a head size whose rotation pairs stay within a lane, the half-split rotation of the whole
+    head or none."""
     if x_dtype != torch.bfloat16 or d % 64 or rotary_half not in (0, d // 2):
+        return False
+    if rotary_half and pairing != "half_split":
         return False
     plan = attention_plan(ctx, group, d)
     return plan.num_tiles == 0 and plan.num_decode > 0

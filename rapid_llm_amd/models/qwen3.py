@@ -8,7 +8,7 @@ reference translates from (rapid_llm/models/weights.py:61-134, base.py:396-404,:
 
 from __future__ import annotations
 
-from ..config.model_config import Qwen3Config
+from ..config.qwen3 import Qwen3Config
 from ..config.registry import register_architecture
 from .spec import IgnoreRule, LayerSpec, ModelSpec, PartSpec, linear_output, token_embedding
 
@@ -84,6 +84,8 @@ def build_qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
     )
 
 
+# Qwen3 releases that are not named "...-Base" are chat models
+# (rapid_llm/utils/prompt_templates.py:96-107)
 register_architecture(
-    "Qwen3ForCausalLM", Qwen3Config, build_qwen3_spec, aliases=("qwen3",), replace=True
+    "Qwen3ForCausalLM", Qwen3Config, build_qwen3_spec, aliases=("qwen3",), replace=True, chat_by_default=True
 )

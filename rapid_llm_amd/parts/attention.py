@@ -5,6 +5,9 @@ and k over head_dim before the rotation (:134-137), rotation (:139-140), write o
 step's keys and values into their pages (rapid_llm/modules/attention.py:126-138), attention
 of every query over its request's cached keys up to its own position (:157-240), output
 projection (base.py:164-165).  The norm, the rotation and the cache write are one kernel.
+How the rotation is applied is the position part's to say (its tables' width: how many of a
+head's channels rotate; its ``pairing``: which of them form a pair); the kernels here take
+every such case, the fastest ones the half-split rotation of the whole head.
 
 Keys and values are always read back from the pages, also for the tokens of the current
 step, so that one code path serves whole prompts, portions and single decoded tokens
@@ -57,6 +60,15 @@ class GQAAttention(Mixer):
         self.qk_norm_eps = qk_norm_eps
         self.window = int(window)
         self.position = position
+        # what the position part says about its rotation must be something the kernels can do
+        rotary_dim = int(getattr(position, "rotary_dim", 0) or 0)
+        pairing = getattr(position, "pairing", "half_split")
+        if rotary_dim % 2 or rotary_dim > head_dim:
+            raise ValueError(f"the position encoding rotates {rotary_dim} channels of heads of {head_dim}")
+        if pairing not in ops.ROTARY_PAIRINGS:
+            raise ValueError(
+                f"the attention kernels rotate pairs as {sorted(ops.ROTARY_PAIRINGS)}, not as {pairing!r}"
+            )
         self.scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(head_dim)
         self.name = name
         self.names = dict(q=q_name, k=k_name, v=v_name, o=o_name, qn=q_norm_name, kn=k_norm_name)
@@ -112,7 +124,10 @@ class GQAAttention(Mixer):
 
     # ---- cache -----------------------------------------------------------------
     def cache_need(self) -> CacheNeed:
-        return CacheNeed("kv", window=self.window, num_kv_heads=self.nkv, head_dim=self.d)
+        return CacheNeed.keys_and_values(self.nkv, self.d, window=self.window)
+
+    def recorded_step_bytes(self, rows: int, context_bound: int, page_size: int) -> int:
+        return ops.decode_scratch_bytes(rows, self.nq, self.nkv, self.d, context_bound, page_size, self.window)
 
     # ---- step ------------------------------------------------------------------
     @property
@@ -129,7 +144,8 @@ class GQAAttention(Mixer):
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
         out = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         rotary_half = cos.shape[1] if cos is not None else 0
-        if ops.decode_attention_fusable(ctx, qkv.dtype, self.nq // self.nkv, self.d, rotary_half):
+        pairing = getattr(pos_enc, "pairing", "half_split") if cos is not None else "half_split"
+        if ops.decode_attention_fusable(ctx, qkv.dtype, self.nq // self.nkv, self.d, rotary_half, pairing):
             # a step of single tokens: norm, rotation, cache write and attention in one kernel
             ops.decode_attention_fused(
                 qkv, cache.k, cache.v, out, ctx, table, cache.page_size, self.nq, self.nkv, self.d,
@@ -143,7 +159,7 @@ class GQAAttention(Mixer):
             cache.v if cache.owns_pages else None,
             self.q_norm_w, self.k_norm_w, cos, sin,
             ctx.positions, ctx.token_slot, table, cache.page_size,
-            self.nq, self.nkv, self.d, eps, ctx.max_position,
+            self.nq, self.nkv, self.d, eps, ctx.max_position, pairing,
         )
         ops.paged_attention(
             q, cache.k, cache.v, out, ctx, table, cache.page_size,

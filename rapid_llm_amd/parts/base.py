@@ -81,11 +81,49 @@ class StateSpec:
 
 
 @dataclass(frozen=True)
+class PagedSpec:
+    """One paged tensor of a mixer: what it keeps per position, and where the positions of a
+    page lie among that array's axes.
+
+    Per position the mixer keeps an array of ``shape``; the cache holds it as
+    ``[pages, *shape[:slot_axis], page_size, *shape[slot_axis:]]``.  Keys of ``h`` heads of ``d``
+    channels with ``slot_axis=1`` are ``[pages, h, page_size, d]`` (a key is one contiguous row);
+    the same shape with ``slot_axis=2`` is ``[pages, h, d, page_size]`` (stored transposed: the
+    positions of a page are contiguous for one channel); one latent row of ``r`` channels per
+    token, ``shape=(r,)`` with ``slot_axis=0``, is ``[pages, page_size, r]``
+    (rapid_llm/engine/kv_cache_spec.py:171-188 is such a row).
+    """
+
+    name: str
+    shape: tuple[int, ...]
+    slot_axis: int = 0
+    dtype: str | None = None  # torch dtype name; None: the engine's compute type
+
+    def __post_init__(self) -> None:
+        if not self.shape or any(int(n) < 1 for n in self.shape):
+            raise ValueError(f"paged tensor {self.name!r} needs a per-position shape of positive sizes, got {self.shape}")
+        if not 0 <= self.slot_axis <= len(self.shape):
+            raise ValueError(f"paged tensor {self.name!r}: slot_axis {self.slot_axis} is outside its shape {self.shape}")
+
+    def page_shape(self, pages: int, page_size: int) -> tuple[int, ...]:
+        return (pages, *self.shape[: self.slot_axis], page_size, *self.shape[self.slot_axis :])
+
+    def elements(self) -> int:
+        """Elements one position costs."""
+        count = 1
+        for n in self.shape:
+            count *= int(n)
+        return count
+
+
+@dataclass(frozen=True)
 class CacheNeed:
     """What a mixer asks of the cache manager.
 
-    ``kind == "kv"``: paged keys and values; ``window`` 0 keeps every position, otherwise
-    only the last ``window`` positions of a request are kept and older pages are given back.
+    ``kind == "paged"``: tensors that grow with the request, in pages, each named and laid out
+    by a :class:`PagedSpec` (keys and values here; a mixer may name one latent row, or keys and
+    values of different widths).  ``window`` 0 keeps every position, otherwise only the last
+    ``window`` positions of a request are kept and older pages are given back.
     ``kind == "state"``: nothing paged.  Fixed-size per-request tensors the mixer owns, zeroed
     when a request takes the slot, may accompany either kind: one as ``state_shape`` (and
     ``state_dtype``), or several, each under a name, as ``states`` (a mixer with a short
@@ -94,14 +132,30 @@ class CacheNeed:
     writing its own.
     """
 
-    kind: str  # "kv" | "state" | "none"
+    kind: str  # "paged" | "state" | "none"
     window: int = 0
-    num_kv_heads: int = 0
-    head_dim: int = 0
+    paged: tuple[PagedSpec, ...] = ()
     state_shape: tuple[int, ...] | None = None
     state_dtype: str | None = None  # torch dtype name; None: the engine's compute type
     share_with: int | None = None
     states: tuple[StateSpec, ...] = ()
+
+    def __post_init__(self) -> None:
+        if self.kind not in ("paged", "state", "none"):
+            raise ValueError(f"a cache need is 'paged', 'state' or 'none', not {self.kind!r}")
+        if (self.kind == "paged") != bool(self.paged):
+            raise ValueError(f"a {self.kind!r} cache need names {len(self.paged)} paged tensors")
+        names = [p.name for p in self.paged]
+        if len(names) != len(set(names)):
+            raise ValueError(f"a mixer names two paged tensors alike: {names}")
+
+    @classmethod
+    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int = 0, **more) -> "CacheNeed":
+        """The layout the attention kernels of this package read: keys ``[pages, heads,
+        page_size, head_dim]`` under ``"k"``, values transposed ``[pages, heads, head_dim,
+        page_size]`` under ``"v"``."""
+        shape = (num_kv_heads, head_dim)
+        return cls("paged", window=window, paged=(PagedSpec("k", shape, 1), PagedSpec("v", shape, 2)), **more)
 
     def state_specs(self) -> tuple[StateSpec, ...]:
         """Every per-request tensor asked for; the one given as ``state_shape`` is named ``"state"``."""
@@ -137,11 +191,30 @@ class Part:
         """Receive the loaded tensors (keyed by ``ParamSpec.name``) and the runtime
         (device, compute type, kernel library, largest sequence length)."""
 
+    def recorded_step_bytes(self, rows: int, context_bound: int, page_size: int) -> int:
+        """Bytes of device memory, beyond a few rows of activations, that one run of this part
+        keeps alive inside a recorded step of ``rows`` single tokens over contexts of at most
+        ``context_bound`` positions (partial results between two of its kernels, work lists).
+        The engine reserves them when it sizes the page pool from what is free."""
+        return 0
+
 
 class PositionEncoding(Part):
-    """Supplies what a mixer needs to encode a token's absolute position."""
+    """Supplies what a mixer needs to encode a token's absolute position, and says how it is
+    applied; the mixer's kernels do the applying, or refuse what they cannot do.
+
+    A rotary encoding exposes, after ``bind``: ``cos`` and ``sin``, float32
+    ``[positions, rotary_dim // 2]``; ``rotary_dim``, the leading channels of a head that
+    rotate (the rest pass unrotated); and ``pairing``, which channels form a rotated pair:
+    ``"half_split"`` pairs channel ``i`` with ``i + rotary_dim // 2``, ``"interleaved"`` channel
+    ``2i`` with ``2i + 1``.  An encoding that rotates nothing leaves ``cos`` and ``sin`` ``None``.
+    """
 
     kind = "none"
+    pairing = "half_split"
+    rotary_dim = 0
+    cos = None
+    sin = None
 
 
 class Mixer(Part):

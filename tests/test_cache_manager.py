@@ -166,7 +166,7 @@ def test_no_page_lost_or_held_twice_under_random_orders(windows, seed):
 
 
 def test_layers_are_grouped_by_what_they_keep():
-    kv = lambda w, share=None: CacheNeed("kv", window=w, num_kv_heads=2, head_dim=16, share_with=share)
+    kv = lambda w, share=None: CacheNeed.keys_and_values(2, 16, window=w, share_with=share)
     needs = [kv(0), kv(16), kv(0), CacheNeed("state", state_shape=(4,)), kv(16), kv(0, share=0)]
     groups, group_of = plan_groups(needs)
     assert [(g.window, g.layers) for g in groups] == [(0, (0, 2, 5)), (16, (1, 4))]
@@ -175,3 +175,32 @@ def test_layers_are_grouped_by_what_they_keep():
         plan_groups([kv(0, share=1), CacheNeed("none")])
     with pytest.raises(ValueError, match="same positions"):
         plan_groups([kv(0), kv(8, share=0)])
+
+
+def test_a_mixer_names_its_paged_tensors_and_their_layout():
+    """What a page holds is the mixer's to say: keys and values of different widths, or one
+    latent row per token without values; the bytes a page id costs are summed from what is named."""
+    from rapid_llm_amd.cache.storage import page_bytes
+    from rapid_llm_amd.parts import PagedSpec
+
+    attention = CacheNeed.keys_and_values(2, 16)
+    assert [(p.name, p.page_shape(10, 4)) for p in attention.paged] == [("k", (10, 2, 4, 16)), ("v", (10, 2, 16, 4))]
+    latent = CacheNeed("paged", paged=(PagedSpec("latent", (24,), 0),))
+    assert latent.paged[0].page_shape(10, 4) == (10, 4, 24)
+    uneven = CacheNeed("paged", window=8, paged=(PagedSpec("k", (3, 32), 1), PagedSpec("v", (3, 8), 1, "float32")))
+    needs = [attention, latent, uneven, CacheNeed("state", state_shape=(4,))]
+    groups, group_of = plan_groups(needs)
+    assert group_of == [0, 0, 1, None]
+    # a page of 4 positions, 2-byte elements: (2*16 + 2*16) + 24 elements in group 0;
+    # 3*32 two-byte and 3*8 four-byte elements in group 1
+    assert page_bytes(needs, group_of, 4, 2) == {0: 4 * 2 * (64 + 24), 1: 4 * (96 * 2 + 24 * 4)}
+    with pytest.raises(ValueError, match="names 0 paged tensors"):
+        CacheNeed("paged")
+    with pytest.raises(ValueError, match="names 1 paged tensors"):
+        CacheNeed("state", paged=(PagedSpec("x", (2,)),))
+    with pytest.raises(ValueError, match="alike"):
+        CacheNeed("paged", paged=(PagedSpec("k", (2,)), PagedSpec("k", (3,))))
+    with pytest.raises(ValueError, match="slot_axis"):
+        PagedSpec("k", (2, 4), 3)
+    with pytest.raises(ValueError, match="other paged tensors"):
+        plan_groups([attention, CacheNeed.keys_and_values(2, 32, share_with=0)])

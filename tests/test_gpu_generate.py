@@ -32,7 +32,7 @@ def _plain_generate(cfg, w, prompt, n, temperature=0.0, top_p=1.0, seed=0, penal
 
 
 def test_greedy_generation_tiny_a_float32(tmp_path):
-    """BASELINE configuration A: prompts of 1/5/13/29 tokens, 12 greedy tokens each."""
+    """Tiny configuration A: prompts of 1/5/13/29 tokens, 12 greedy tokens each."""
     from rapid_llm_amd import SamplingParams
 
     cfg, page, seed = TINY["A"]
@@ -53,7 +53,7 @@ def test_greedy_generation_tiny_a_float32(tmp_path):
 
 
 def test_sampled_generation_tiny_b_chunked_and_mixed(tmp_path):
-    """BASELINE configuration B: prompts of 2/17/31/64/90/150 tokens in portions of 24 mixed
+    """Tiny configuration B: prompts of 2/17/31/64/90/150 tokens in portions of 24 mixed
     with decodes, then 20 tokens each at temperature 0.8 with a fixed seed."""
     from rapid_llm_amd import SamplingParams
 
@@ -425,6 +425,17 @@ def test_the_page_pool_is_what_memory_is_left_and_a_budget_of_nothing_is_refused
     estimate = runner._graph_pool_estimate()
     assert estimate > 0 and runner.state_bytes == 0
     assert ModelRunner(model_dir, EngineConfig(use_graph=False, **common))._graph_pool_estimate() == 0
+    # a batch is padded up to the next size of the ladder: five requests record eight rows, and
+    # the split results that the decode attention keeps between its kernels are counted
+    by_seqs = {
+        n: ModelRunner(model_dir, EngineConfig(**dict(common, max_num_seqs=n, num_pages=8)))._graph_pool_estimate()
+        for n in (4, 5, 8)
+    }
+    assert by_seqs[5] == by_seqs[8] > by_seqs[4]
+    mixer = runner.model.blocks[0].mixer
+    assert mixer.recorded_step_bytes(1, 128, page) == 0  # too few keys to split
+    kept = mixer.recorded_step_bytes(1, 4096, page)
+    assert kept == 1 * cfg["num_attention_heads"] * 32 * (cfg["head_dim"] + 2) * 4  # 32 splits of 128 keys
     # keep back more than is free: nothing is left for pages
     too_little = max(1e-6, min(0.5, 0.5 * free / total) * 1e-3)
     with pytest.raises(ValueError, match="no memory is left for the cache"):
@@ -514,6 +525,34 @@ def test_command_line_bench(tmp_path, capsys):
                  "--input-len", "64", "--range-ratio", "0.25", "--gen-len", "5", "--iterations", "1", "--warmup", "0"])
     line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
     assert code == 0 and (line["input_len_min"], line["input_len_max"]) == (16, 64)
+
+
+def test_command_line_bench_profile(tmp_path, capsys):
+    """``--profile`` prints the device time of every part by kind of step: every part of the
+    model is there, the decode steps were timed eagerly, and the regions add up to their total."""
+    import json
+    import re
+
+    from rapid_llm_amd.cli import main
+
+    model_dir = make_model_dir(tmp_path, "D", "bfloat16")
+    code = main(["bench", "--model-dir", str(model_dir), "--max-seq-len", "128", "--batch-size", "3",
+                 "--input-len", "20", "--gen-len", "6", "--iterations", "1", "--warmup", "0", "--profile"])
+    shown = capsys.readouterr()
+    assert code == 0 and json.loads(shown.out.strip().splitlines()[-1])["tgs"] > 0
+    table = shown.err
+    assert "steps with prompt portions:" in table and "decode steps:" in table
+    decode = table.split("decode steps:")[1]
+    for region in ("embedding (TokenEmbedding)", "mixer norm (RMSNorm)", "mixer (GQAAttention)",
+                   "feed-forward norm (RMSNorm)", "feed-forward (SwiGLU)", "final norm (RMSNorm)",
+                   "output projection (LinearOutput)"):
+        assert region in decode, f"{region} is missing:\n{table}"
+    # five decode steps of a two-layer model: ten calls of every part of a layer, five of the ends
+    calls = {m.group(1).strip(): int(m.group(2)) for m in re.finditer(r"^  (.+?)\s+(\d+) calls", decode, re.M)}
+    assert calls["mixer (GQAAttention)"] == 10 and calls["output projection (LinearOutput)"] == 5
+    total = float(re.search(r"^\s*([0-9.]+) ms inside parts", decode, re.M).group(1))
+    parts = sum(float(m.group(1)) for m in re.finditer(r"calls\s+([0-9.]+) ms", decode))
+    assert abs(parts - total) < 0.01 * total + 0.01
 
 
 def test_smoke_entry():

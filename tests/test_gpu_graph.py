@@ -140,7 +140,7 @@ def test_graph_of_more_requests_than_the_chip_holds_workgroups(tmp_path):
     from rapid_llm_amd.kernels import ops
 
     batch, page, seed = 200, 8, 91
-    assert batch * MANY_HEADS["num_key_value_heads"] > ops._DECODE_ORDER_ABOVE
+    assert batch * MANY_HEADS["num_key_value_heads"] > ops.chip().decode_resident
     model_dir = tmp_path / "many_heads"
     write_random_model(dict(MANY_HEADS), seed, model_dir, dtype="bfloat16", norm_std=0.1)
     make = lambda graph: ModelRunner(

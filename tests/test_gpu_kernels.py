@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from plain_model import plain_attention, plain_inv_freq, plain_rmsnorm, plain_rope_apply, plain_rope_tables
+from rotation_reference import rotate_pairs
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -99,6 +100,10 @@ ATTN_CASES = [
     (4, 1, 64, 8, 3000, [(12000, 1), (5000, 40)]),               # a window deep in a long context
     (8, 2, 128, 16, 0, [(3584, 512)]),   # one portion of a long prompt: few, long tiles, their keys cut into runs
     (6, 3, 64, 8, 0, [(1500, 300), (40, 1), (2100, 33)]),  # the same beside a single token, odd lengths
+    # the head counts of the family's two larger dense models (groups of 8 and of 5 query heads a
+    # kv head): a single token over 9,000 keys, a portion of 512 behind 7,000, a two-token portion
+    (64, 8, 128, 16, 0, [(9000, 1), (7000, 512), (5, 2)]),
+    (40, 8, 128, 16, 0, [(9001, 1), (6990, 512), (0, 2)]),
 ]
 
 
@@ -186,7 +191,7 @@ def test_decode_attention_of_many_requests_of_mixed_lengths(dtype):
     ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, 0, 1.0 / math.sqrt(d))
     if dtype == torch.bfloat16:
         plan = ops.attention_plan(ctx, nq // nkv, d)
-        assert plan.num_decode == 260 and plan.num_decode * nkv > ops._DECODE_ORDER_ABOVE
+        assert plan.num_decode == 260 and plan.num_decode * nkv > ops.chip().decode_resident
         order = plan._decode_order
         assert order is not None, "the launch was not ordered"
         tokens = plan.seq_token.cpu().tolist()
@@ -311,7 +316,7 @@ def _decode_splits(ops, context, nkv, page):
     lays out splits of at most ``chunk`` keys, the kernel deals the request's keys to them evenly
     in runs of a multiple of 32, at least 128."""
     pairs = nkv
-    want = max(1, ops._TARGET_BLOCKS // pairs)
+    want = max(1, ops.chip().units // pairs)
     chunk = max(ops._MIN_SPLIT_KEYS, -(-(-(-context // want)) // 128) * 128)
     chunk = min(chunk, max(32, ((ops._MAX_SPLIT_PAGES - 1) * page - 31) // 32 * 32))
     nsplit = -(-context // chunk)
@@ -489,6 +494,76 @@ def test_qknorm_rope_kvwrite(dtype, shape, many):
     assert torch.isnan(kc[~written_k]).all()  # nothing else was touched
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("case", [
+    # nq, nkv, d, page, channels that rotate, pairing
+    (4, 2, 64, 8, 32, "half_split"),     # the first half of the head only
+    (4, 2, 64, 8, 64, "interleaved"),    # pairs (2i, 2i + 1) over the whole head
+    (6, 3, 48, 4, 16, "interleaved"),    # a third of the head, interleaved
+    (3, 1, 128, 16, 64, "half_split"),
+    (2, 2, 24, 4, 12, "half_split"),     # a head size that no vector access divides evenly
+    (5, 5, 256, 8, 2, "interleaved"),    # one pair
+], ids=lambda c: f"h{c[0]}kv{c[1]}d{c[2]}r{c[4]}{c[5]}")
+@pytest.mark.parametrize("many", [False, True], ids=["few", "many"])
+def test_qknorm_rope_in_other_pairings_and_widths(dtype, case, many):
+    """How a rotation is applied is the position part's to say: the first ``rotary_dim`` channels
+    of a head rotate, as half-split or as interleaved pairs, the rest pass with the norm alone.
+    Against the rotation written as a complex product."""
+    ops = _ops()
+    nq, nkv, d, page, rot, pairing = case
+    theta, eps = 5000.0, 1e-5
+    positions = (list(range(2, 31)) + [90, 91, 400]) if many else [0, 1, 5, 400]
+    slots = ([1] * 29 + [0, 0, 2]) if many else [1, 1, 0, 2]
+    t = len(positions)
+    gen = torch.Generator().manual_seed(d + rot)
+    qkv = torch.randn((t, (nq + 2 * nkv) * d), generator=gen).to(dtype)
+    qw = 1 + 0.1 * torch.randn(d, generator=gen)
+    kw = 1 + 0.1 * torch.randn(d, generator=gen)
+    table = torch.zeros((3, 401 // page + 1), dtype=torch.int32)
+    pid = 1
+    for p, s in zip(positions, slots):
+        if table[s, p // page] == 0:
+            table[s, p // page] = pid
+            pid += 1
+    kc = torch.full((pid, nkv, page, d), float("nan"), dtype=dtype, device=DEV)
+    vc = torch.full((pid, nkv, d, page), float("nan"), dtype=dtype, device=DEV)
+    inv = 1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
+    cos, sin = ops.rope_table(inv.to(DEV), 401)
+    assert cos.shape == (401, rot // 2)
+    q_out = torch.empty(t, nq * d, dtype=dtype, device=DEV)
+    ops.qknorm_rope_kvwrite(
+        qkv.to(DEV), q_out, kc, vc, qw.to(DEV), kw.to(DEV), cos, sin,
+        torch.tensor(positions, dtype=torch.int32, device=DEV),
+        torch.tensor(slots, dtype=torch.int32, device=DEV), table.to(DEV), page, nq, nkv, d, eps, max(positions),
+        pairing,
+    )
+    x = qkv.float()
+    q = x[:, : nq * d].view(t, nq, d)
+    k = x[:, nq * d : (nq + nkv) * d].view(t, nkv, d)
+    v = x[:, (nq + nkv) * d :].view(t, nkv, d)
+    pos = torch.tensor(positions)
+    want_q = rotate_pairs(plain_rmsnorm(q, qw, eps), pos, rot, theta, pairing).reshape(t, nq * d)
+    want_k = rotate_pairs(plain_rmsnorm(k, kw, eps), pos, rot, theta, pairing)
+    tol = dict(rtol=1e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=8e-3, atol=8e-3)
+    torch.testing.assert_close(q_out.float().cpu(), want_q, **tol)
+    # the channels beyond the rotated ones are the normed input, whatever the position
+    if rot < d:
+        torch.testing.assert_close(
+            q_out.float().cpu().view(t, nq, d)[..., rot:], plain_rmsnorm(q, qw, eps)[..., rot:], **tol)
+    kc, vc = kc.float().cpu(), vc.float().cpu()
+    for i, (p, s) in enumerate(zip(positions, slots)):
+        page_id, off = int(table[s, p // page]), p % page
+        torch.testing.assert_close(kc[page_id, :, off, :], want_k[i], **tol)
+        torch.testing.assert_close(vc[page_id, :, :, off], v[i], rtol=0, atol=0)
+    with pytest.raises(ops.KernelError, match="pairing"):
+        ops.qknorm_rope_kvwrite(
+            qkv.to(DEV), q_out, kc.to(DEV, dtype), vc.to(DEV, dtype), qw.to(DEV), kw.to(DEV), cos, sin,
+            torch.tensor(positions, dtype=torch.int32, device=DEV),
+            torch.tensor(slots, dtype=torch.int32, device=DEV), table.to(DEV), page, nq, nkv, d, eps, max(positions),
+            "by_threes",
+        )
+
+
 @pytest.mark.parametrize("shape", [(1, 96, 64), (7, 503, 96), (130, 200, 333), (64, 64, 16), (33, 48, 7),
                                    (40, 1000, 4100), (19, 70, 130)])
 def test_gemm_f32(shape):
@@ -646,7 +721,7 @@ def test_gate_up_product_that_streams_several_pairs_a_workgroup(shape, scaled):
         out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
         rc = core.rl_gemm_skinny_swiglu(
             ctypes.c_void_p(xd.data_ptr()), ctypes.c_void_p(wd.data_ptr()), ctypes.c_void_p(out.data_ptr()),
-            m, inter, k, k, k, inter, nt, ctypes.c_void_p(partial.data_ptr() if scaled else 0),
+            m, inter, k, k, k, inter, nt, ops.chip().units, ctypes.c_void_p(partial.data_ptr() if scaled else 0),
             7 if scaled else 0, k if scaled else 0, ctypes.c_float(1e-6), ops._stream())
         assert rc == 0
         return out

@@ -21,6 +21,15 @@ def _close(got, want, dtype, label):
         parity.assert_bf16_close(got, want, label)
 
 
+def _bucket(position, longest):
+    """The context bound of the recorded step that serves a step whose largest position is
+    ``position``: the next power of two from 512 on, within the engine's longest sequence."""
+    bound = 512
+    while bound <= position:
+        bound *= 2
+    return min(bound, longest)
+
+
 def _runner(model_dir, dtype, page, max_seq_len, graph=False, num_pages=None, seqs=4):
     from rapid_llm_amd import EngineConfig, ModelRunner
 
@@ -61,9 +70,36 @@ def test_long_decoding(tmp_path, which, dtype, graph):
         _close(out, want[rid], dtype, f"long/{which}/{'graph' if graph else 'eager'}/{rid}")
         runner.finish(rid)
     if graph:
-        assert len({key[1] for key in runner._graphs}) >= 1
+        # two rows side by side from position 70 on, then the short request's row alone; every
+        # context bucket those positions cross was recorded, and no other
+        assert {key[0] for key in runner._graphs} == {1, 2}
+        assert {key[1] for key in runner._graphs} == {_bucket(p, limit) for p in range(70, limit)}
     if which in ("C", "D"):  # windowed layers gave pages back while decoding
         assert runner.cache.num_free_pages(1) == runner.cache.pools[1].num_usable
+    runner.cache.check_invariants()
+
+
+def test_decoding_across_three_context_buckets(tmp_path):
+    """One request decodes from position 400 to 1,099 from graphs: the recordings for contexts
+    of up to 512, up to 1,024 and up to the engine's longest sequence follow each other, each
+    with its own layout of the key splits, and every token's logits are the plain ones."""
+    from rapid_llm_amd import StepEntry
+    from rapid_llm_amd.weights import write_random_model
+
+    cfg, page, seed = TINY["B"]
+    limit = 1100
+    model_dir = tmp_path / "long_b"
+    write_random_model(dict(cfg, max_position_embeddings=limit), seed, model_dir, dtype="bfloat16", norm_std=0.1)
+    pcfg, pw = plain_load(model_dir)
+    toks = random_tokens(limit, cfg["vocab_size"], seed + 5)
+    want = plain_forward(pcfg, pw, toks)
+    runner = _runner(model_dir, "bfloat16", page, limit, graph=True, seqs=1)
+    got = [runner.step([StepEntry("r", toks[:400], [399])]).cpu()]
+    for t in toks[400:]:
+        got.append(runner.step([StepEntry("r", [t], [0])]).cpu())
+    _close(torch.cat(got), want[399:], "bfloat16", "long/three buckets")
+    assert set(runner._graphs) == {(1, 512), (1, 1024), (1, limit)}
+    runner.finish("r")
     runner.cache.check_invariants()
 
 

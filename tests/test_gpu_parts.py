@@ -10,6 +10,7 @@ import pytest
 import torch
 
 import parity
+from rotation_reference import rotate_pairs
 from plain_model import (
     plain_attention,
     plain_load,
@@ -139,19 +140,23 @@ class ToyConfig:
     ends: bool = False  # an embedding that scales its rows and an output projection that caps its logits
     replay: bool = False  # the toy mixer runs on the device alone and declares itself replayable
     bias: bool = False  # the attention's projections have biases (Qwen3 has none; the part can)
+    latent: int = 0  # > 0: layer 0's mixer pages one latent row of so many channels per token, and no values
+    rotation: str = "whole"  # "half": a position part defined here rotates the first half of a head; "interleaved"
 
     @classmethod
     def from_dict(cls, data, overrides=None):
         return cls(data["hidden"], data["vocab"], data["heads"], data["head_dim"], data["inter"],
                    data["decay"], data.get("twice", False), data.get("share", False),
                    data.get("experts", 0), data.get("period", 0.0), data.get("toynorm", False),
-                   data.get("ends", False), data.get("replay", False), data.get("bias", False))
+                   data.get("ends", False), data.get("replay", False), data.get("bias", False),
+                   data.get("latent", 0), data.get("rotation", "whole"))
 
     def to_dict(self):
         return dict(architectures=["ToyForCausalLM"], hidden=self.hidden, vocab=self.vocab, heads=self.heads,
                     head_dim=self.head_dim, inter=self.inter, decay=self.decay, twice=self.twice,
                     share=self.share, experts=self.experts, period=self.period, toynorm=self.toynorm,
-                    ends=self.ends, replay=self.replay, bias=self.bias, torch_dtype="float32")
+                    ends=self.ends, replay=self.replay, bias=self.bias, latent=self.latent,
+                    rotation=self.rotation, torch_dtype="float32")
 
 
 CAP = 0.3  # the toy output projection's cap: logits = CAP * tanh(h W^T / CAP)
@@ -167,7 +172,7 @@ def _toy_parts():
     from rapid_llm_amd.kernels.upload import upload_ints
     from rapid_llm_amd.parts import (
         EMBEDDINGS, FEED_FORWARDS, MIXERS, NORMS, OUTPUT_PROJECTIONS, POSITION_ENCODINGS, CacheNeed, Embedding,
-        FeedForward, Mixer, Norm, OutputProjection, ParamSpec, PositionEncoding, Source, StateSpec,
+        FeedForward, Mixer, Norm, OutputProjection, PagedSpec, ParamSpec, PositionEncoding, Source, StateSpec,
     )
     from rapid_llm_amd.parts.linear import Linear
 
@@ -367,6 +372,74 @@ def _toy_parts():
             return self.proj(out.to(x.dtype))
 
     MIXERS.register("toy_device_decaying_sum", DeviceDecayingSum, replace=True)
+
+    class LatentMemory(Mixer):
+        """A mixer that pages one latent row per token and no values: ``c_t = x_t Wd`` is written
+        to the token's place in the request's pages (``[pages, page_size, rank]``, as this mixer
+        names it), a token attends over the latents up to its own with ``q_t = x_t Wq``, and the
+        mix of latents goes up through ``Wu``.  The cache manager, the device cache and the step
+        function see only a paged tensor called "latent"."""
+
+        def __init__(self, hidden_size, rank, checkpoint_prefix, position=None, name="mixer"):
+            self.h, self.r, self.prefix, self.name = hidden_size, rank, checkpoint_prefix, name
+            self.down, self.query, self.up = Linear(hidden_size, rank), Linear(hidden_size, rank), Linear(rank, hidden_size)
+
+        def param_specs(self):
+            p, n = self.prefix, self.name
+            return [ParamSpec(n + ".wd", (self.r, self.h), "matrix", (Source(p + "wd", self.r),)),
+                    ParamSpec(n + ".wq", (self.r, self.h), "matrix", (Source(p + "wq", self.r),)),
+                    ParamSpec(n + ".wu", (self.h, self.r), "matrix", (Source(p + "wu", self.h),))]
+
+        def bind(self, params, runtime):
+            self.down.bind(params[self.name + ".wd"])
+            self.query.bind(params[self.name + ".wq"])
+            self.up.bind(params[self.name + ".wu"])
+
+        def cache_need(self):
+            return CacheNeed("paged", paged=(PagedSpec("latent", (self.r,), 0),))
+
+        def forward(self, x, ctx, cache):
+            store, size = cache.pages["latent"], cache.page_size
+            table = ctx.block_tables[cache.group_id]
+            assert store.shape[1:] == (size, self.r) and cache.k is None and cache.v is None
+            c, q = self.down(x), self.query(x)
+            pos, slots = ctx.positions.long(), ctx.token_slot.long()
+            page = table[slots, pos // size].long()
+            store[page, pos % size] = c  # this step's latents first, then everything is read back
+            out = torch.empty_like(c, dtype=torch.float32)
+            at = 0
+            for slot, start, n in zip(ctx.h_seq_slots, ctx.h_seq_starts, ctx.h_seq_lens):
+                total = start + n
+                pages = table[slot, : -(-total // size)].long()
+                mem = store[pages].reshape(-1, self.r)[:total].float()
+                scores = q[at : at + n].float() @ mem.T / math.sqrt(self.r)
+                seen = torch.arange(total, device=x.device)[None, :] <= (start + torch.arange(n, device=x.device))[:, None]
+                out[at : at + n] = torch.softmax(scores.masked_fill(~seen, float("-inf")), dim=-1) @ mem
+                at += n
+            return self.up(out.to(x.dtype))
+
+    MIXERS.register("toy_latent_memory", LatentMemory, replace=True)
+
+    class HalfHeadRotary(PositionEncoding):
+        """A rotation of the first half of a head only, tables made here with tensor operations.
+        It says how it is to be applied (``rotary_dim``, ``pairing``); the attention part of the
+        package and its kernels do the applying."""
+
+        kind = "toy_half_rotary"
+        replayable = True
+        pairing = "half_split"
+
+        def __init__(self, head_dim, theta):
+            self.head_dim, self.theta, self.rotary_dim = head_dim, theta, head_dim // 2
+
+        def bind(self, params, runtime):
+            rot = self.rotary_dim
+            inv = 1.0 / (self.theta ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
+            angle = (torch.arange(runtime.max_seq_len).float()[:, None] * inv[None, :]).double()
+            self.cos = angle.cos().float().to(runtime.device).contiguous()
+            self.sin = angle.sin().float().to(runtime.device).contiguous()
+
+    POSITION_ENCODINGS.register("toy_half_rotary", HalfHeadRotary, replace=True)
     return DeviceDecayingSum
 
 
@@ -381,6 +454,10 @@ def _toy_spec(cfg: ToyConfig):
                                    "checkpoint_prefix": f"l{i}.ff."})
 
     rope = PartSpec("rope_half_split", {"head_dim": cfg.head_dim, "theta": 100.0})
+    if cfg.rotation == "half":
+        rope = PartSpec("toy_half_rotary", {"head_dim": cfg.head_dim, "theta": 100.0})
+    elif cfg.rotation == "interleaved":
+        rope = PartSpec("rope", {"head_dim": cfg.head_dim, "theta": 100.0, "pairing": "interleaved"})
 
     def attn(i):
         return PartSpec("gqa_attention", {"hidden_size": cfg.hidden, "num_heads": cfg.heads, "num_kv_heads": 1,
@@ -397,10 +474,13 @@ def _toy_spec(cfg: ToyConfig):
             return PartSpec("toy_plain_norm", {"size": cfg.hidden, "eps": 1e-5, "checkpoint_name": name})
         return norm(name)
 
+    mixer0 = PartSpec("toy_device_decaying_sum" if cfg.replay else "toy_decaying_sum",
+                      {"hidden_size": cfg.hidden, "decay": cfg.decay, "checkpoint_prefix": "l0.mix."})
+    if cfg.latent:
+        mixer0 = PartSpec("toy_latent_memory", {"hidden_size": cfg.hidden, "rank": cfg.latent,
+                                                "checkpoint_prefix": "l0.mix."})
     layers = [
-        LayerSpec(PartSpec("toy_device_decaying_sum" if cfg.replay else "toy_decaying_sum",
-                           {"hidden_size": cfg.hidden, "decay": cfg.decay, "checkpoint_prefix": "l0.mix."}),
-                  ff0, norm("l0.n1"), norm("l0.n2"), position=pos0),
+        LayerSpec(mixer0, ff0, norm("l0.n1"), norm("l0.n2"), position=pos0),
         LayerSpec(attn(1), ff(1), norm1("l1.n1"), norm1("l1.n2"), position=rope),
     ]
     if cfg.share:
@@ -436,8 +516,19 @@ def _toy_plain(w, cfg: ToyConfig, toks):
         return h + plain_swiglu_mlp(x, w[f"l{i}.ff.gate_proj.weight"], w[f"l{i}.ff.up_proj.weight"],
                                     w[f"l{i}.ff.down_proj.weight"])
 
+    def rotate(x):
+        if cfg.rotation == "whole":
+            c, s = plain_rope_tables(pos, cfg.head_dim, 100.0)
+            return plain_rope_apply(x, c, s)
+        rot = cfg.head_dim // 2 if cfg.rotation == "half" else cfg.head_dim
+        return rotate_pairs(x, pos, rot, 100.0, "half_split" if cfg.rotation == "half" else "interleaved")
+
     def toy(h):
         x = plain_rmsnorm(h, w["l0.n1"], 1e-5)
+        if cfg.latent:
+            c, q = x @ w["l0.mix.wd"].T, x @ w["l0.mix.wq"].T
+            scores = (q @ c.T / math.sqrt(cfg.latent)).masked_fill(pos[None, :] > pos[:, None], float("-inf"))
+            return ffn(0, h + (torch.softmax(scores, dim=-1) @ c) @ w["l0.mix.wu"].T)
         s, rows = torch.zeros(cfg.hidden), []
         if cfg.period:
             x = x + _phase(pos, cfg.period, cfg.hidden)
@@ -452,14 +543,12 @@ def _toy_plain(w, cfg: ToyConfig, toks):
 
     def kv_of(i, h):
         x = plain_rmsnorm(h, w[f"l{i}.n1"], 1e-5)
-        c, s = plain_rope_tables(pos, cfg.head_dim, 100.0)
-        k = plain_rope_apply(proj(i, "k", x).view(t, 1, cfg.head_dim), c, s)
+        k = rotate(proj(i, "k", x).view(t, 1, cfg.head_dim))
         return k, proj(i, "v", x).view(t, 1, cfg.head_dim)
 
     def attn(i, h, kv=None):
         x = plain_rmsnorm(h, w[f"l{i}.n1"], 1e-5)
-        c, s = plain_rope_tables(pos, cfg.head_dim, 100.0)
-        q = plain_rope_apply(proj(i, "q", x).view(t, cfg.heads, cfg.head_dim), c, s)
+        q = rotate(proj(i, "q", x).view(t, cfg.heads, cfg.head_dim))
         k, v = kv if kv is not None else kv_of(i, h)
         o = plain_attention(q, k, v, cfg.head_dim**-0.5).reshape(t, -1)
         return ffn(i, h + proj(i, "o", o))
@@ -485,6 +574,8 @@ def _unregister_toys():
     unregister_architecture("ToyForCausalLM")
     MIXERS.unregister("toy_decaying_sum")
     MIXERS.unregister("toy_device_decaying_sum")
+    MIXERS.unregister("toy_latent_memory")
+    POSITION_ENCODINGS.unregister("toy_half_rotary")
     FEED_FORWARDS.unregister("toy_routed")
     POSITION_ENCODINGS.unregister("toy_phase")
     NORMS.unregister("toy_plain_norm")
@@ -495,8 +586,10 @@ def _unregister_toys():
 @pytest.mark.parametrize("variant,dtype", [("plain", "float32"), ("twice", "float32"), ("share", "float32"),
                                            ("routed", "float32"), ("toynorm", "float32"), ("ends", "float32"),
                                            ("replay", "float32"), ("bias", "float32"),
+                                           ("latent", "float32"), ("halfrot", "float32"), ("interleaved", "float32"),
                                            ("routed", "bfloat16"), ("toynorm", "bfloat16"), ("twice", "bfloat16"),
-                                           ("ends", "bfloat16"), ("bias", "bfloat16")])
+                                           ("ends", "bfloat16"), ("bias", "bfloat16"),
+                                           ("latent", "bfloat16"), ("halfrot", "bfloat16"), ("interleaved", "bfloat16")])
 def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
     """In bfloat16 the built-in parts hand unfinished products and unscaled rows to each other
     in steps of few tokens; the toy parts declare nothing and must only ever see tensors."""
@@ -508,11 +601,14 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
     _toy_parts()
     register_architecture("ToyForCausalLM", ToyConfig, _toy_spec, replace=True)
     try:
-        cfg = ToyConfig(hidden=48, vocab=97, heads=3, head_dim=16, inter=80, decay=0.8,
-                        twice=variant == "twice", share=variant == "share",
+        # the other rotations at a head size whose single-token steps would otherwise run the
+        # kernel that rotates inside the attention: it must be passed by for them
+        other_rotation = {"halfrot": "half", "interleaved": "interleaved"}.get(variant, "whole")
+        cfg = ToyConfig(hidden=48, vocab=97, heads=3, head_dim=64 if other_rotation != "whole" else 16, inter=80,
+                        decay=0.8, twice=variant == "twice", share=variant == "share",
                         experts=3 if variant == "routed" else 0, period=9.0 if variant == "routed" else 0.0,
                         toynorm=variant == "toynorm", ends=variant == "ends", replay=variant == "replay",
-                        bias=variant == "bias")
+                        bias=variant == "bias", latent=24 if variant == "latent" else 0, rotation=other_rotation)
         folder = write_random_model(cfg.to_dict(), 3, tmp_path / "toy", dtype=dtype)
         weights = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
         if variant == "share":  # the sharing layer's own k/v projections exist but are never used
@@ -521,7 +617,18 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, variant, dtype):
         needs = runner.model.cache_needs()
         if variant == "toynorm":
             assert type(runner.model.blocks[1].mixer_norm).__name__ == "PlainTorchNorm"
-        assert needs[0].kind == "state" and needs[1].kind == "kv"
+        assert needs[0].kind == ("paged" if variant == "latent" else "state") and needs[1].kind == "paged"
+        if variant == "latent":
+            # a page of the shared group costs the latent row and layer 1's keys and values
+            elem = 4 if dtype == "float32" else 2
+            assert [p.name for p in needs[0].paged] == ["latent"] and runner.device_cache.layers[0].k is None
+            assert runner.device_cache.layers[0].pages["latent"].shape[1:] == (8, cfg.latent)
+            assert runner.page_bytes == {0: 8 * elem * (cfg.latent + 2 * cfg.head_dim)}
+        if variant == "halfrot":
+            position = runner.model.blocks[1].mixer.position
+            assert type(position).__name__ == "HalfHeadRotary" and position.cos.shape[1] == cfg.head_dim // 4
+        if variant == "interleaved":
+            assert runner.model.blocks[1].mixer.position.pairing == "interleaved"
         if variant == "bias":
             assert weights["l1.attn.q_proj.bias"].shape == (cfg.heads * cfg.head_dim,)
             assert weights["l1.attn.o_proj.bias"].abs().max() > 0

@@ -151,6 +151,104 @@ def test_benchmark_widths_match_plain(model, reference, dtype):
     assert not runner.cache.live_requests()
 
 
+# Two layers at the widths of the family's largest dense model (hidden 5,120, 64 query heads on 8
+# kv heads of 128: groups of 8, intermediate 25,600) with the vocabulary cut to 32,000 so that
+# the plain implementation's float32 copy stays within a few gigabytes, at a long context: a
+# 9,000-token prompt in portions of 8,192 and 808 (the second a few long tiles behind a long
+# prefix), then single tokens at batch 1, 8 and 32 replayed from graphs of the 16,384 bucket.
+LARGE = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
+    head_dim=128, intermediate_size=25600, vocab_size=32000, rope_theta=1000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=16384,
+    hidden_act="silu", attention_bias=False,
+)
+LARGE_PROMPT = 9000
+LARGE_STEPS = 2  # single-token steps at each batch size
+
+
+def _large_plan():
+    """(tokens by request, steps as (label, [(request, start, count, wanted places)], graph))."""
+    vocab = LARGE["vocab_size"]
+    prompt = {"long": LARGE_PROMPT}
+    for i in range(31):
+        prompt[f"s{i}"] = 2 + (i * 11) % 70
+    tokens = {r: random_tokens(n + 3 * LARGE_STEPS, vocab, 2000 + k) for k, (r, n) in enumerate(prompt.items())}
+    done = {r: 0 for r in prompt}
+    steps = []
+
+    def entry(rid, count, want):
+        e = (rid, done[rid], count, want)
+        done[rid] += count
+        return e
+
+    steps.append(("first portion of 8,192", [entry("long", 8192, [0, 1, 4095, 4096, 8190, 8191])], False))
+    steps.append(("second portion behind 8,192", [entry("long", LARGE_PROMPT - 8192, [0, 1, 400, 806, 807])], False))
+    for i in range(LARGE_STEPS):
+        steps.append((f"batch 1 step {i}", [entry("long", 1, [0])], True))
+    seven = [f"s{i}" for i in range(7)]
+    steps.append(("seven prompts", [entry(r, prompt[r], [prompt[r] - 1]) for r in seven], False))
+    for i in range(LARGE_STEPS):
+        steps.append((f"batch 8 step {i}", [entry(r, 1, [0]) for r in ["long"] + seven], True))
+    rest = [f"s{i}" for i in range(7, 31)]
+    steps.append(("24 prompts", [entry(r, prompt[r], [prompt[r] - 1]) for r in rest], False))
+    for i in range(LARGE_STEPS):
+        steps.append((f"batch 32 step {i}", [entry(r, 1, [0]) for r in ["long"] + seven + rest], True))
+    return tokens, steps
+
+
+@pytest.fixture(scope="module")
+def large(tmp_path_factory):
+    """The model folder, the plan and the plain logits at every compared position."""
+    from rapid_llm_amd import write_random_model
+
+    folder = tmp_path_factory.mktemp("largest_widths") / "two_layers"
+    write_random_model(dict(LARGE), 13, folder, dtype="bfloat16", norm_std=0.1)
+    tokens, steps = _large_plan()
+    rows: dict[str, list[int]] = {r: [] for r in tokens}
+    for _label, entries, _graph in steps:
+        for rid, start, _count, want in entries:
+            rows[rid].extend(start + w for w in want)
+    pcfg, pw = plain_load(folder)
+    plain = {}
+    for rid, at in rows.items():
+        logits = plain_forward(pcfg, pw, tokens[rid][: max(at) + 1], rows=at)
+        plain[rid] = {pos: logits[i] for i, pos in enumerate(at)}
+    del pw
+    return folder, tokens, steps, plain
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_largest_widths_at_a_long_context_match_plain(large, dtype):
+    from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
+
+    folder, tokens, steps, plain = large
+    runner = ModelRunner(
+        folder,
+        EngineConfig(dtype=dtype, max_seq_len=16384, page_size=PAGE, num_pages=800, max_num_seqs=32, use_graph=True),
+    )
+    for label, entries, graph in steps:
+        before = set(runner._graphs)
+        logits = runner.step(
+            [StepEntry(rid, tokens[rid][start : start + count], want) for rid, start, count, want in entries]
+        ).cpu()
+        want = torch.stack([plain[rid][start + w] for rid, start, count, ws in entries for w in ws])
+        assert logits.shape == want.shape, label
+        if graph:
+            assert (len(entries), 16384) in runner._graphs, f"{label}: no graph of the 16,384 bucket ({sorted(runner._graphs)})"
+        else:
+            assert set(runner._graphs) == before, f"{label}: a step with a portion was recorded"
+        if dtype == "float32":
+            err = float((logits - want).abs().max())
+            print(f"largest widths float32 {label}: worst error {err:.3e} (logits spread {float(want.std()):.3f})")
+            torch.testing.assert_close(logits, want, **F32_TOL)
+        else:
+            parity.assert_bf16_close(logits, want, f"largest widths/{label}")
+    for rid in tokens:
+        runner.finish(rid)
+    runner.cache.check_invariants()
+
+
 # Two layers at the widths of the family's smallest model (hidden 1,024, 16 query and 8 kv heads
 # of 128, intermediate 3,072), a short vocabulary: its QKV and gate/up matrices are the few
 # megabytes for which steps of 17 to 512 rows run the one-launch tile product (with SwiGLU in

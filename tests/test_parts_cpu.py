@@ -109,10 +109,10 @@ def test_a_mixer_may_ask_for_several_state_tensors():
 
     one = CacheNeed("state", state_shape=(48,), state_dtype="float32")
     assert [(s.name, s.shape, s.dtype) for s in one.state_specs()] == [("state", (48,), "float32")]
-    two = CacheNeed("kv", num_kv_heads=2, head_dim=16,
+    two = CacheNeed.keys_and_values(2, 16,
                     states=(StateSpec("conv", (3, 48)), StateSpec("count", (1,), "int32")))
     assert [s.name for s in two.state_specs()] == ["conv", "count"]
-    assert CacheNeed("kv", num_kv_heads=1, head_dim=16).state_specs() == ()
+    assert CacheNeed.keys_and_values(1, 16).state_specs() == ()
     # five slots: 48 float32 each; 3 x 48 in the engine's type (2 bytes) and one int32 each
     assert state_bytes([one, two], 5, 2) == 5 * 48 * 4 + 5 * (3 * 48 * 2 + 4)
     with pytest.raises(ValueError, match="alike"):
@@ -174,12 +174,27 @@ def test_which_products_run_in_one_launch_of_this_package():
     assert not ops._tile_applies(64, 4098, 1024, 4098)    # four result columns a lane
 
 
-def test_the_decode_launch_is_ordered_only_beyond_what_runs_at_once():
-    """Decode attention asks for the requests' order by length only when the launch has more
-    workgroups than the chip holds at a time (three on each of 256 compute units)."""
+def test_launch_rules_follow_the_number_of_compute_units():
+    """Every launch rule takes the chip's geometry from one place on the host
+    (``ops.chip()``; without a device the chip the rules were measured on), so that a part
+    with another number of compute units gets shapes for itself: decode attention asks for the
+    requests' order by length only beyond three workgroups a unit, and the few-row product's
+    rows a workgroup and the runs of K of the mid-size product move with the unit count."""
+    from types import SimpleNamespace
+
     from rapid_llm_amd.kernels import ops
 
-    assert ops._DECODE_ORDER_ABOVE == 3 * 256
+    assert ops.chip().units == 256 and ops.chip().decode_resident == 3 * 256
+    assert ops.Chip(304).first_round == 304 and ops.Chip(304).prefill_slots == 608
+    # 384 tiles of 16 rows: one round of 24 rows on 256 units, nothing to gain on 384 units
+    assert ops._skinny_tiles(8, 6144, plain=True, units=256) == 3
+    assert ops._skinny_tiles(8, 6144, plain=True, units=384) == 1
+    # 64 blocks of 64 rows: four runs of K fill 256 units, one run fills 64
+    assert ops.mid_runs(4096, 4096, units=256) == 4 and ops.mid_runs(4096, 4096, units=64) == 1
+    # a portion behind a long prefix is cut into key runs only while the launch leaves slots free
+    tile = SimpleNamespace(tile_keys=[4096] * 4, num_tiles=4)
+    assert ops._prefill_shape(tile, 8, 0, 128, units=256)[1] > 1
+    assert ops._prefill_shape(tile, 8, 0, 128, units=8) == (1, 1)
 
 
 def test_weight_rows_a_workgroup_of_the_few_row_product():

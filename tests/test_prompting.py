@@ -92,3 +92,52 @@ def test_stop_ids_are_the_tokenizers_and_the_generation_configs(tmp_path):
         eos_token_id = 9
 
     assert load_stop_token_ids(folder, (), WithId()) == {9}
+
+
+def test_whether_an_architecture_chats_by_default_is_its_registry_entrys_flag(tmp_path):
+    """No architecture is named beside the prompt code: a newly registered one says itself
+    whether its releases are chat models, and one that is not registered gets prompts verbatim."""
+    from rapid_llm_amd.config import register_architecture, unregister_architecture
+
+    class ToyConfig:
+        @classmethod
+        def from_dict(cls, data, overrides=None):
+            return cls()
+
+    folder = _folder(tmp_path, "Toy-1B", model_type="toy_chat", chat_template=TEMPLATE)
+    assert not is_instruct(folder) and build_prompter(folder) is None
+    register_architecture("ToyChatLM", ToyConfig, lambda cfg: None, aliases=("toy_chat",), chat_by_default=True)
+    register_architecture("ToyBaseLM", ToyConfig, lambda cfg: None, aliases=("toy_base",))
+    try:
+        assert is_instruct(folder) and build_prompter(folder).insert_prompt("x").endswith("<assistant>")
+        assert not is_instruct(_folder(tmp_path, "Toy-1B-Base", model_type="toy_chat"))
+        assert not is_instruct(_folder(tmp_path, "Other-1B", model_type="toy_base"))
+        by_name = _folder(tmp_path, "Named-1B")
+        (by_name / "config.json").write_text(json.dumps({"architectures": ["ToyChatLM"]}))
+        assert is_instruct(by_name)
+    finally:
+        unregister_architecture("ToyChatLM")
+        unregister_architecture("ToyBaseLM")
+    assert not is_instruct(folder)
+
+
+def test_templates_may_use_what_model_folders_templates_use():
+    """Loop controls, a ``tojson`` that writes plain JSON (no HTML escapes, which would change the
+    prompt's tokens; ``ensure_ascii`` and ``indent`` as arguments) and ``strftime_now``."""
+    import datetime
+
+    template = (
+        "{% for m in messages %}{% if m['role'] == 'skip' %}{% continue %}{% endif %}"
+        "{% if m['role'] == 'stop' %}{% break %}{% endif %}"
+        "{{ m['content'] | tojson }};{% endfor %}"
+        "{{ {'k': ['<a>', 'é']} | tojson(indent=1) }}|{{ 'é' | tojson(ensure_ascii=true) }}|{{ strftime_now('%Y') }}"
+    )
+    talk = [{"role": "user", "content": "<b> & \"q\" 'é'"}, {"role": "skip", "content": "no"},
+            {"role": "user", "content": "two"}, {"role": "stop", "content": "x"}, {"role": "user", "content": "late"}]
+    text = ChatPrompter(template).apply(talk)
+    first, second, tail = text.split(";", 2)
+    assert json.loads(first) == talk[0]["content"] and "<b> & " in first and "é" in first
+    assert second == '"two"' and "late" not in text and '"no"' not in text
+    indented, ascii_only, year = tail.split("|")
+    assert indented == json.dumps({"k": ["<a>", "é"]}, ensure_ascii=False, indent=1)
+    assert ascii_only == '"\\u00e9"' and year == str(datetime.datetime.now().year)

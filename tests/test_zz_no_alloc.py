@@ -70,3 +70,36 @@ def test_sizes_beyond_the_array_are_refused():
     assert _call(lib, logits[:ok_rows], out[:ok_rows]) == 0
     torch.cuda.synchronize()
     assert (out[:ok_rows] == 0).all()
+
+
+def test_it_runs_under_graph_capture_and_leaves_the_devices_memory_as_it_was():
+    """What the entry point is for: after ``rl_argmax_static_prepare()`` a call may be recorded
+    into a HIP graph (an allocation, or the lookup of the array's address, would fail the
+    capture), and eager calls change nothing in the device's free memory.  The graph is replayed
+    several times with other logits and eager work in between; every replay must be right."""
+    lib = _lib()
+    assert lib.rl_argmax_static_prepare() == 0
+    gen = torch.Generator().manual_seed(5)
+    rows, vocab = 6, 9001
+    logits = torch.randn((rows, vocab), generator=gen).cuda()
+    out = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
+    assert _call(lib, logits, out) == 0  # the kernels' code is loaded before anything is measured
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        assert _call(lib, logits, out) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.equal(out.cpu().long(), logits.cpu().argmax(dim=1))
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        code = _call(lib, logits, out)  # the current stream is the capturing one
+    assert code == 0
+    for _ in range(3):
+        fresh = torch.randn((rows, vocab), generator=gen)
+        logits.copy_(fresh.cuda())
+        out.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu().long(), fresh.argmax(dim=1))
