@@ -185,6 +185,75 @@ def test_causal_and_prefix_consistent(models, which):
     assert not torch.allclose(changed[30:], full[30:])
 
 
+def _library_block(h, cfg, w, layer, order="reference"):
+    """One block written a second time, from library routines alone (``F.rms_norm``,
+    ``torch.polar``, ``F.scaled_dot_product_attention``, ``F.silu``, ``F.linear``), in the order
+    of rapid_llm/models/base.py:231-266 (norm, mixer, add, norm, feed-forward, add) and :121-165
+    (projection, head norms *before* the rotation, attention, output projection).  ``order``
+    names a plausible misreading instead: the head norms after the rotation, or the norms
+    behind the sub-layers (post-norm)."""
+    p = f"model.layers.{layer}."
+    eps, nq = cfg["rms_norm_eps"], cfg["num_attention_heads"]
+    nkv, d, t = cfg["num_key_value_heads"], cfg["head_dim"], h.shape[0]
+    angle = torch.outer(torch.arange(t, dtype=torch.float32), plain_inv_freq(d, cfg["rope_theta"])).double()
+    unit = torch.polar(torch.ones_like(angle), angle)[:, None, :]
+
+    def rotate(x):
+        z = torch.complex(x[..., : d // 2], x[..., d // 2 :]) * unit
+        return torch.cat((z.real, z.imag), dim=-1)
+
+    def head_norm(x, name):
+        return F.rms_norm(x, (d,), w[p + name], eps)
+
+    def mixer(x):
+        q = F.linear(x, w[p + "self_attn.q_proj.weight"]).view(t, nq, d)
+        k = F.linear(x, w[p + "self_attn.k_proj.weight"]).view(t, nkv, d)
+        v = F.linear(x, w[p + "self_attn.v_proj.weight"]).view(t, nkv, d)
+        if order == "norm after rotation":
+            q, k = head_norm(rotate(q), "self_attn.q_norm.weight"), head_norm(rotate(k), "self_attn.k_norm.weight")
+        else:
+            q, k = rotate(head_norm(q, "self_attn.q_norm.weight")), rotate(head_norm(k, "self_attn.k_norm.weight"))
+        group = nq // nkv
+        o = F.scaled_dot_product_attention(
+            q.transpose(0, 1)[None], k.transpose(0, 1).repeat_interleave(group, 0)[None],
+            v.transpose(0, 1).repeat_interleave(group, 0)[None], is_causal=True, scale=d**-0.5,
+        )[0].transpose(0, 1).reshape(t, nq * d)
+        return F.linear(o, w[p + "self_attn.o_proj.weight"])
+
+    def feed_forward(x):
+        gate, up = F.linear(x, w[p + "mlp.gate_proj.weight"]), F.linear(x, w[p + "mlp.up_proj.weight"])
+        return F.linear(F.silu(gate) * up, w[p + "mlp.down_proj.weight"])
+
+    n1 = lambda x: F.rms_norm(x, (x.shape[-1],), w[p + "input_layernorm.weight"], eps)
+    n2 = lambda x: F.rms_norm(x, (x.shape[-1],), w[p + "post_attention_layernorm.weight"], eps)
+    if order == "post-norm":
+        h = n1(h + mixer(h))
+        return n2(h + feed_forward(h))
+    h = h + mixer(n1(h))
+    return h + feed_forward(n2(h))
+
+
+@pytest.mark.parametrize("which", ["A", "B", "E"])
+def test_block_is_library_routines_in_the_references_order(models, which):
+    """The order of a block (which norm feeds what, where the residual is added, the head norms
+    before the rotation) is pinned by a second writing of the block from library routines; the
+    two misreadings that a reader could fall into are shown to give other numbers, so the
+    comparison could fail."""
+    cfg, w = models[which]
+    assert plain_layer_windows(cfg) == [None] * cfg["num_hidden_layers"]
+    t = 23
+    h = torch.randn(t, cfg["hidden_size"], dtype=torch.float64, generator=torch.Generator().manual_seed(8))
+    for layer in range(cfg["num_hidden_layers"]):
+        got = plain_block(h, cfg, w, layer, torch.arange(t), None)
+        torch.testing.assert_close(got, _library_block(h, cfg, w, layer), atol=1e-9, rtol=1e-9)
+        for wrong in ("norm after rotation", "post-norm"):
+            other = _library_block(h, cfg, w, layer, wrong)
+            # far beyond the comparison's tolerance (the sub-layers of a random model add little
+            # to a stream of unit size, hence no larger a figure)
+            assert float((other - got).abs().max()) > 1e-4, wrong
+        h = got
+
+
 def test_tied_and_untied_output(models):
     cfg, w = models["A"]
     assert cfg["tie_word_embeddings"] and "lm_head.weight" not in w
