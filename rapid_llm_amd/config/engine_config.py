@@ -24,6 +24,10 @@ class EngineConfig:
     max_num_batched_tokens: int = 8192
     max_chunk_size: int = 512  # 0 turns chunked prefill off
     use_graph: bool = True  # replay decode-only steps from a captured HIP graph
+    # what to do with a decode step whose recording would hold a product of the library (a step
+    # of more rows than this package's own products take, or a matrix whose sizes they refuse):
+    # "record" it as it is, run such steps "eager"ly, or "refuse" with an error (tests)
+    library_in_graph: str = "record"
     # queue the next step before the last one's tokens are read (rapid_llm/engine/scheduler.py:
     # 302-303); None: the environment variable RAPID_LLM_PIPELINE, on when it is not set
     pipeline: bool | None = None
@@ -42,6 +46,10 @@ class EngineConfig:
         for name in ("max_num_seqs", "max_num_batched_tokens"):
             if getattr(self, name) < 1:
                 raise ConfigError(f"{name} must be positive, got {getattr(self, name)}")
+        if self.library_in_graph not in ("record", "eager", "refuse"):
+            raise ConfigError(
+                f"library_in_graph must be 'record', 'eager' or 'refuse', got {self.library_in_graph!r}"
+            )
         if self.max_chunk_size < 0:
             raise ConfigError(f"max_chunk_size must be >= 0, got {self.max_chunk_size}")
         if self.max_chunk_size == 0 and self.max_num_batched_tokens < self.max_seq_len:

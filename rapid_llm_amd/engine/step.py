@@ -157,6 +157,9 @@ class ModelRunner:
         self.computed: dict[str, int] = {}
         self.vocab_size = self.spec.vocab_size
         self._graphs: dict[tuple[int, int], tuple] = {}
+        # (rows, context bound) -> products of the library that the recorded step holds; a key
+        # whose step is not replayed because of them (library_in_graph="eager") is listed too
+        self.graph_library_products: dict[tuple[int, int], int] = {}
         # a part that does not promise to be replayable keeps every step eager
         self.graphs_allowed = self.model.replayable()
         # where the sampling kernels leave their choices, one row per sampled request of a
@@ -378,12 +381,14 @@ class ModelRunner:
         )
         return host, offs, padded
 
-    def _graph_step(self, entries, meta) -> torch.Tensor:
-        """A step of single tokens, all wanted: replayed from a HIP graph.  Graphs exist for a
+    def _graph_step(self, entries, meta) -> torch.Tensor | None:
+        """A step of single tokens, all wanted: replayed from a HIP graph (``None``: this shape's
+        step holds a product of the library and the engine is told to run such steps eagerly).  Graphs exist for a
         ladder of batch sizes and for context buckets (the next power of two); a batch is
         padded with filler rows to the next size of the ladder, so that a few captures serve
-        every batch a scheduler produces.  The graph holds only this package's kernels (and
-        the library's products above 16 rows); its inputs are one static int32 buffer,
+        every batch a scheduler produces.  The graph holds this package's kernels, and the
+        library's products where a step has more rows than the package's own products take
+        (``graph_library_products`` says how many); its inputs are one static int32 buffer,
         refreshed by a copy on the same stream before each replay.  Launch decisions that
         depend on the context length are made for the bucket's longest context."""
         batch = len(entries)
@@ -397,6 +402,8 @@ class ModelRunner:
         bound = min(bound, self.engine.max_seq_len)
         key = (rows, bound)
         entry = self._graphs.get(key)
+        if entry is None and self.engine.library_in_graph == "eager" and self.graph_library_products.get(key):
+            return None  # found out at the first try: this shape's step holds a library product
         if entry is None:
             # One eager run first, on a side stream: kernels get loaded, the allocator warm, and
             # the parts make the launch data they keep in ctx.static.  It runs filler rows only
@@ -411,6 +418,7 @@ class ModelRunner:
             )
             ctx.static["decode_only_tokens"] = torch.arange(rows, dtype=torch.int32, device=self.device)
             ctx.static["context_bound"] = bound
+            library_before = ops.library_products
             current = torch.cuda.current_stream()
             side = torch.cuda.Stream()
             side.wait_stream(current)
@@ -422,9 +430,22 @@ class ModelRunner:
             # only) was uploaded by that run and is kept: nothing may be copied from the host
             # while the graph is recorded.  Everything else of that run is dropped.
             ctx.extra = {}
+            # The eager run told which products of this shape go to the library.  Its kernels
+            # are not this package's: some clear a workspace first, and which one runs depends
+            # on the rows, the matrix and the library's version.
+            library = ops.library_products
+            if library != library_before and self.engine.library_in_graph != "record":
+                self.graph_library_products[key] = library - library_before
+                if self.engine.library_in_graph == "refuse":
+                    raise ops.KernelError(
+                        f"a decode step of {rows} rows would record {library - library_before} products of "
+                        "the library into its graph (library_in_graph='refuse')"
+                    )
+                return None
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, self.device_cache.layers)
+            self.graph_library_products[key] = ops.library_products - library
             # the graph's kernel nodes hold raw pointers: everything they point at that was
             # allocated outside the capture (the static inputs, what ctx.static holds) must
             # live as long as the graph does, so the context is kept with it
@@ -453,6 +474,8 @@ class ModelRunner:
         ):
             logits = self._graph_step(entries, meta)
         else:
+            logits = None
+        if logits is None:
             host, offs = self._pack(entries, meta)
             dev = upload(host, self.device)
             logits = self.model.forward(self._context(dev, offs, meta), self.device_cache.layers)

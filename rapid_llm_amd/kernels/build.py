@@ -39,6 +39,7 @@ CORE_SOURCES = (
     "attention_generic.hip",
     "sampling.hip",
     "gemm_bf16.hip",
+    "gemm_rows.hip",
 )
 ATTENTION_SOURCES = ("attention_mfma.hip", "attention_f32.hip")
 HEADERS = ("common.h", "static_entry.h")

@@ -8,6 +8,7 @@ GPU or without the compiled library these raise.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
 
 import torch
@@ -550,8 +551,10 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, scaled=N
     the result (see ``gemm_bf16_residual``).
 
     Up to 16 rows (decode) run the hand-written bandwidth-bound kernel, which can write
-    float32 directly.  More rows go to the library product, as the reference's dense products do
-    (``F.linear``); its bfloat16 result is returned as is and widened by the caller."""
+    float32 directly; so does the kernel for 17 to 64 rows over wide matrices.  Small matrices
+    run the one-launch tile product up to 512 rows.  Everything else goes to the library
+    product, as the reference's dense products do (``F.linear``); a bfloat16 result is returned
+    as is and widened by the caller."""
     _need(x, "x", torch.bfloat16)
     _need(w, "w", torch.bfloat16)
     m, k = x.shape
@@ -576,7 +579,66 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, scaled=N
         out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
         _ok(core().rl_gemm_tile(_p(x), _p(w), _p(out), m, n, k, k, k, n, 0, _stream()), "rl_gemm_tile")
         return out
+    plan = rows_plan(m, n, k, swiglu=False)
+    if plan is not None:
+        wide = torch.float32 if out_dtype == torch.float32 else torch.bfloat16
+        out = torch.empty((m, n), dtype=wide, device=x.device)
+        _ok(
+            core().rl_gemm_rows(_p(x), _p(w), _p(out), m, n, k, k, k, n, 0, _tag(wide), *plan, _stream()),
+            "rl_gemm_rows",
+        )
+        return out
+    return library_product(x, w)
+
+
+# How many products went to the library since the process started.  A step that is recorded into
+# a graph is meant to hold this package's kernels only where they exist; whoever records one
+# reads the counter before and after.
+library_products = 0
+
+
+def library_product(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x w^T`` by the library (hipBLASLt behind ``torch.matmul``), as the reference's dense
+    products are ``F.linear``: the many-row products of prompt steps, and what no kernel of
+    this package takes."""
+    global library_products
+    library_products += 1
     return torch.matmul(x, w.t())
+
+
+ROWS_MAX_ROWS = 64  # rows up to which wide matrices run the kernel that keeps X in registers
+
+
+def rows_plan(m: int, n: int, k: int, swiglu: bool, units: int | None = None) -> tuple[int, int] | None:
+    """(result tiles a workgroup holds, workgroups) for the product of 17 to 64 rows over a wide
+    matrix with ``n`` result columns (with SwiGLU a tile is a gate and an up tile), ``None`` where
+    that kernel does not apply.  A compute unit gets one workgroup with an even share of the
+    tiles where a workgroup can hold such a share (the packed gate and up matrices of Qwen3-8B:
+    768 pairs, three a unit); a matrix with more tiles than that (the vocabulary) is cut into
+    workgroups of the most tiles one holds, which the chip takes in turn."""
+    if not (SKINNY_MAX_ROWS < m <= ROWS_MAX_ROWS) or n % 16 or k % 128 or k < 128:
+        return None
+    if os.environ.get("RAPID_LLM_ROWS_PRODUCT") == "0":  # the library instead, for comparing the two
+        return None
+    units = chip().units if units is None else units
+    tiles = n // 16
+    if 2 * tiles < units:  # too few workgroups to stream from
+        return None
+    holds = ((2, 3, 5) if m <= 48 else (2, 3)) if swiglu else (1, 2, 3, 6)
+    share = -(-tiles // min(units, tiles))
+    for per in holds:
+        if per >= share:
+            return per, min(units, tiles)
+    if (swiglu and share > 5) or (not swiglu and share < 24):
+        # More tiles a compute unit than a workgroup holds (beyond 48 rows a workgroup holds
+        # three pairs, and a matrix of up to five pairs a unit is cut into groups of three).  For the packed gate and up matrices
+        # of the 32B shape (524 MB, 12.5 tiles a unit) the library's kernel streams at 5.4 TB/s
+        # at every row count: 97 to 106 us at 17 to 64 rows against 99 to 136 here in any cut with
+        # SwiGLU, 91 against 116 at 32 rows without.  Only for the vocabulary (37 tiles a unit)
+        # are its kernels the slower ones (348 us against 294 at 32 rows of the 32B shape).
+        return None
+    per = holds[-1]
+    return per, -(-tiles // per)
 
 
 def gemm_bf16_residual(
@@ -711,11 +773,22 @@ def gemm_bf16_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, scaled=None) -> t
         return None
     if m > SKINNY_MAX_ROWS:
         inter = two_i // 2
-        if scaled is not None or not _tile_applies(m, two_i, k, inter):
+        if scaled is not None:
             return None
+        _need(x, "x", torch.bfloat16)
         _need(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, k))
+        if _tile_applies(m, two_i, k, inter):
+            out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
+            _ok(core().rl_gemm_tile(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, 1, _stream()), "rl_gemm_tile")
+            return out
+        plan = rows_plan(m, inter, k, swiglu=True)
+        if plan is None:
+            return None
         out = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
-        _ok(core().rl_gemm_tile(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, 1, _stream()), "rl_gemm_tile")
+        _ok(
+            core().rl_gemm_rows(_p(x), _p(w_gate_up), _p(out), m, inter, k, k, k, inter, 1, BF16, *plan, _stream()),
+            "rl_gemm_rows",
+        )
         return out
     _need(x, "x", torch.bfloat16)
     _need(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, k))

@@ -627,7 +627,8 @@ def test_gemm_bf16_swiglu_fused(shape):
     gu = (x.float() @ w.float().T).bfloat16().float()
     want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
     torch.testing.assert_close(got.float().cpu(), want, rtol=2e-2, atol=2e-2)
-    assert ops.gemm_bf16_swiglu(torch.zeros(33, k, dtype=torch.bfloat16, device=DEV), w.to(DEV)) is None
+    if ops.rows_plan(33, inter, k, swiglu=True) is None and not ops._tile_applies(33, 2 * inter, k, inter):
+        assert ops.gemm_bf16_swiglu(torch.zeros(33, k, dtype=torch.bfloat16, device=DEV), w.to(DEV)) is None
 
 
 # rows, result columns, K: row counts around the blocks of 16 and 64 rows, column counts that end
@@ -829,7 +830,76 @@ def test_product_in_runs_of_k_and_the_norm_that_adds_them(shape):
     assert torch.equal(res2, got_res) and torch.equal(out2, out)
 
 
-def test_wide_matrices_stay_with_the_library():
+# rows, result columns, K, SwiGLU, float32 result: every number of tiles a workgroup may hold
+# (1, 2, 3, 6 tiles; 2, 3, 5 pairs), shares that leave some workgroups a tile short, more tiles
+# than one round of workgroups holds (the vocabulary), 17 to 64 rows around the blocks of 16,
+# one chunk of K (most waves then have none) and K that the waves do not share evenly
+ROWS_SHAPES = [
+    (17, 4096, 4096, False, False), (33, 6144, 2048, False, False), (48, 10240, 768, False, False),
+    (64, 6144, 4096, False, False), (20, 16000, 512, False, False), (64, 19200, 384, False, True),
+    (33, 151936, 256, False, True), (64, 151936, 128, False, True), (50, 2048, 4096, False, True),
+    (17, 6144, 2048, True, False), (32, 12288, 4096, True, False), (64, 12288, 1152, True, False),
+    (40, 17408, 256, True, False), (64, 17408, 256, True, False), (48, 20480, 384, True, False),
+    (18, 3088, 1280, True, False),
+]
+
+
+@pytest.mark.parametrize("shape", ROWS_SHAPES, ids=lambda c: f"m{c[0]}n{c[1]}k{c[2]}{'sw' if c[3] else ''}{'f32' if c[4] else ''}")
+def test_rows_product_of_wide_matrices(shape):
+    """The product for 17 to 64 rows that keeps a chunk of X in registers for all the tiles a
+    workgroup owns, through the entry points the parts call; the first and the last result
+    columns, and those where one workgroup's share ends and the next begins, are checked like
+    all others (every column's weights are its own)."""
+    ops = _ops()
+    m, n, k, swiglu, wide_out = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn((m, k), generator=gen).bfloat16()
+    w = (torch.randn(((2 if swiglu else 1) * n, k), generator=gen) / math.sqrt(k)).bfloat16()
+    plan = ops.rows_plan(m, n, k, swiglu)
+    assert plan is not None and not ops._tile_applies(m, w.shape[0], k, n)
+    per, groups = plan
+    assert ops.core().rl_gemm_rows_holds(int(swiglu), per, m) and -(-(n // 16) // groups) <= per
+    before = ops.library_products
+    if swiglu:
+        got = ops.gemm_bf16_swiglu(x.to(DEV), w.to(DEV))
+        gu = (x.float() @ w.float().T).bfloat16().float()
+        want = torch.nn.functional.silu(gu[:, :n]) * gu[:, n:]
+        tol = dict(rtol=2e-2, atol=2e-2)
+    else:
+        got = ops.gemm_bf16(x.to(DEV), w.to(DEV), torch.float32 if wide_out else torch.bfloat16)
+        want = x.float() @ w.float().T
+        tol = dict(rtol=1e-4, atol=1e-4) if wide_out else dict(rtol=1e-2, atol=1e-2)
+    assert ops.library_products == before, "the product went to the library"
+    assert got.shape == (m, n) and got.dtype == (torch.float32 if wide_out else torch.bfloat16)
+    torch.testing.assert_close(got.float().cpu(), want, **tol)
+    # the same bits every run: the waves' sums are added in a fixed order
+    again = ops.gemm_bf16_swiglu(x.to(DEV), w.to(DEV)) if swiglu else ops.gemm_bf16(x.to(DEV), w.to(DEV), got.dtype)
+    assert torch.equal(got, again)
+
+
+def test_rows_product_refuses_what_it_was_not_built_for():
+    import ctypes
+
+    ops = _ops()
+    core = ops.core()
+    x = torch.zeros((64, 256), dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros((2 * 25600, 256), dtype=torch.bfloat16, device=DEV)
+    out = torch.zeros((64, 25600), dtype=torch.bfloat16, device=DEV)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    call = lambda m, n, k, sw, per, groups: core.rl_gemm_rows(P(x), P(w), P(out), m, n, k, k, k, n, sw, 1, per, groups, ops._stream())
+    assert call(64, 25600, 256, 1, 5, 320) == 1   # five pairs beside 64 rows: not built
+    assert call(48, 25600, 256, 1, 5, 320) == 0
+    assert call(48, 25600, 256, 1, 5, 256) == 1   # a share of seven pairs in a workgroup that holds five
+    assert call(48, 25600, 256, 1, 4, 400) == 1   # no kernel holds four pairs
+    assert call(65, 25600, 256, 1, 5, 320) == 1 and call(48, 25608, 256, 1, 5, 321) == 1 and call(48, 25600, 200, 1, 5, 320) == 1
+    torch.cuda.synchronize()
+    assert ops.rows_plan(16, 12288, 4096, True) is None and ops.rows_plan(65, 12288, 4096, True) is None
+    assert ops.rows_plan(33, 12288, 4000, True) is None and ops.rows_plan(33, 1000, 4096, False) is None
+    assert ops.rows_plan(33, 1024, 4096, False) is None  # 64 tiles: too few workgroups to stream from
+    assert ops.rows_plan(33, 25600, 5120, True) is None  # more than five pairs a compute unit: the library's
+
+
+def test_wide_matrices_are_not_cut_into_runs_of_k():
     ops = _ops()
     assert ops.mid_runs(24576, 4096) == 0 and ops.mid_runs(151936, 4096) == 0
     assert ops.mid_runs(4096, 4096) == 4 and ops.mid_runs(4096, 12288) == 4

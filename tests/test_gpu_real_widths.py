@@ -28,9 +28,8 @@ CONFIG = dict(
 )
 PAGE = 16
 DECODE_STEPS = 2  # single-token steps at batch 1 and 8
-# at batch 64 the recorded step holds the library's products, some of them kernels that clear a
-# workspace first: three replays, with an eager prompt step of another request between them,
-# each checked against the plain implementation
+# at batch 64: three replays, with an eager prompt step of another request between them, each
+# checked against the plain implementation
 BATCH64_STEPS = 3
 # float32: sums of 4,096 to 12,288 terms in another order than the plain product's
 F32_TOL = dict(rtol=1e-4, atol=5e-5)
@@ -123,7 +122,9 @@ def test_benchmark_widths_match_plain(model, reference, dtype):
     seqs, steps, plain = reference
     runner = ModelRunner(
         model,
-        EngineConfig(dtype=dtype, max_seq_len=4096, page_size=PAGE, num_pages=1200, max_num_seqs=68, use_graph=True),
+        # a recorded step of up to 64 rows holds this package's kernels only, or the engine raises
+        EngineConfig(dtype=dtype, max_seq_len=4096, page_size=PAGE, num_pages=1200, max_num_seqs=68, use_graph=True,
+                     library_in_graph="refuse"),
     )
     for label, entries, graph in steps:
         before = set(runner._graphs)
@@ -145,10 +146,52 @@ def test_benchmark_widths_match_plain(model, reference, dtype):
             torch.testing.assert_close(logits, want, **F32_TOL)
         else:
             parity.assert_bf16_close(logits, want, f"real widths/{label}")
+    assert runner.graph_library_products and not any(runner.graph_library_products.values())
     for rid in seqs.prompt:
         runner.finish(rid)
     runner.cache.check_invariants()
     assert not runner.cache.live_requests()
+
+
+def test_recorded_steps_of_up_to_64_rows_hold_no_library_product(model):
+    """Every batch size of the ladder up to 64 at the benchmark's widths: the step is recorded
+    under ``library_in_graph="refuse"`` (a product that went to the library would raise), replayed,
+    and gives the plain implementation's logits.  Beyond 64 rows the wide products are the
+    library's: such a step is recorded as it is by default, runs eagerly when the engine is
+    told so, and is refused when it is told that."""
+    from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
+    from rapid_llm_amd.engine.step import GRAPH_BATCHES
+    from rapid_llm_amd.kernels import ops
+
+    pcfg, pw = plain_load(model)
+    vocab = CONFIG["vocab_size"]
+    tokens = random_tokens(96, vocab, 77)
+    plain = {t: plain_forward(pcfg, pw, [t])[0] for t in sorted(set(tokens))}
+    del pw
+    common = dict(dtype="bfloat16", max_seq_len=4096, page_size=PAGE, num_pages=200, max_num_seqs=100, use_graph=True)
+    runner = ModelRunner(model, EngineConfig(library_in_graph="refuse", **common))
+    for rows in [b for b in GRAPH_BATCHES if b <= 64]:
+        for rep in range(2):  # the recording's first replay, and a second with other tokens
+            chosen = tokens[rep : rep + rows]
+            logits = runner.step([StepEntry(f"r{i}", [t], [0]) for i, t in enumerate(chosen)]).cpu()
+            parity.assert_bf16_close(logits, torch.stack([plain[t] for t in chosen]), f"ladder/{rows} rows/{rep}")
+            for i in range(rows):
+                runner.finish(f"r{i}")
+        assert runner.graph_library_products[(rows, 512)] == 0
+    ninety_six = [StepEntry(f"r{i}", [t], [0]) for i, t in enumerate(tokens)]
+    with pytest.raises(ops.KernelError, match="96 rows would record"):
+        runner.step(ninety_six)
+    for i in range(96):
+        runner.finish(f"r{i}")
+    want = torch.stack([plain[t] for t in tokens])
+    for policy in ("eager", "record"):
+        other = ModelRunner(model, EngineConfig(library_in_graph=policy, **common))
+        for rep in range(2):
+            parity.assert_bf16_close(other.step(ninety_six).cpu(), want, f"ladder/96 rows/{policy}/{rep}")
+            for i in range(96):
+                other.finish(f"r{i}")
+        assert ((96, 512) in other._graphs) == (policy == "record")
+        assert other.graph_library_products[(96, 512)] > 0
 
 
 # Two layers at the widths of the family's largest dense model (hidden 5,120, 64 query heads on 8

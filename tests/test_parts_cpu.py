@@ -209,3 +209,23 @@ def test_weight_rows_a_workgroup_of_the_few_row_product():
     assert ops._skinny_tiles(8, 4096, plain=True) == 1      # one tile a unit already
     assert ops._skinny_tiles(16, 151936, plain=True) == 2   # a thousand tiles and more: as measured
     assert ops._skinny_tiles(8, 151936, plain=True) == 1
+
+
+def test_tiles_a_workgroup_of_the_product_for_tens_of_rows():
+    """The host's rule for the product of 17 to 64 rows over wide matrices: a compute unit gets
+    one workgroup with an even share of the tiles where a workgroup can hold such a share, and a
+    matrix with more tiles is cut into workgroups of the most tiles one holds."""
+    from rapid_llm_amd.kernels import ops
+
+    plan = lambda m, n, k, sw: ops.rows_plan(m, n, k, sw, units=256)
+    assert plan(64, 12288, 4096, True) == (3, 256)     # Qwen3-8B gate/up: 768 pairs, three a unit
+    assert plan(32, 6144, 4096, False) == (2, 256)     # its QKV: 384 tiles, one or two a unit
+    assert plan(64, 151936, 4096, False) == (6, 1583)  # the vocabulary: 9,496 tiles in groups of six
+    assert plan(48, 25600, 5120, True) is None         # the 32B shape's gate/up, 1,600 pairs: the library's,
+    assert plan(48, 51200, 5120, False) is None        # with the activation or without
+    assert plan(33, 17408, 5120, True) == (5, 256) and plan(33, 10240, 5120, False) == (3, 256)
+    assert plan(64, 17408, 5120, True) == (3, 363)     # at 64 rows a workgroup holds three pairs at most
+    assert plan(33, 4096, 2048, False) == (1, 256) and plan(33, 2048, 2048, False) == (1, 128)
+    assert plan(33, 12288, 4096, True) == (3, 256) and ops.rows_plan(33, 12288, 4096, True, units=304) == (3, 304)
+    assert plan(16, 12288, 4096, True) is None and plan(65, 12288, 4096, True) is None
+    assert plan(33, 12296, 4096, True) is None and plan(33, 12288, 4160, True) is None
