@@ -69,8 +69,9 @@ __global__ __launch_bounds__(NW* RL_WAVE) void gemm_rows_kernel(
     static_assert(!SWIGLU || TB % 2 == 0, "gate and up tiles come in pairs");
     constexpr int TPU = SWIGLU ? 2 : 1;  // tiles per unit
     constexpr int UNITS = TB / TPU;      // units a workgroup holds at most
-    // units whose partial sums cross LDS together: what fits 64 KB
-    constexpr int UPR_FIT = 64 / (NW * TPU * MB);
+    // units whose partial sums cross LDS together: what fits 96 KB (every barrier of the epilogue
+    // stands in the open, nothing streams behind it)
+    constexpr int UPR_FIT = 96 / (NW * TPU * MB);
     constexpr int UPR = UPR_FIT < 1 ? 1 : (UPR_FIT > UNITS ? UNITS : UPR_FIT);
     __shared__ __attribute__((aligned(16))) unsigned char wtile[NW][16 * RT_PITCH];
     __shared__ float red[NW][UPR * TPU * MB * 256];
