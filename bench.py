@@ -332,8 +332,25 @@ def main() -> int:
     if args.layers is not None:
         shape["num_hidden_layers"] = args.layers
     points = [int(p) for p in args.points.split(",") if p]
-    max_batch = max([args.batch] + points)
     elem = 2 if args.dtype == "bfloat16" else 4
+
+    # batch sizes whose caches do not fit beside the weights are left out, and said so: the
+    # pool is made for the largest batch that is measured
+    from rapid_llm_amd.config.registry import config_from_dict
+
+    _, sized = config_from_dict(shape)
+    per_request = (-(-(prompt_len + room) // 16)) * 16 * kv_bytes_per_token(sized, elem)
+    free, _ = torch.cuda.mem_get_info()
+    most = int((0.92 * free - weight_bytes(sized, elem)) // per_request)
+    if args.batch > most:
+        print(f"a batch of {args.batch} requests of {prompt_len + room} tokens does not fit this device "
+              f"beside the weights ({most} do)")
+        return 2
+    for b in [b for b in points if b > most]:
+        print(f"[bench] batch {b} left out: {most} requests of {prompt_len + room} tokens fit beside the weights",
+              file=sys.stderr, flush=True)
+    points = [b for b in points if b <= most]
+    max_batch = max([args.batch] + points)
 
     engine = EngineConfig(
         dtype=args.dtype,

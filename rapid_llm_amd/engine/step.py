@@ -172,10 +172,23 @@ class ModelRunner:
     # ------------------------------------------------------------------ sizing
     def _decide_num_pages(self, groups) -> int:
         e = self.engine
-        if e.num_pages is not None:
-            return e.num_pages
-        if e.max_gpu_num_blocks is not None:  # the reference's knob counts tokens (README.md:121)
-            return -(-e.max_gpu_num_blocks // e.page_size) + 1
+        asked = e.num_pages
+        if asked is None and e.max_gpu_num_blocks is not None:
+            # the reference's knob counts tokens (README.md:121)
+            asked = -(-e.max_gpu_num_blocks // e.page_size) + 1
+        if asked is not None:
+            # a pool of a given size is made as asked or not at all: say what does not fit
+            # before the allocator fails somewhere in the middle of it
+            per_page = sum(self.page_bytes.values())
+            free, _ = torch.cuda.mem_get_info(self.device)
+            if asked * per_page + self.state_bytes > free:
+                raise ValueError(
+                    f"a cache of {asked} pages of {e.page_size} tokens takes "
+                    f"{(asked * per_page + self.state_bytes) >> 20} MiB ({per_page >> 10} KiB a page over the "
+                    f"groups' layers) and {free >> 20} MiB are free beside the weights; ask for at most "
+                    f"{max(0, free - self.state_bytes) // max(per_page, 1)} pages"
+                )
+            return asked
         # what is left of the device after the weights, times the utilisation, less what else the
         # engine will allocate (the per-request state tensors, the recorded steps' private
         # buffers, a step's activations), shared by the groups

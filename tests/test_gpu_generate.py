@@ -440,6 +440,13 @@ def test_the_page_pool_is_what_memory_is_left_and_a_budget_of_nothing_is_refused
     too_little = max(1e-6, min(0.5, 0.5 * free / total) * 1e-3)
     with pytest.raises(ValueError, match="no memory is left for the cache"):
         ModelRunner(model_dir, EngineConfig(gpu_memory_utilization=too_little, **common))
+    # a pool of a given size that cannot be made says so, and how many pages can, before anything
+    # is allocated
+    per_page = sum(runner.page_bytes.values())
+    with pytest.raises(ValueError, match=r"a cache of \d+ pages .* ask for at most \d+ pages"):
+        ModelRunner(model_dir, EngineConfig(num_pages=total // per_page + 2, **common))
+    with pytest.raises(ValueError, match="ask for at most"):
+        ModelRunner(model_dir, EngineConfig(max_gpu_num_blocks=(total // per_page + 2) * page, **common))
 
 
 def test_template_and_stop_token_of_the_model_folder(tmp_path, capsys):
