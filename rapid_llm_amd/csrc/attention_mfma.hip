@@ -24,7 +24,8 @@
 //
 //   rl_attn_prefill: portions of prompts.  Workgroup = 4 waves x 32 rows; K and V^T tiles of
 //                    64 keys go through LDS, the next tile travelling from memory while this
-//                    one is multiplied; one softmax step per 64 keys.
+//                    one is multiplied (straight into a second set of tiles for heads of 128
+//                    channels, through registers otherwise); one softmax step per 64 keys.
 //   rl_attn_decode:  single tokens.  Workgroup = (request, kv head, split of the keys); its
 //                    4 waves stride over 32-key steps reading K and V^T straight from
 //                    global memory (nothing is reused), combine through LDS,
@@ -649,7 +650,22 @@ extern "C" int rl_attn_decode_fusable() { return D % 64 == 0 ? 1 : 0; }
 // one's matrix products overlap the other's softmax; better when there is enough work to keep
 // every unit busy (2,048 tokens of Qwen3-8B from the start: 78 against 86 us; 8,192 tokens:
 // 819 against 731 us).
-template <int GROUPS>
+//
+// DIRECT (head size 128, pages of a multiple of eight keys): a step's keys and values go from
+// memory straight into LDS (the loads that name an LDS address, 16 bytes a lane), into one of two
+// sets of tiles in turn, so that a step has one barrier, no wave holds a tile's share in
+// registers and none stores it.  Such a load writes a wave's 64 x 16 bytes side by side, so the
+// tiles have no padding: instead, 16-byte unit u of row r lies at unit u ^ (r % 16) of a key row
+// and u ^ (r / 2 % 8) of a value row (two to 256 bytes), which spreads an operand read's sixteen
+// rows over the banks; a lane asks memory for the unit that belongs at its place.
+typedef __attribute__((address_space(3))) void* rl_lds_ptr;
+typedef const __attribute__((address_space(1))) void* rl_global_ptr;
+constexpr bool PF_DIRECT_OK = (D == 128);
+constexpr int PF_DIRECT_TILE = PF_KEYS * D * 2;      // bytes of a key tile and of a value tile
+constexpr int PF_DIRECT_SET = 2 * PF_DIRECT_TILE;    // one step's tiles
+constexpr int PF_DIRECT_GROUP = 2 * PF_DIRECT_SET;   // a wave group's two sets
+
+template <int GROUPS, bool DIRECT>
 __global__ __launch_bounds__(GROUPS* PF_THREADS) __attribute__((amdgpu_waves_per_eu(1, 2))) void
 attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
@@ -658,7 +674,8 @@ attn_prefill_kernel(
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, unsigned page_magic, int nq, int nkv, int window, float scale_log2, int nsplit,
     float* __restrict__ part_o, float* __restrict__ part_ml) {
-    __shared__ __attribute__((aligned(16))) bf16_t tiles[GROUPS * PF_TILE_ELEMS];
+    constexpr int GROUP_ELEMS = DIRECT ? PF_DIRECT_GROUP / 2 : PF_TILE_ELEMS;  // bfloat16 elements
+    __shared__ __attribute__((aligned(1024))) bf16_t tiles[GROUPS * GROUP_ELEMS];
     __shared__ float fold_ml[GROUPS > 1 ? PF_WAVES * PF_NQ * 2 * RL_WAVE : 1];
 
     const int G = nq / nkv;
@@ -684,8 +701,9 @@ attn_prefill_kernel(
     const int wave = tid / RL_WAVE;
     const int col = lane & 15;
     const int g = lane >> 4;
-    bf16_t* const Ks = tiles + grp * PF_TILE_ELEMS;
-    bf16_t* const Vs = Ks + PF_KEYS * K_LD;
+    bf16_t* const Ks = tiles + grp * GROUP_ELEMS;
+    bf16_t* const Vs = Ks + PF_KEYS * K_LD;  // (the padded layout's; DIRECT: see direct_issue)
+    unsigned char* const dtiles = reinterpret_cast<unsigned char*>(tiles) + grp * (GROUP_ELEMS * 2);
 
     // rows of this lane: one per 16-row block
     int r_tok[PF_NQ], r_head[PF_NQ], r_pos[PF_NQ];
@@ -747,10 +765,16 @@ attn_prefill_kernel(
         v_key = min(base + 4 * (tid % KG), (seq_end - 1) & ~3);
         v_page = table[__umulhi((unsigned)v_key, page_magic)];
     };
+    // a page of one layer's keys (or values) is nkv * page_size * D elements, a count that fits
+    // 32 bits (host-checked), so an address is one 32 x 32 -> 64 bit multiply-add of the page id
+    // and an offset of 32 bits within the page
+    const unsigned page_elems = (unsigned)nkv * (unsigned)page_size * (unsigned)D;
+    const unsigned head_off = (unsigned)hk * (unsigned)page_size * (unsigned)D;
     auto stage_load = [&]() {
         {
-            const int in_page = k_key - (int)__umulhi((unsigned)k_key, page_magic) * page_size;
-            const bf16_t* krow = k_cache + (((size_t)k_page * nkv + hk) * page_size + in_page) * D;
+            const unsigned in_page = (unsigned)k_key - __umulhi((unsigned)k_key, page_magic) * (unsigned)page_size;
+            const bf16_t* krow =
+                k_cache + ((unsigned long long)(unsigned)k_page * page_elems + (head_off + in_page * (unsigned)D));
 #pragma unroll
             for (int i = 0; i < KCH; ++i) {
                 const int ch = tid % TPK + i * TPK;
@@ -758,12 +782,12 @@ attn_prefill_kernel(
             }
         }
         {
-            const int in_page = v_key - (int)__umulhi((unsigned)v_key, page_magic) * page_size;
-            const bf16_t* vbase = v_cache + (((size_t)v_page * nkv + hk) * D) * page_size + in_page;
+            const unsigned in_page = (unsigned)v_key - __umulhi((unsigned)v_key, page_magic) * (unsigned)page_size;
+            const bf16_t* vbase = v_cache + ((unsigned long long)(unsigned)v_page * page_elems + (head_off + in_page));
 #pragma unroll
             for (int i = 0; i < VCH; ++i) {
                 const int d = tid / KG + i * (PF_THREADS / KG);
-                if (d < D) vreg[i] = *reinterpret_cast<const u32x2*>(vbase + (size_t)d * page_size);
+                if (d < D) vreg[i] = *reinterpret_cast<const u32x2*>(vbase + (unsigned)d * (unsigned)page_size);
             }
         }
     };
@@ -783,29 +807,102 @@ attn_prefill_kernel(
         }
         {
             const int kg = tid % KG;
-            const int key = base + 4 * kg;
-            // keys of the group that may be multiplied: written ones (below seq_end) that no
-            // row's window has left behind (their pages may have been given back already)
-            const int lo_cut = tile_kstart - key;  // keys i < lo_cut are out
-            const int hi_cut = seq_end - key;      // keys i >= hi_cut are out
-            const bool all_in = lo_cut <= 0 && hi_cut >= 4;
-            unsigned keep_x = 0, keep_y = 0;  // never multiply stale data, not even by zero
-            if (0 >= lo_cut && 0 < hi_cut) keep_x |= 0x0000ffffu;
-            if (1 >= lo_cut && 1 < hi_cut) keep_x |= 0xffff0000u;
-            if (2 >= lo_cut && 2 < hi_cut) keep_y |= 0x0000ffffu;
-            if (3 >= lo_cut && 3 < hi_cut) keep_y |= 0xffff0000u;
+            // keys that may be multiplied: written ones (below seq_end) that no row's window has
+            // left behind (their pages may have been given back already).  Most steps hold such
+            // keys only (the same for every thread): their values go to LDS as they came
+            if (base >= tile_kstart && base + PF_KEYS <= seq_end) {
 #pragma unroll
-            for (int i = 0; i < VCH; ++i) {
-                const int d = tid / KG + i * (PF_THREADS / KG);
-                if (d < D) {
-                    u32x2 v = vreg[i];
-                    if (!all_in) {
+                for (int i = 0; i < VCH; ++i) {
+                    const int d = tid / KG + i * (PF_THREADS / KG);
+                    if (d < D) *reinterpret_cast<u32x2*>(&Vs[d * V_LD + 4 * kg]) = vreg[i];
+                }
+            } else {
+                const int key = base + 4 * kg;
+                const int lo_cut = tile_kstart - key;  // keys i < lo_cut are out
+                const int hi_cut = seq_end - key;      // keys i >= hi_cut are out
+                unsigned keep_x = 0, keep_y = 0;  // never multiply stale data, not even by zero
+                if (0 >= lo_cut && 0 < hi_cut) keep_x |= 0x0000ffffu;
+                if (1 >= lo_cut && 1 < hi_cut) keep_x |= 0xffff0000u;
+                if (2 >= lo_cut && 2 < hi_cut) keep_y |= 0x0000ffffu;
+                if (3 >= lo_cut && 3 < hi_cut) keep_y |= 0xffff0000u;
+#pragma unroll
+                for (int i = 0; i < VCH; ++i) {
+                    const int d = tid / KG + i * (PF_THREADS / KG);
+                    if (d < D) {
+                        u32x2 v = vreg[i];
                         v.x &= keep_x;
                         v.y &= keep_y;
+                        *reinterpret_cast<u32x2*>(&Vs[d * V_LD + 4 * kg]) = v;
                     }
-                    *reinterpret_cast<u32x2*>(&Vs[d * V_LD + 4 * kg]) = v;
                 }
             }
+        }
+    };
+
+    // ---- DIRECT: the loads of a step, and the repair of a step at the sequence's or window's edge
+    // Instruction i of wave w fills rows 4 (4 i + w) .. + 3 of the key tile (a lane: row lane / 16,
+    // unit lane % 16) and rows 8 (4 i + w) .. + 7 of the value tile (row lane / 8, unit lane % 8).
+    // Key row r holds key 32 (r / 32) + 8 (r % 16 / 4) + 4 (r / 16 % 2) + r % 4 of the step (see
+    // stage_store): an instruction's four rows are four consecutive keys of one page, whose id is
+    // the same for the wave.  A lane's value unit is the same in all four instructions.
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    int d_kpage[4] = {0, 0, 0, 0}, d_kin[4] = {0, 0, 0, 0};  // wave-uniform: page id, first key's place in it
+    int d_vpage = 0, d_vin = 0;
+    const int d_vunit = (lane & 7) ^ ((4 * wave + (lane >> 4)) & 7);  // keys 8 d_vunit .. + 7 of the step
+    auto direct_pages = [&](int base) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 4 * (4 * i + wave_u);
+            const int key = min(base + 32 * (r >> 5) + 8 * ((r & 15) >> 2) + 4 * ((r >> 4) & 1), (seq_end - 1) & ~3);
+            const int pg = (int)__umulhi((unsigned)key, page_magic);
+            d_kpage[i] = table[pg];
+            d_kin[i] = key - pg * page_size;
+        }
+        const int key = min(base + 8 * d_vunit, (seq_end - 1) & ~7);
+        const int pg = (int)__umulhi((unsigned)key, page_magic);
+        d_vpage = table[pg];
+        d_vin = key - pg * page_size;
+    };
+    auto direct_issue = [&](int set) {
+        unsigned char* kt = dtiles + set * PF_DIRECT_SET;
+        unsigned char* vt = kt + PF_DIRECT_TILE;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 4 * (4 * i + wave_u) + (lane >> 4);  // this lane's row
+            const bf16_t* src = k_cache + ((unsigned long long)(unsigned)d_kpage[i] * page_elems +
+                                           (head_off + (unsigned)(d_kin[i] + (lane >> 4)) * (unsigned)D)) +
+                                8 * ((lane & 15) ^ (r & 15));
+            __builtin_amdgcn_global_load_lds((rl_global_ptr)src, (rl_lds_ptr)(kt + 1024 * (4 * i + wave_u)), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int d = 8 * (4 * i + wave_u) + (lane >> 3);
+            const bf16_t* src = v_cache + ((unsigned long long)(unsigned)d_vpage * page_elems +
+                                           (head_off + (unsigned)d * (unsigned)page_size + (unsigned)d_vin));
+            __builtin_amdgcn_global_load_lds((rl_global_ptr)src, (rl_lds_ptr)(vt + 1024 * (4 * i + wave_u)), 16, 0, 0);
+        }
+    };
+    // values of keys that no row may see (never written, or behind every row's window: their
+    // pages may hold anything) are zeroed where they lie: each lane repairs what it asked for
+    auto direct_repair = [&](int set, int base) {
+        unsigned char* vt = dtiles + set * PF_DIRECT_SET + PF_DIRECT_TILE;
+        const int key0 = base + 8 * d_vunit;
+        unsigned keep[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            keep[j] = 0;
+            if (key0 + 2 * j >= tile_kstart && key0 + 2 * j < seq_end) keep[j] |= 0x0000ffffu;
+            if (key0 + 2 * j + 1 >= tile_kstart && key0 + 2 * j + 1 < seq_end) keep[j] |= 0xffff0000u;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint4* at = reinterpret_cast<uint4*>(vt + 1024 * (4 * i + wave_u) + 16 * lane);
+            uint4 v = *at;
+            v.x &= keep[0];
+            v.y &= keep[1];
+            v.z &= keep[2];
+            v.w &= keep[3];
+            *at = v;
         }
     };
 
@@ -819,9 +916,15 @@ attn_prefill_kernel(
     }
     constexpr int STRIDE = GROUPS * PF_KEYS;  // the groups advance together
     if (first_base + grp * PF_KEYS < run_end) {
-        stage_pages(first_base + grp * PF_KEYS);
-        stage_load();
-        if (first_base + grp * PF_KEYS + STRIDE < run_end) stage_pages(first_base + grp * PF_KEYS + STRIDE);
+        if constexpr (DIRECT) {
+            direct_pages(first_base + grp * PF_KEYS);
+            direct_issue(0);
+            if (first_base + grp * PF_KEYS + STRIDE < run_end) direct_pages(first_base + grp * PF_KEYS + STRIDE);
+        } else {
+            stage_pages(first_base + grp * PF_KEYS);
+            stage_load();
+            if (first_base + grp * PF_KEYS + STRIDE < run_end) stage_pages(first_base + grp * PF_KEYS + STRIDE);
+        }
     }
     // q has arrived before the loop starts: inside it, waiting for q would mean waiting for
     // everything asked for since, the next step's keys and values included
@@ -829,17 +932,31 @@ attn_prefill_kernel(
     for (int n = 0; n < PF_NQ; ++n)
 #pragma unroll
         for (int c = 0; c < DC; ++c) asm volatile("" : "+v"(qf[n][c]));
-    for (int both = first_base; both < run_end; both += STRIDE) {
+    int set = 0;  // DIRECT: the set of tiles this step reads
+    for (int both = first_base; both < run_end; both += STRIDE, set ^= 1) {
         const int base = both + grp * PF_KEYS;  // this group's step
         const bool live = base < run_end;       // group 1 may have no last step
-        __syncthreads();  // the previous tile has been consumed
-        if (live) stage_store(base);
-        __syncthreads();
-        if (base + STRIDE < run_end) {
-            stage_load();  // of the step whose page ids were asked for a step ago
-            if (base + 2 * STRIDE < run_end) stage_pages(base + 2 * STRIDE);
+        if constexpr (DIRECT) {
+            // what this wave asked for has arrived in LDS (such loads count as loads from memory)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (live && (base < tile_kstart || base + PF_KEYS > seq_end)) direct_repair(set, base);
+            __syncthreads();  // every wave's share is there, and the other set has been consumed
+            if (base + STRIDE < run_end) {
+                direct_issue(set ^ 1);  // of the step whose page ids were asked for a step ago
+                if (base + 2 * STRIDE < run_end) direct_pages(base + 2 * STRIDE);
+            }
+        } else {
+            __syncthreads();  // the previous tile has been consumed
+            if (live) stage_store(base);
+            __syncthreads();
+            if (base + STRIDE < run_end) {
+                stage_load();  // of the step whose page ids were asked for a step ago
+                if (base + 2 * STRIDE < run_end) stage_pages(base + 2 * STRIDE);
+            }
         }
         if (!live || base > wave_max_pos) continue;  // no key of the step is visible to this wave's rows
+        const unsigned char* const kt = dtiles + set * PF_DIRECT_SET;
+        const unsigned char* const vt = kt + PF_DIRECT_TILE;
         // masks are needed where the diagonal or a window's edge crosses the tile
         const bool need_mask =
             (base + PF_KEYS - 1 > wave_min_pos) || (window > 0 && base < wave_max_pos - window + 1);
@@ -854,7 +971,10 @@ attn_prefill_kernel(
 #pragma unroll
             for (int c = 0; c < DC; ++c) {
                 const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
-                kf[c] = chan_ok ? load16(&Ks[krow * K_LD + 32 * c + 8 * g]) : zero8();
+                if constexpr (DIRECT)
+                    kf[c] = *reinterpret_cast<const bf16x8*>(kt + krow * (2 * D) + 16 * ((4 * c + g) ^ col));
+                else
+                    kf[c] = chan_ok ? load16(&Ks[krow * K_LD + 32 * c + 8 * g]) : zero8();
             }
 #pragma unroll
             for (int n = 0; n < PF_NQ; ++n) {
@@ -926,7 +1046,12 @@ attn_prefill_kernel(
         for (int hf = 0; hf < 2; ++hf) {
 #pragma unroll
             for (int b = 0; b < DB; ++b) {
-                const bf16x8 v = load16(&Vs[(16 * b + col) * V_LD + 32 * hf + 8 * g]);
+                bf16x8 v;
+                if constexpr (DIRECT)
+                    v = *reinterpret_cast<const bf16x8*>(vt + (16 * b + col) * (2 * PF_KEYS) +
+                                                         16 * ((4 * hf + g) ^ ((col >> 1) & 7)));
+                else
+                    v = load16(&Vs[(16 * b + col) * V_LD + 32 * hf + 8 * g]);
 #pragma unroll
                 for (int n = 0; n < PF_NQ; ++n) acc[n][b] = mfma(v, p[n][hf], acc[n][b]);
             }
@@ -937,8 +1062,7 @@ attn_prefill_kernel(
         // [wave][j][lane]; group 0 folds it into its own
         float* fold_acc = reinterpret_cast<float*>(tiles);
         constexpr int PER_LANE = PF_NQ * DB * 4;
-        static_assert(GROUPS == 1 ||
-                          sizeof(float) * PF_WAVES * PER_LANE * RL_WAVE <= sizeof(bf16_t) * GROUPS * PF_TILE_ELEMS,
+        static_assert(GROUPS == 1 || sizeof(float) * PF_WAVES * PER_LANE * RL_WAVE <= sizeof(tiles),
                       "the accumulators of one group fit where the tiles were");
         __syncthreads();  // every wave has read its last tile
         if (grp == 1) {
@@ -1029,8 +1153,14 @@ extern "C" int rl_attn_prefill(const void* q, const void* k_cache, const void* v
     const float scale_log2 = scale * 1.4426950408889634f;
     const unsigned page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     if ((long)num_tiles * nkv * nsplit > 0x7fffffffL) return RL_ERR_ARG;
+    // the kernel's addresses are page id x elements of a page (32 bits) + an offset in the page
+    if ((long)nkv * page_size * D > 0x7fffffffL) return RL_ERR_ARG;
     dim3 grid(num_tiles * nkv * nsplit), block(groups * PF_THREADS);
-    auto kernel = groups == 2 ? attn_prefill_kernel<2> : attn_prefill_kernel<1>;
+    auto kernel = groups == 2 ? attn_prefill_kernel<2, false> : attn_prefill_kernel<1, false>;
+    if constexpr (PF_DIRECT_OK) {
+        if (page_size % 8 == 0)
+            kernel = groups == 2 ? attn_prefill_kernel<2, true> : attn_prefill_kernel<1, true>;
+    }
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache,
                        (const bf16_t*)v_cache, (bf16_t*)out, tile_info, work_order, token_slot,
                        block_table, table_stride, page_size, page_magic, nq, nkv, window, scale_log2,

@@ -212,6 +212,13 @@ PREFILL_SHAPE_CASES = [
     (6, 2, 48, 4, 70, [(0, 300), (500, 40)]),              # a window: steps before it are never read
     (4, 4, 256, 32, 0, [(40, 100)]),                       # the largest tiles in LDS
     (5, 5, 16, 4, 0, [(0, 77), (90, 2)]),                  # the smallest
+    # head size 128 with pages of a multiple of eight keys: tiles loaded straight into LDS, two
+    # sets in turn; a window (the first and last steps of a tile are repaired in LDS), and
+    # pages of four and twelve keys, which keep to the tiles staged through registers
+    (8, 2, 128, 16, 150, [(0, 333), (900, 100), (40, 2)]),
+    (4, 4, 128, 8, 0, [(0, 129), (260, 70)]),
+    (8, 4, 128, 4, 0, [(100, 90), (0, 3)]),
+    (6, 2, 128, 12, 50, [(30, 200)]),
 ]
 
 
@@ -379,6 +386,34 @@ def test_attention_window_edge():
                 torch.testing.assert_close(out.cpu(), want, rtol=1e-5, atol=2e-6)
             else:
                 _close_bf16_attention(out.float().cpu(), want, seqs, "window edge")
+
+
+@pytest.mark.parametrize("page", [16, 4], ids=["p16", "p4"])
+def test_prefill_attention_reads_nothing_usable_behind_the_window(page):
+    """Pages that lie wholly behind the window of a portion's first token have been given back:
+    here they hold NaN, keys and values, and so does everything after the last token.  The
+    tiles' first and last steps still touch them; nothing of it may reach a product."""
+    ops = _ops()
+    nq, nkv, d, window = 8, 2, 128, 100
+    seqs = [(700, 150), (90, 40), (0, 260)]
+    q, kc, vc, table, ctx, want = _paged_problem(seqs, nq, nkv, d, page, torch.bfloat16, seed=11, window=window)
+    slot_of = {}
+    for tok, slot in enumerate(ctx.token_slot.tolist()):
+        slot_of.setdefault(slot, ctx.positions[tok].item())  # the portion's first position
+    host_table = table.cpu()
+    poisoned = 0
+    for slot, first in slot_of.items():
+        gone = max(0, first - window + 1) // page  # pages whose every key is out of every row's window
+        for pid in host_table[slot, :gone].tolist():
+            kc[pid] = float("nan")
+            vc[pid] = float("nan")
+            poisoned += 1
+    assert poisoned > 10
+    out = torch.full_like(q, float("nan"))
+    ops.paged_attention(q, kc, vc, out, ctx, table, page, nq, nkv, d, window, 1.0 / math.sqrt(d))
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    _close_bf16_attention(got, want, seqs, "behind the window")
 
 
 # --------------------------------------------------------------------------- #
