@@ -194,9 +194,9 @@ __device__ inline void decode_load(DecodeFrags& f, const bf16_t* k_cache, const 
     }
 }
 
-// What the fused variant needs beside the attention's own operands: the per-head norm
-// weights (null: no norm), the rotation tables (null: no rotation), and whether this layer
-// writes its keys and values.
+// What the kernels need to finish a head themselves: the per-head norm weights (null: no
+// norm), the rotation tables (null: no rotation), where the token's own key and value go (the
+// decode kernel; null: this layer writes no cache).
 struct DecodeExtra {
     const float* q_norm_w;
     const float* k_norm_w;
@@ -207,6 +207,50 @@ struct DecodeExtra {
     float eps;
     int qkv_stride;  // elements between the rows of `q` (fused: the packed q|k|v row)
 };
+
+// Q^T as the B operand of one row (lane (col, g) holds channels 32 c + 8 g .. + 7 of its row) from
+// the raw head in the packed row: norm over the head, then the rotation of channel i with
+// i + D / 2 by the position's angle (rapid_llm/models/base.py:134-140), in float32, rounded to
+// bfloat16 once.  Needs D % 64 == 0: a lane then holds both channels of every pair.
+__device__ inline void prepared_query(bf16x8 (&qf)[DC], const bf16_t* qrow, bool row_ok, int pos, int g,
+                                      const DecodeExtra& ex) {
+    float x[DC][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+        const bf16x8 raw = row_ok ? load16(qrow + 32 * c + 8 * g) : zero8();
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            x[c][j] = (float)raw[j];
+            ss += x[c][j] * x[c][j];
+        }
+    }
+    if (ex.q_norm_w) {
+        const float rrms = rsqrtf(row_sum4(ss) / (float)D + ex.eps);
+#pragma unroll
+        for (int c = 0; c < DC; ++c)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) x[c][j] *= rrms * ex.q_norm_w[32 * c + 8 * g + j];
+    }
+    if (ex.cos_tab) {
+        constexpr int HC = DC / 2;  // chunk c pairs with chunk c + HC, same lane and slot
+#pragma unroll
+        for (int c = 0; c < HC; ++c)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int i = 32 * c + 8 * g + j;
+                const float cs = ex.cos_tab[(size_t)pos * (D / 2) + i];
+                const float sn = ex.sin_tab[(size_t)pos * (D / 2) + i];
+                const float a = x[c][j], bb = x[c + HC][j];
+                x[c][j] = a * cs - bb * sn;
+                x[c + HC][j] = bb * cs + a * sn;
+            }
+    }
+#pragma unroll
+    for (int c = 0; c < DC; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[c][j] = (__bf16)x[c][j];
+}
 
 // k_cache and v_cache carry no promise of being the only way to their memory: in the fused
 // form the token's own key and value are stored through ex.k_write / ex.v_write, which point
@@ -289,42 +333,7 @@ __global__ __launch_bounds__(DEC_WAVES* RL_WAVE) void attn_decode_kernel(
         // Q^T as B operand: lane (row col, group g) holds channels 32c + 8g .. + 7
         bf16x8 qf[DC];
         if (FUSED) {
-            float x[DC][8];
-            float ss = 0.f;
-#pragma unroll
-            for (int c = 0; c < DC; ++c) {
-                const bf16x8 raw = head_ok ? load16(qrow + 32 * c + 8 * g) : zero8();
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    x[c][j] = (float)raw[j];
-                    ss += x[c][j] * x[c][j];
-                }
-            }
-            if (ex.q_norm_w) {
-                const float rrms = rsqrtf(row_sum4(ss) / (float)D + ex.eps);
-#pragma unroll
-                for (int c = 0; c < DC; ++c)
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) x[c][j] *= rrms * ex.q_norm_w[32 * c + 8 * g + j];
-            }
-            if (ex.cos_tab) {
-                constexpr int HC = DC / 2;  // chunk c pairs with chunk c + HC, same lane and slot
-#pragma unroll
-                for (int c = 0; c < HC; ++c)
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const int i = 32 * c + 8 * g + j;
-                        const float cs = ex.cos_tab[(size_t)pos * (D / 2) + i];
-                        const float sn = ex.sin_tab[(size_t)pos * (D / 2) + i];
-                        const float a = x[c][j], bb = x[c + HC][j];
-                        x[c][j] = a * cs - bb * sn;
-                        x[c + HC][j] = bb * cs + a * sn;
-                    }
-            }
-#pragma unroll
-            for (int c = 0; c < DC; ++c)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) qf[c][j] = (__bf16)x[c][j];
+            prepared_query(qf, qrow, head_ok, pos, g, ex);
             // the token's own key and value: written by the split that holds its position
             // (with more than 16 heads on a kv head every chunk of heads writes the same bytes:
             // each reads them back after its own barrier only)
@@ -673,7 +682,7 @@ attn_prefill_kernel(
     const int* __restrict__ tile_info, const int* __restrict__ work_order,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, unsigned page_magic, int nq, int nkv, int window, float scale_log2, int nsplit,
-    float* __restrict__ part_o, float* __restrict__ part_ml) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int prep_q, DecodeExtra ex) {
     constexpr int GROUP_ELEMS = DIRECT ? PF_DIRECT_GROUP / 2 : PF_TILE_ELEMS;  // bfloat16 elements
     __shared__ __attribute__((aligned(1024))) bf16_t tiles[GROUPS * GROUP_ELEMS];
     __shared__ float fold_ml[GROUPS > 1 ? PF_WAVES * PF_NQ * 2 * RL_WAVE : 1];
@@ -717,13 +726,26 @@ attn_prefill_kernel(
         r_tok[n] = tok0 + rr / G;
         r_head[n] = hk * G + rr % G;
         r_pos[n] = start + rr / G;
-        const bf16_t* qrow = q + ((size_t)r_tok[n] * nq + r_head[n]) * D;
-#pragma unroll
-        for (int c = 0; c < DC; ++c) {
-            const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
-            qf[n][c] = (r_ok[n] && chan_ok) ? load16(qrow + 32 * c + 8 * g) : zero8();
-        }
     }
+    // prep_q: `q` holds the raw packed [q | k | v] rows, and the workgroup norms and rotates its
+    // rows' heads itself, as the decode kernel does (the host asks for it only where
+    // D % 64 == 0); else `q` holds finished queries.  Called once the first tile has been asked
+    // for: finishing a query waits for its channels, and the tile travels meanwhile.
+    auto load_queries = [&]() {
+#pragma unroll
+        for (int n = 0; n < PF_NQ; ++n) {
+            const bf16_t* qrow = q + (size_t)r_tok[n] * ex.qkv_stride + (size_t)r_head[n] * D;
+            if (prep_q) {
+                prepared_query(qf[n], qrow, r_ok[n], r_pos[n], g, ex);
+            } else {
+#pragma unroll
+                for (int c = 0; c < DC; ++c) {
+                    const bool chan_ok = !(D_TAIL && c == DC - 1 && g >= 2);
+                    qf[n][c] = (r_ok[n] && chan_ok) ? load16(qrow + 32 * c + 8 * g) : zero8();
+                }
+            }
+        }
+    };
     // keys the tile needs: up to the position of its last row; from the window of its first
     const int last_row = min(row0 + PF_ROWS, rows) - 1;
     const int tile_kend = start + last_row / G + 1;
@@ -926,6 +948,7 @@ attn_prefill_kernel(
             if (first_base + grp * PF_KEYS + STRIDE < run_end) stage_pages(first_base + grp * PF_KEYS + STRIDE);
         }
     }
+    load_queries();
     // q has arrived before the loop starts: inside it, waiting for q would mean waiting for
     // everything asked for since, the next step's keys and values included
 #pragma unroll
@@ -1137,19 +1160,31 @@ extern "C" int rl_attn_prefill_rows() { return PF_ROWS; }
 // nsplit > 1 cuts every tile's keys into that many runs (for launches of few, long tiles);
 // part_o [tokens of the step, nq, nsplit, D] and part_ml [.., 2] then hold the runs' results
 // and prefill_tokens [num_prefill_tokens] names the tokens the merge kernel writes.
+// prep_q != 0: `q` is the packed [q | k | v] row of every token; the kernel norms (q_norm_w, eps;
+// null: no norm) and rotates (cos_tab, sin_tab; null: no rotation) the query heads it reads.
 extern "C" int rl_attn_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                                const int* tile_info, const int* work_order, int num_tiles,
                                const int* token_slot,
                                const int* block_table, int table_stride, int page_size, int nq,
                                int nkv, int window, float scale, int groups, int nsplit, float* part_o,
                                float* part_ml, const int* prefill_tokens, int num_prefill_tokens,
-                               hipStream_t stream) {
+                               int prep_q, const float* q_norm_w, const float* cos_tab,
+                               const float* sin_tab, float eps, hipStream_t stream) {
     if (num_tiles <= 0) return RL_OK;
     if (nkv < 1 || nq % nkv || page_size < 4 || page_size % 4 || nkv > 65535 || nsplit < 1 ||
         (groups != 1 && groups != 2))
         return RL_ERR_ARG;
     if (nsplit > 1 && (!part_o || !part_ml || !prefill_tokens || num_prefill_tokens < 1 || nq > 65535))
         return RL_ERR_ARG;
+    if (prep_q && (D % 64 != 0 || (cos_tab && !sin_tab))) return RL_ERR_ARG;
+    DecodeExtra ex;
+    ex.q_norm_w = prep_q ? q_norm_w : nullptr;
+    ex.k_norm_w = nullptr;
+    ex.cos_tab = prep_q ? cos_tab : nullptr;
+    ex.sin_tab = prep_q ? sin_tab : nullptr;
+    ex.k_write = ex.v_write = nullptr;
+    ex.eps = eps;
+    ex.qkv_stride = prep_q ? (nq + 2 * nkv) * D : nq * D;
     const float scale_log2 = scale * 1.4426950408889634f;
     const unsigned page_magic = (unsigned)(((1ull << 32) + page_size - 1) / page_size);
     if ((long)num_tiles * nkv * nsplit > 0x7fffffffL) return RL_ERR_ARG;
@@ -1164,7 +1199,7 @@ extern "C" int rl_attn_prefill(const void* q, const void* k_cache, const void* v
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache,
                        (const bf16_t*)v_cache, (bf16_t*)out, tile_info, work_order, token_slot,
                        block_table, table_stride, page_size, page_magic, nq, nkv, window, scale_log2,
-                       nsplit, part_o, part_ml);
+                       nsplit, part_o, part_ml, prep_q ? 1 : 0, ex);
     if (hipGetLastError() != hipSuccess) return RL_ERR_LAUNCH;
     if (nsplit > 1)
         hipLaunchKernelGGL(attn_merge_kernel, dim3(num_prefill_tokens, nq), dim3(D < 64 ? 64 : D), 0,

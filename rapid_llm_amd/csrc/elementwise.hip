@@ -465,7 +465,7 @@ __global__ void qknorm_rope_kvwrite_kernel(
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
     int page_size, int nq, int nkv, int d, int rotary_half, int interleaved, float eps,
-    int write_cache, int write_values) {
+    int write_cache, int write_values, int head0) {
     const int t = blockIdx.x;
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -482,7 +482,9 @@ __global__ void qknorm_rope_kvwrite_kernel(
         off = pos % page_size;
     }
 
-    for (int head = blockIdx.y * nwaves + wave; head < total_heads; head += nwaves * gridDim.y) {
+    // head0: the first head to work on (the number of query heads where the attention kernels
+    // finish the queries themselves)
+    for (int head = head0 + blockIdx.y * nwaves + wave; head < total_heads; head += nwaves * gridDim.y) {
         const T* x = row + (size_t)head * d;
         if (head >= nq + nkv) {
             // value head: copy into the transposed page (unless the tile kernel below does it)
@@ -559,7 +561,7 @@ __device__ inline void qknorm_rope_kvwrite_vec(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values) {
+    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0) {
     constexpr int HPW = RL_WAVE / LPH;  // heads per wave
     const int lane = threadIdx.x & (RL_WAVE - 1);
     const int wave = threadIdx.x / RL_WAVE;
@@ -575,7 +577,7 @@ __device__ inline void qknorm_rope_kvwrite_vec(
         page = (size_t)block_table[(size_t)token_slot[t] * table_stride + pos / page_size];
         off = pos % page_size;
     }
-    const int head = (head_group * (blockDim.x / RL_WAVE) + wave) * HPW + sub;
+    const int head = head0 + (head_group * (blockDim.x / RL_WAVE) + wave) * HPW + sub;
     if (head >= total_heads) return;  // whole groups of LPH lanes leave together
     const T* x = row + (size_t)head * d;
     const bool active = 4 * li < half;
@@ -644,10 +646,10 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_vec_kernel(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values) {
+    int page_size, int nq, int nkv, int d, float eps, int write_cache, int write_values, int head0) {
     qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x, blockIdx.y, qkv, q_out, k_cache, v_cache, q_norm_w, k_norm_w,
                                     cos_tab, sin_tab, positions, token_slot, block_table, table_stride,
-                                    page_size, nq, nkv, d, eps, write_cache, write_values);
+                                    page_size, nq, nkv, d, eps, write_cache, write_values, head0);
 }
 
 template <typename T>
@@ -656,8 +658,8 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
                           const int* positions, const int* token_slot, const int* block_table,
                           int table_stride, int page_size, int tokens, int nq, int nkv, int d,
                           int rotary_half, int interleaved, float eps, int write_cache,
-                          int write_values, hipStream_t stream) {
-    const int total_heads = nq + (write_values ? 2 * nkv : nkv);
+                          int write_values, int head0, hipStream_t stream) {
+    const int total_heads = nq + (write_values ? 2 * nkv : nkv) - head0;  // heads to work on
     // the vectorised kernel: head sizes in steps of 8, the half-split rotation of the whole head
     if (d % 8 == 0 && (!cos_tab || (rotary_half == d / 2 && !interleaved))) {
         const int lph = d <= 128 ? 16 : 32;
@@ -668,12 +670,12 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
             hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 16>), grid, block, 0, stream, qkv,
                                q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
                                positions, token_slot, block_table, table_stride, page_size, nq, nkv,
-                               d, eps, write_cache, write_values);
+                               d, eps, write_cache, write_values, head0);
         else
             hipLaunchKernelGGL((qknorm_rope_kvwrite_vec_kernel<T, 32>), grid, block, 0, stream, qkv,
                                q_out, k_cache, v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab,
                                positions, token_slot, block_table, table_stride, page_size, nq, nkv,
-                               d, eps, write_cache, write_values);
+                               d, eps, write_cache, write_values, head0);
         return;
     }
     const int head_groups = (total_heads + 3) / 4;
@@ -681,7 +683,7 @@ static void launch_qknorm(const T* qkv, T* q_out, T* k_cache, T* v_cache, const 
     hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, grid, block, 0, stream, qkv, q_out, k_cache,
                        v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                        block_table, table_stride, page_size, nq, nkv, d, rotary_half, interleaved, eps,
-                       write_cache, write_values);
+                       write_cache, write_values, head0);
 }
 
 // Values of 16 consecutive tokens of the batch and one kv head, written by one workgroup.
@@ -754,12 +756,12 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_tab,
     const float* __restrict__ sin_tab, const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ block_table, int table_stride,
-    int page_size, int tokens, int head_groups, int nq, int nkv, int d, float eps) {
+    int page_size, int tokens, int head_groups, int nq, int nkv, int d, float eps, int head0) {
     const int qk_blocks = tokens * head_groups;
     if ((int)blockIdx.x < qk_blocks) {
         qknorm_rope_kvwrite_vec<T, LPH>(blockIdx.x / head_groups, blockIdx.x % head_groups, qkv, q_out, k_cache,
                                         v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
-                                        block_table, table_stride, page_size, nq, nkv, d, eps, 1, 0);
+                                        block_table, table_stride, page_size, nq, nkv, d, eps, 1, 0, head0);
     } else {
         const int b = blockIdx.x - qk_blocks;
         v_tile_write<T>(b / nkv, b % nkv, qkv, v_cache, positions, token_slot, block_table, table_stride,
@@ -782,22 +784,22 @@ static bool launch_qkv_prepare(const T* qkv, T* q_out, T* k_cache, T* v_cache, c
                                const float* k_norm_w, const float* cos_tab, const float* sin_tab,
                                const int* positions, const int* token_slot, const int* block_table,
                                int table_stride, int page_size, int tokens, int nq, int nkv, int d,
-                               float eps, hipStream_t stream) {
+                               float eps, int head0, hipStream_t stream) {
     if (d % 8) return false;
     const int lph = d <= 128 ? 16 : 32;
     const int heads_per_block = 4 * (RL_WAVE / lph);
-    const int head_groups = (nq + nkv + heads_per_block - 1) / heads_per_block;
+    const int head_groups = (nq + nkv - head0 + heads_per_block - 1) / heads_per_block;
     const long blocks = (long)tokens * head_groups + (long)((tokens + VT_TOKENS - 1) / VT_TOKENS) * nkv;
     if (blocks > 0x7fffffffL) return false;
     dim3 grid((unsigned)blocks), block(256);
     if (lph == 16)
         hipLaunchKernelGGL((qkv_prepare_kernel<T, 16>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
                            q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps);
+                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0);
     else
         hipLaunchKernelGGL((qkv_prepare_kernel<T, 32>), grid, block, 0, stream, qkv, q_out, k_cache, v_cache,
                            q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps);
+                           table_stride, page_size, tokens, head_groups, nq, nkv, d, eps, head0);
     return true;
 }
 
@@ -811,6 +813,10 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
                                       hipStream_t stream) {
     if (tokens <= 0) return RL_OK;
     if (d % 2 || d > 256) return RL_ERR_ARG;
+    // q_out null: the attention kernels finish the query heads themselves, and the work here
+    // starts at the first key head
+    const int head0 = q_out ? 0 : nq;
+    if (!q_out && !write_cache) return RL_OK;  // nothing to write at all
     // the first 2 * rotary_half channels of a head rotate: at least one pair, at most all
     if (cos_tab && (rotary_half < 1 || rotary_half > d / 2)) return RL_ERR_ARG;
     const bool whole_split = !cos_tab || (rotary_half == d / 2 && !interleaved);
@@ -823,18 +829,18 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
     if (tile_values && whole_split && act_type == RL_F32 &&
         launch_qkv_prepare<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache, q_norm_w,
                                   k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                                  table_stride, page_size, tokens, nq, nkv, d, eps, stream))
+                                  table_stride, page_size, tokens, nq, nkv, d, eps, head0, stream))
         return rl_launch_status();
     if (tile_values && whole_split && act_type == RL_BF16 &&
         launch_qkv_prepare<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache,
                                    q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot, block_table,
-                                   table_stride, page_size, tokens, nq, nkv, d, eps, stream))
+                                   table_stride, page_size, tokens, nq, nkv, d, eps, head0, stream))
         return rl_launch_status();
     if (act_type == RL_F32) {
         launch_qknorm<float>((const float*)qkv, (float*)q_out, (float*)k_cache, (float*)v_cache,
                              q_norm_w, k_norm_w, cos_tab, sin_tab, positions, token_slot,
                              block_table, table_stride, page_size, tokens, nq, nkv, d, rotary_half,
-                             interleaved, eps, write_cache, !tile_values, stream);
+                             interleaved, eps, write_cache, !tile_values, head0, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, block, 0, stream,
                                (const float*)qkv, (float*)v_cache, positions, token_slot,
@@ -843,7 +849,7 @@ extern "C" int rl_qknorm_rope_kvwrite(const void* qkv, void* q_out, void* k_cach
         launch_qknorm<bf16_t>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
                               (bf16_t*)v_cache, q_norm_w, k_norm_w, cos_tab, sin_tab, positions,
                               token_slot, block_table, table_stride, page_size, tokens, nq, nkv, d,
-                              rotary_half, interleaved, eps, write_cache, !tile_values, stream);
+                              rotary_half, interleaved, eps, write_cache, !tile_values, head0, stream);
         if (tile_values)
             hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, block, 0, stream,
                                (const bf16_t*)qkv, (bf16_t*)v_cache, positions, token_slot,

@@ -228,7 +228,7 @@ ROTARY_PAIRINGS = {"half_split": 0, "interleaved": 1}
 
 def qknorm_rope_kvwrite(
     qkv: torch.Tensor,
-    q_out: torch.Tensor,
+    q_out: Optional[torch.Tensor],
     k_cache: Optional[torch.Tensor],
     v_cache: Optional[torch.Tensor],
     q_norm_w: Optional[torch.Tensor],
@@ -247,7 +247,9 @@ def qknorm_rope_kvwrite(
     pairing: str = "half_split",
 ) -> None:
     """Norm + rotate q and k, write k and v to the cache pages (skipped when the caches
-    are ``None``: a layer that reads another layer's cache).  ``max_position`` is the
+    are ``None``: a layer that reads another layer's cache).  ``q_out`` ``None``: the query
+    heads are left as they are (the attention kernels finish them themselves, see
+    :func:`attention_prepares_queries`).  ``max_position`` is the
     largest position in the batch, checked against the rotation table and block table.
     The tables' width says how many channels rotate (``2 * cos.shape[1]``, the first of a
     head), ``pairing`` which of them form a pair (:data:`ROTARY_PAIRINGS`)."""
@@ -255,7 +257,8 @@ def qknorm_rope_kvwrite(
         raise KernelError(f"rotation pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
     tokens = qkv.shape[0]
     _need(qkv, "qkv", None, (tokens, (nq + 2 * nkv) * d))
-    _need(q_out, "q_out", qkv.dtype, (tokens, nq * d))
+    if q_out is not None:
+        _need(q_out, "q_out", qkv.dtype, (tokens, nq * d))
     _need(positions, "positions", torch.int32, (tokens,))
     _need(token_slot, "token_slot", torch.int32, (tokens,))
     _need(block_table, "block_table", torch.int32)
@@ -1037,12 +1040,19 @@ def paged_attention(
     d: int,
     window: int,
     scale: float,
+    prepare: Optional[tuple] = None,
 ) -> None:
     """Attention of every token of the step over its request's cached keys.
 
     Head sizes in steps of 16 run on the matrix cores: float32 on the float32 kernel,
     bfloat16 on the bfloat16 kernels (single tokens go to the split-key decode kernel, portions
-    to the tiled prefill kernel).  Other head sizes run the FMA kernel in either type."""
+    to the tiled prefill kernel).  Other head sizes run the FMA kernel in either type.
+
+    ``prepare`` = ``(q_norm_w, cos, sin, eps)``: ``q`` is the packed [q | k | v] row of every token,
+    and the kernels norm and rotate the query heads as they read them (only where
+    :func:`attention_prepares_queries` says so)."""
+    if prepare is not None and not attention_prepares_queries(q.dtype, d, 0 if prepare[1] is None else prepare[1].shape[1]):
+        raise KernelError("the attention kernels do not finish the queries of this head size, type or rotation")
     if q.dtype == torch.float32 and d % 16 == 0:
         attention_f32(q, k_cache, v_cache, out, ctx, block_table, page_size, nq, nkv, d, window, scale)
         return
@@ -1054,7 +1064,7 @@ def paged_attention(
         return
     tokens = q.shape[0]
     pages = k_cache.shape[0]
-    _need(q, "q", torch.bfloat16, (tokens, nq * d))
+    _need(q, "q", torch.bfloat16, (tokens, (nq * d) if prepare is None else (nq + 2 * nkv) * d))
     _need(out, "out", torch.bfloat16, (tokens, nq * d))
     _need(k_cache, "k_cache", torch.bfloat16, (pages, nkv, page_size, d))
     _need(v_cache, "v_cache", torch.bfloat16, (pages, nkv, d, page_size))
@@ -1066,6 +1076,19 @@ def paged_attention(
             f"position {ctx.max_position} needs page {ctx.max_position // page_size} of a block "
             f"table with {block_table.shape[1]} columns"
         )
+    q_norm_w = cos = sin = None
+    eps = 0.0
+    if prepare is not None:
+        q_norm_w, cos, sin, eps = prepare
+        if q_norm_w is not None:
+            _need(q_norm_w, "q_norm weight", torch.float32, (d,))
+        if cos is not None:
+            _need(cos, "cos table", torch.float32, (None, d // 2))
+            _need(sin, "sin table", torch.float32, tuple(cos.shape))
+            if ctx.max_position >= cos.shape[0]:
+                raise KernelError(
+                    f"position {ctx.max_position} is beyond the rotation table of {cos.shape[0]} positions"
+                )
     if ctx.max_position >= (1 << 32) // page_size:
         # the prefill kernel divides positions by the page size with one multiplication
         raise KernelError(f"position {ctx.max_position} is too large for pages of {page_size} tokens")
@@ -1085,13 +1108,25 @@ def paged_attention(
                 _p(plan.work_order(nkv, q.device, 2 // groups)), plan.num_tiles,
                 _p(ctx.token_slot), _p(block_table), block_table.stride(0), page_size, nq, nkv,
                 window, ctypes.c_float(scale), groups, nsplit, _p(part_o), _p(part_ml), _p(tokens_list),
-                0 if tokens_list is None else tokens_list.numel(), _stream(),
+                0 if tokens_list is None else tokens_list.numel(),
+                int(prepare is not None), _p(q_norm_w), _p(cos), _p(sin), ctypes.c_float(eps), _stream(),
             ),
             "rl_attn_prefill",
         )
     if plan.num_decode:
+        # single tokens beside portions: their keys and values are in the cache already
+        fused = None if prepare is None else (q_norm_w, None, cos, sin, None, None, eps)
         _decode_launch(lib, plan, ctx, q, k_cache, v_cache, out, block_table, page_size, nq, nkv, d,
-                       window, scale, None)
+                       window, scale, fused)
+
+
+def attention_prepares_queries(x_dtype: torch.dtype, d: int, rotary_half: int, pairing: str = "half_split") -> bool:
+    """Whether the bfloat16 attention kernels can norm and rotate the query heads themselves, from
+    the packed rows: a head size whose rotation pairs stay within a lane, the half-split rotation
+    of the whole head or none."""
+    if x_dtype != torch.bfloat16 or d % 64 or rotary_half not in (0, d // 2):
+        return False
+    return not (rotary_half and pairing != "half_split")
 
 
 def attention_plan(ctx, group: int, d: int) -> AttentionPlan:
@@ -1164,9 +1199,7 @@ def decode_attention_fusable(ctx, x_dtype: torch.dtype, group: int, d: int, rota
     """Whether the step is one the fused decode kernel takes: bfloat16, single tokens only,
     a head size whose rotation pairs stay within a lane, the half-split rotation of the whole
     head or none."""
-    if x_dtype != torch.bfloat16 or d % 64 or rotary_half not in (0, d // 2):
-        return False
-    if rotary_half and pairing != "half_split":
+    if not attention_prepares_queries(x_dtype, d, rotary_half, pairing):
         return False
     plan = attention_plan(ctx, group, d)
     return plan.num_tiles == 0 and plan.num_decode > 0

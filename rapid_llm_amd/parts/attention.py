@@ -152,7 +152,10 @@ class GQAAttention(Mixer):
                 self.window, self.scale, self.q_norm_w, self.k_norm_w, cos, sin, eps, cache.owns_pages,
             )
             return self.o.deferred(out, ctx)
-        q = torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
+        # where the attention kernels can finish the query heads as they read them, only the keys
+        # and values are prepared here, and the queries are never written out
+        in_kernel = ops.attention_prepares_queries(qkv.dtype, self.d, rotary_half, pairing)
+        q = None if in_kernel else torch.empty((tokens, self.nq * self.d), dtype=qkv.dtype, device=x.device)
         ops.qknorm_rope_kvwrite(
             qkv, q,
             cache.k if cache.owns_pages else None,
@@ -162,8 +165,9 @@ class GQAAttention(Mixer):
             self.nq, self.nkv, self.d, eps, ctx.max_position, pairing,
         )
         ops.paged_attention(
-            q, cache.k, cache.v, out, ctx, table, cache.page_size,
+            qkv if in_kernel else q, cache.k, cache.v, out, ctx, table, cache.page_size,
             self.nq, self.nkv, self.d, self.window, self.scale,
+            prepare=(self.q_norm_w, cos, sin, eps) if in_kernel else None,
         )
         return self.o.deferred(out, ctx)
 

@@ -975,6 +975,99 @@ def test_embed_and_argmax():
     assert int(out[3]) == 777
 
 
+PREPARED_CASES = [
+    # nq, nkv, d, page, window, (tokens cached, tokens in the step) of every request
+    (8, 2, 128, 16, 0, [(0, 70), (300, 1), (40, 33)]),     # portions beside a single token
+    (6, 3, 64, 8, 0, [(100, 40), (5, 1), (0, 2)]),
+    (4, 4, 192, 32, 57, [(400, 3), (20, 90)]),             # window
+    (32, 8, 128, 16, 0, [(1000, 600)]),                    # few, long tiles: the keys cut into runs
+]
+
+
+@pytest.mark.parametrize("case", PREPARED_CASES, ids=lambda c: f"h{c[0]}kv{c[1]}d{c[2]}p{c[3]}w{c[4]}")
+@pytest.mark.parametrize("normed", [True, False], ids=["norm", "nonorm"])
+def test_attention_that_finishes_the_queries_itself(case, normed):
+    """A step of portions and single tokens from the packed rows: the keys and values are
+    normed, rotated and written by the head kernel (which leaves the queries alone), the
+    attention kernels norm and rotate the query heads as they read them.  Against the plain
+    formulas, and against the same step with the queries written out first."""
+    ops = _ops()
+    nq, nkv, d, page, window, seqs = case
+    theta, eps = 50000.0, 3e-6
+    gen = torch.Generator().manual_seed(d + nq + 1)
+    rng = random.Random(nq * 17 + d)
+    assert ops.attention_prepares_queries(torch.bfloat16, d, d // 2)
+    total_pages = sum(-(-(a + n) // page) for a, n in seqs) + 1
+    order = list(range(1, total_pages))
+    rng.shuffle(order)
+    max_pages = max(-(-(a + n) // page) for a, n in seqs) + 1
+    table = torch.zeros((len(seqs) + 2, max_pages), dtype=torch.int32)
+    kc = torch.full((total_pages, nkv, page, d), float("nan"))
+    vc = torch.full((total_pages, nkv, d, page), float("nan"))
+    slots = list(range(len(seqs) + 2))
+    rng.shuffle(slots)
+    qw = 1 + 0.1 * torch.randn(d, generator=gen) if normed else None
+    kw = 1 + 0.1 * torch.randn(d, generator=gen) if normed else None
+    rows, positions, token_slot, expect = [], [], [], []
+    for i, (a, n) in enumerate(seqs):
+        k_old = torch.randn(a, nkv, d, generator=gen).bfloat16().float()
+        v_old = torch.randn(a, nkv, d, generator=gen).bfloat16().float()
+        for p in range(-(-(a + n) // page)):
+            pid = order.pop()
+            table[slots[i], p] = pid
+            lo, hi = p * page, min(a, (p + 1) * page)
+            if hi > lo:
+                kc[pid, :, : hi - lo, :] = k_old[lo:hi].transpose(0, 1)
+                vc[pid, :, :, : hi - lo] = v_old[lo:hi].permute(1, 2, 0)
+        raw = torch.randn(n, (nq + 2 * nkv) * d, generator=gen).bfloat16()
+        rows.append(raw)
+        q = raw.float()[:, : nq * d].view(n, nq, d)
+        k = raw.float()[:, nq * d : (nq + nkv) * d].view(n, nkv, d)
+        v = raw.float()[:, (nq + nkv) * d :].view(n, nkv, d)
+        if normed:
+            q, k = plain_rmsnorm(q, qw, eps), plain_rmsnorm(k, kw, eps)
+        qpos = torch.arange(a, a + n)
+        pc, ps = plain_rope_tables(qpos, d, theta)
+        q, k = plain_rope_apply(q, pc, ps), plain_rope_apply(k, pc, ps)
+        q, k = q.bfloat16().float(), k.bfloat16().float()  # what the products hold
+        expect.append(
+            plain_attention(q, torch.cat([k_old, k]), torch.cat([v_old, v]), d**-0.5, window or None, qpos,
+                            torch.arange(a + n)).reshape(n, nq * d)
+        )
+        positions += list(range(a, a + n))
+        token_slot += [slots[i]] * n
+    tokens = len(positions)
+    ctx = SimpleNamespace(
+        positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+        token_slot=torch.tensor(token_slot, dtype=torch.int32, device=DEV),
+        token_ids=torch.zeros(tokens, dtype=torch.int32, device=DEV),
+        h_seq_starts=[a for a, _ in seqs], h_seq_lens=[n for _, n in seqs], max_position=max(positions), extra={},
+    )
+    cos, sin = ops.rope_table(plain_inv_freq(d, theta).to(DEV), max(positions) + 1)
+    qkv = torch.cat(rows).to(DEV)
+    tab = table.to(DEV)
+    qwd, kwd = (qw.to(DEV), kw.to(DEV)) if normed else (None, None)
+    want = torch.cat(expect)
+    outs = []
+    for in_kernel in (True, False):
+        kcd, vcd = kc.bfloat16().to(DEV), vc.bfloat16().to(DEV)
+        q_out = None if in_kernel else torch.full((tokens, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.qknorm_rope_kvwrite(qkv, q_out, kcd, vcd, qwd, kwd, cos, sin, ctx.positions, ctx.token_slot, tab, page,
+                                nq, nkv, d, eps, ctx.max_position)
+        out = torch.full((tokens, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.paged_attention(qkv if in_kernel else q_out, kcd, vcd, out, ctx, tab, page, nq, nkv, d, window, d**-0.5,
+                            prepare=(qwd, cos, sin, eps) if in_kernel else None)
+        got = out.float().cpu()
+        assert torch.isfinite(got).all()
+        _close_bf16_attention(got, want, seqs, "queries finished in the kernel" if in_kernel else "queries written out")
+        outs.append(got)
+    # the two ways round a query's channels alike but for the order of two multiplications
+    assert (outs[0] - outs[1]).abs().max() <= 0.05 * want.abs().max()
+    with pytest.raises(ops.KernelError, match="do not finish the queries"):
+        ops.paged_attention(qkv.float(), kcd.float(), vcd.float(), out.float(), ctx, tab, page, nq, nkv, d, window,
+                            d**-0.5, prepare=(qwd, cos, sin, eps))
+
+
 FUSED_CASES = [
     # nq, nkv, d, page, window, cached lengths of the requests
     (8, 2, 128, 16, 0, [0, 5, 699, 31, 256]),
