@@ -157,7 +157,7 @@ def test_logprob_records_of_prompt_and_output(tmp_path):
             assert [r and r.token_id for r in again.prompt_logprobs] == [r and r.token_id for r in out.prompt_logprobs]
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "F"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "F", "H"])
 def test_bfloat16_generation_stays_near_the_plain_choice(tmp_path, which):
     from rapid_llm_amd import SamplingParams
 

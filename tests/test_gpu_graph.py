@@ -20,7 +20,7 @@ def _runner(model_dir, dtype, page, graph):
     )
 
 
-@pytest.mark.parametrize("which", ["A", "C", "D", "F"])
+@pytest.mark.parametrize("which", ["A", "C", "D", "F", "H"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replays_match_eager(tmp_path, which, dtype):
     from rapid_llm_amd import StepEntry

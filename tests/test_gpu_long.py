@@ -41,7 +41,7 @@ def _runner(model_dir, dtype, page, max_seq_len, graph=False, num_pages=None, se
     )
 
 
-@pytest.mark.parametrize("which", ["B", "C", "D", "F", "G"])
+@pytest.mark.parametrize("which", ["B", "C", "D", "F", "G", "H"])
 @pytest.mark.parametrize("dtype,graph", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
 def test_long_decoding(tmp_path, which, dtype, graph):
     from rapid_llm_amd import StepEntry
@@ -103,7 +103,7 @@ def test_decoding_across_three_context_buckets(tmp_path):
     runner.cache.check_invariants()
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "F", "G"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "F", "G", "H"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens(tmp_path, which, dtype):
     """Positions 0, 1, 2: a one-token prompt, its first decoded tokens, a two-token prompt cut

@@ -26,6 +26,7 @@ LENGTHS = {
     "E": [20, 35, 49, 64, 90, 200],          # portions of 17 to 64 tokens take the mid-size product
     "F": [3, 31, 33, 64, 97, 180],           # page of 32: requests within one page, at its edge, across several
     "G": [6, 21, 38, 75, 120, 190],          # head size 24; the window of 37 passes whole pages of 4
+    "H": [5, 30, 65, 129, 260, 520],         # head size 128: tiles of 64 keys at, around and well beyond one and the window of 70
 }
 
 
@@ -78,7 +79,7 @@ def _check(got, want, dtype, label):
             raise AssertionError(f"{label}: request {rid}, first wrong position {first}: {exc}") from None
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F", "G"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F", "G", "H"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_every_cut_matches_plain(tmp_path, which, dtype):
     cfg, page, seed = TINY[which]

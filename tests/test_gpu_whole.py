@@ -21,7 +21,7 @@ def _runner(model_dir, dtype, page, **kw):
     return ModelRunner(model_dir, EngineConfig(**body))
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F", "G"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F", "G", "H"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_whole_prompts(tmp_path, which, dtype):
     from rapid_llm_amd import StepEntry

@@ -27,7 +27,7 @@ def _rejects(got, want, label):
         parity.assert_bf16_close(got, want, label)
 
 
-@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F", "G"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D", "E", "F", "G", "H"])
 def test_rounding_alone_passes_and_a_lost_key_does_not(tmp_path, which):
     pcfg, pw, page, seed = _model(tmp_path, which)
     n = min(pcfg["max_position_embeddings"], 200)

@@ -81,7 +81,20 @@ TINY_G = dict(
 )
 PAGE_G = 4
 
-TINY = {"A": (TINY_A, PAGE_A, 11), "B": (TINY_B, PAGE_B, 22), "C": (TINY_C, PAGE_C, 33),
+# H: head 128, the family's own: from this size on a prompt step's key and value tiles go from
+# memory straight into LDS, and the attention kernels finish the query heads' norm and rotation
+# themselves; a window on the first layer, group 2, heads * head_dim = 512 beside a width of 192
+TINY_H = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=192, num_attention_heads=4, num_key_value_heads=2,
+    head_dim=128, intermediate_size=272, vocab_size=401, rope_theta=1000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=640,
+    hidden_act="silu", attention_bias=False,
+    sliding_window=70, layer_types=["sliding_attention", "full_attention"],
+)
+PAGE_H = 16
+
+TINY = {"H": (TINY_H, PAGE_H, 88), "A": (TINY_A, PAGE_A, 11), "B": (TINY_B, PAGE_B, 22), "C": (TINY_C, PAGE_C, 33),
         "D": (TINY_D, PAGE_D, 44), "E": (TINY_E, PAGE_E, 55), "F": (TINY_F, PAGE_F, 66),
         "G": (TINY_G, PAGE_G, 77)}
 
