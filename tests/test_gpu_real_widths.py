@@ -206,14 +206,22 @@ LARGE = dict(
     rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=16384,
     hidden_act="silu", attention_bias=False,
 )
-LARGE_PROMPT = 9000
+# The same at the widths of the family's 14B model (40 query heads on 8 kv heads: groups of 5,
+# which fill five sixteenths of the attention kernels' blocks of 16 rows; intermediate 17,408,
+# whose gate/up matrix is 5.3 tiles a compute unit for the product for 17 to 64 rows), a
+# 2,600-token prompt in portions of 2,048 and 552 and graphs of the 4,096 bucket.
+GROUP5 = dict(LARGE, num_attention_heads=40, intermediate_size=17408, vocab_size=20000, max_position_embeddings=4096)
+# name -> (configuration, prompt tokens, first portion, context bucket = max_seq_len, pages)
+LARGE_CASES = {
+    "largest": (LARGE, 9000, 8192, 16384, 800),
+    "group5": (GROUP5, 2600, 2048, 4096, 400),
+}
 LARGE_STEPS = 2  # single-token steps at each batch size
 
 
-def _large_plan():
+def _large_plan(vocab, prompt_len, portion):
     """(tokens by request, steps as (label, [(request, start, count, wanted places)], graph))."""
-    vocab = LARGE["vocab_size"]
-    prompt = {"long": LARGE_PROMPT}
+    prompt = {"long": prompt_len}
     for i in range(31):
         prompt[f"s{i}"] = 2 + (i * 11) % 70
     tokens = {r: random_tokens(n + 3 * LARGE_STEPS, vocab, 2000 + k) for k, (r, n) in enumerate(prompt.items())}
@@ -225,8 +233,9 @@ def _large_plan():
         done[rid] += count
         return e
 
-    steps.append(("first portion of 8,192", [entry("long", 8192, [0, 1, 4095, 4096, 8190, 8191])], False))
-    steps.append(("second portion behind 8,192", [entry("long", LARGE_PROMPT - 8192, [0, 1, 400, 806, 807])], False))
+    rest_len = prompt_len - portion
+    steps.append(("first portion", [entry("long", portion, [0, 1, portion // 2 - 1, portion // 2, portion - 2, portion - 1])], False))
+    steps.append(("second portion behind the first", [entry("long", rest_len, [0, 1, rest_len // 2, rest_len - 2, rest_len - 1])], False))
     for i in range(LARGE_STEPS):
         steps.append((f"batch 1 step {i}", [entry("long", 1, [0])], True))
     seven = [f"s{i}" for i in range(7)]
@@ -240,14 +249,15 @@ def _large_plan():
     return tokens, steps
 
 
-@pytest.fixture(scope="module")
-def large(tmp_path_factory):
+@pytest.fixture(scope="module", params=sorted(LARGE_CASES))
+def large(request, tmp_path_factory):
     """The model folder, the plan and the plain logits at every compared position."""
     from rapid_llm_amd import write_random_model
 
-    folder = tmp_path_factory.mktemp("largest_widths") / "two_layers"
-    write_random_model(dict(LARGE), 13, folder, dtype="bfloat16", norm_std=0.1)
-    tokens, steps = _large_plan()
+    config, prompt_len, portion, bucket, pages = LARGE_CASES[request.param]
+    folder = tmp_path_factory.mktemp(f"{request.param}_widths") / "two_layers"
+    write_random_model(dict(config), 13, folder, dtype="bfloat16", norm_std=0.1)
+    tokens, steps = _large_plan(config["vocab_size"], prompt_len, portion)
     rows: dict[str, list[int]] = {r: [] for r in tokens}
     for _label, entries, _graph in steps:
         for rid, start, _count, want in entries:
@@ -258,17 +268,17 @@ def large(tmp_path_factory):
         logits = plain_forward(pcfg, pw, tokens[rid][: max(at) + 1], rows=at)
         plain[rid] = {pos: logits[i] for i, pos in enumerate(at)}
     del pw
-    return folder, tokens, steps, plain
+    return request.param, folder, tokens, steps, plain, bucket, pages
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_largest_widths_at_a_long_context_match_plain(large, dtype):
+def test_large_widths_at_a_long_context_match_plain(large, dtype):
     from rapid_llm_amd import EngineConfig, ModelRunner, StepEntry
 
-    folder, tokens, steps, plain = large
+    name, folder, tokens, steps, plain, bucket, pages = large
     runner = ModelRunner(
         folder,
-        EngineConfig(dtype=dtype, max_seq_len=16384, page_size=PAGE, num_pages=800, max_num_seqs=32, use_graph=True),
+        EngineConfig(dtype=dtype, max_seq_len=bucket, page_size=PAGE, num_pages=pages, max_num_seqs=32, use_graph=True),
     )
     for label, entries, graph in steps:
         before = set(runner._graphs)
@@ -278,15 +288,15 @@ def test_largest_widths_at_a_long_context_match_plain(large, dtype):
         want = torch.stack([plain[rid][start + w] for rid, start, count, ws in entries for w in ws])
         assert logits.shape == want.shape, label
         if graph:
-            assert (len(entries), 16384) in runner._graphs, f"{label}: no graph of the 16,384 bucket ({sorted(runner._graphs)})"
+            assert (len(entries), bucket) in runner._graphs, f"{label}: no graph of the {bucket} bucket ({sorted(runner._graphs)})"
         else:
             assert set(runner._graphs) == before, f"{label}: a step with a portion was recorded"
         if dtype == "float32":
             err = float((logits - want).abs().max())
-            print(f"largest widths float32 {label}: worst error {err:.3e} (logits spread {float(want.std()):.3f})")
+            print(f"{name} widths float32 {label}: worst error {err:.3e} (logits spread {float(want.std()):.3f})")
             torch.testing.assert_close(logits, want, **F32_TOL)
         else:
-            parity.assert_bf16_close(logits, want, f"largest widths/{label}")
+            parity.assert_bf16_close(logits, want, f"{name} widths/{label}")
     for rid in tokens:
         runner.finish(rid)
     runner.cache.check_invariants()
